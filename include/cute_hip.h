@@ -1,0 +1,164 @@
+/*
+ * cute_hip.h — C ABI of the gfx950 (MI355X) kernel library behind the `cute_kernels` Python API.
+ *
+ * Conventions shared by every entry point
+ *   - every pointer is a DEVICE pointer unless the comment says otherwise;
+ *   - the caller owns every buffer (inputs, outputs and workspaces); the library never allocates,
+ *     frees or keeps a reference after the call returns;
+ *   - `stream` is a hipStream_t passed as void*; the work is enqueued there and the call returns
+ *     without synchronising;
+ *   - the return value is a ck_status (0 = CK_OK).  Nothing is launched when it is non-zero;
+ *   - `dtype` is a ck_dtype; fp32 accumulation is used for every floating-point type;
+ *   - index tensors are int64 unless an `ids_are_i32`-style flag says otherwise.
+ *
+ * Each declaration cites the reference interface it replaces (paths under the reference repo).
+ */
+#ifndef CUTE_HIP_H
+#define CUTE_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum { CK_F32 = 0, CK_F16 = 1, CK_BF16 = 2 } ck_dtype;
+
+typedef enum {
+    CK_OK = 0,
+    CK_ERR_DTYPE = 1,     /* unsupported ck_dtype */
+    CK_ERR_SHAPE = 2,     /* a size / stride the kernels cannot handle */
+    CK_ERR_NULL = 3,      /* required pointer is NULL */
+    CK_ERR_WORKSPACE = 4, /* workspace smaller than the *_workspace_size query */
+    CK_ERR_LAUNCH = 5,    /* hipGetLastError() reported a launch failure */
+    CK_ERR_ALIGN = 6      /* pointer not aligned to the element size */
+} ck_status;
+
+/* Human-readable text for a ck_status (host pointer to a static string). */
+const char* ck_status_string(int status);
+/* Library version, bumped when a signature changes. */
+int ck_abi_version(void);
+
+/* ---------------------------------------------------------------------------------------------
+ * SwiGLU on two tensors: y = up * gate * sigmoid(gate)
+ * replaces cute_kernels/kernels/swiglu/cuda_implementation/ops.cpp:3-18
+ *   (swiglu_forward_cuda(gate, up, output, BLOCK_SIZE), swiglu_backward_cuda(...))
+ * and the Triton launchers swiglu/triton_implementation/kernels_forward.py:28-39,
+ * kernels_backward.py:36-56.  `block_size` is the threads per workgroup (64..1024, multiple of 64).
+ * ------------------------------------------------------------------------------------------- */
+int ck_swiglu_forward(const void* gate, const void* up, void* output, int64_t num_elements, int dtype,
+                      int block_size, void* stream);
+int ck_swiglu_backward(const void* gate, const void* up, const void* output_grad, void* gate_grad,
+                       void* up_grad, int64_t num_elements, int dtype, int block_size, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * SwiGLU on one tensor x[B, 2h]: up = x[:, :h], gate = x[:, h:], y[B, h]
+ * replaces swiglu_unchunked/triton_implementation/kernels_forward.py:41-56 and
+ * kernels_backward.py:51-71.  x_grad has x's layout (d_up in the first half, d_gate in the second).
+ * ------------------------------------------------------------------------------------------- */
+int ck_swiglu_unchunked_forward(const void* x, void* output, int64_t B, int64_t H_full, int dtype,
+                                int block_size, void* stream);
+int ck_swiglu_unchunked_backward(const void* x, const void* output_grad, void* x_grad, int64_t B,
+                                 int64_t H_full, int dtype, int block_size, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * RMSNorm over the last dimension of x[B, H]
+ * replaces rmsnorm/triton_implementation/kernels_forward.py:77-107 (rmsnorm_forward_triton) and
+ * kernels_backward.py:99-228 (rmsnorm_backward_triton, weighted and unweighted).
+ *   weight   : [H] or NULL
+ *   rstd     : fp32 [B] or NULL.  forward: written when non-NULL.  backward: read when non-NULL,
+ *              recomputed from x when NULL (the reference's `memory_efficient` mode)
+ *   backward : weight_grad ([H], dtype of x) is written when weight != NULL; it is reduced without
+ *              atomics through `workspace` (ck_rmsnorm_backward_workspace_size bytes).
+ * H must be <= 65536 (the reference's MAX_TRITON_BLOCK_SIZE limit, rmsnorm/forward.py:31-32).
+ * ------------------------------------------------------------------------------------------- */
+int ck_rmsnorm_forward(const void* x, const void* weight, void* output, float* rstd, int64_t B, int64_t H,
+                       float eps, int dtype, void* stream);
+int64_t ck_rmsnorm_backward_workspace_size(int64_t B, int64_t H);
+int ck_rmsnorm_backward(const void* x, const void* weight, const void* output_grad, const float* rstd,
+                        void* x_grad, void* weight_grad, void* workspace, int64_t workspace_bytes,
+                        int64_t B, int64_t H, float eps, int dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Embedding gather / scatter-add
+ * replaces embedding/triton_implementation/kernels_forward.py:42-64 (embedding_forward_triton) and
+ * kernels_backward.py:48-75 (embedding_backward_triton).
+ *   forward : output[i, :] = weight[ids[i], :]  (bit-exact copy; an id outside [0, V) yields a zero row)
+ *   backward: weight_grad[V, H] is written completely (rows no id selects become zero); duplicates are
+ *             accumulated in fp32 in ascending token position and rounded once.
+ * ------------------------------------------------------------------------------------------- */
+int ck_embedding_forward(const void* ids, int ids_are_i32, const void* weight, void* output,
+                         int64_t num_ids, int64_t V, int64_t H, int dtype, void* stream);
+int64_t ck_embedding_backward_workspace_size(int64_t num_ids, int64_t V, int64_t H);
+int ck_embedding_backward(const void* ids, int ids_are_i32, const void* output_grad, void* weight_grad,
+                          void* workspace, int64_t workspace_bytes, int64_t num_ids, int64_t V, int64_t H,
+                          int dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Histogram of small non-negative integers: out[c] = #{i : x[i] == c}, c < size, int32
+ * replaces contiguous_count/triton_implementation/kernels_forward.py:46-66 (contiguous_count_triton).
+ * Values outside [0, size) are ignored.
+ * ------------------------------------------------------------------------------------------- */
+int ck_contiguous_count(const void* x, int x_is_i32, int32_t* output, int64_t n, int64_t size, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Expert sort for the MoE layer: STABLE ascending sort of expert ids with their positions, plus the
+ * inclusive prefix sum of the per-expert counts.
+ * replaces scattermoe/triton_implementation/__init__.py:80-81
+ *   (selected_experts.flatten().sort(); contiguous_count_cute(...).cumsum(-1)).
+ *   expert_ids            : int64 (or int32) [M], values in [0, E)
+ *   sorted_expert_idxs    : int64 [M]
+ *   sorted_scattered_idxs : int64 [M]  (position in expert_ids of each sorted element)
+ *   expert_offsets        : int64 [E]  (expert_offsets[e] = number of ids <= e)
+ * ------------------------------------------------------------------------------------------- */
+int64_t ck_moe_sort_workspace_size(int64_t M, int64_t E);
+int ck_moe_sort(const void* expert_ids, int ids_are_i32, int64_t* sorted_expert_idxs,
+                int64_t* sorted_scattered_idxs, int64_t* expert_offsets, void* workspace,
+                int64_t workspace_bytes, int64_t M, int64_t E, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Grouped GEMM with row gather / scatter ("scatter2scatter")
+ * replaces scattermoe/triton_implementation/ops.py:16-63 (cute::scatter2scatter).
+ * For every sorted slot i in [0, num_slots):
+ *   out[out_row(i), :] = X[in_row(i), :] @ W[e(i)]         (fp32 accumulation)
+ *   e(i)       = expert owning slot i according to expert_offsets
+ *   in_row(i)  = i if x_grouped else sorted_scattered_idxs[i] / fan_out
+ *   out_row(i) = i if y_grouped else sorted_scattered_idxs[i]
+ * X is [*, K] with row stride x_stride (elements, K contiguous); W is a strided view [E, K, N] with
+ * element strides (w_stride_e, w_stride_k, w_stride_n), one of w_stride_k / w_stride_n being 1;
+ * out is [num_slots, N] with row stride out_stride.  expert_offsets is int64 [E] (inclusive ends).
+ * ------------------------------------------------------------------------------------------- */
+int ck_scatter2scatter(const void* X, int64_t x_stride, const void* W, int64_t w_stride_e,
+                       int64_t w_stride_k, int64_t w_stride_n, const int64_t* sorted_scattered_idxs,
+                       const int64_t* expert_offsets, void* out, int64_t out_stride, int64_t num_slots,
+                       int64_t K, int64_t N, int64_t E, int64_t fan_out, int x_grouped, int y_grouped,
+                       int dtype, void* stream);
+
+/* Inclusive expert offsets from already-sorted expert ids (int64 [M] -> int64 [E]); used when a caller
+ * of cute::scatter2scatter has the sorted ids but not the offsets (ops.py:16-24 takes only the ids). */
+int ck_offsets_from_sorted(const int64_t* sorted_expert_idxs, int64_t* expert_offsets, int64_t M, int64_t E,
+                           void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Per-expert weight gradient ("groupXtY"): DW[e] (K x N) = X_e^T (K x M_e) @ DY_e (M_e x N)
+ * replaces scattermoe/triton_implementation/ops.py:67-94 (cute::group_bwd_W).
+ * X [M, K] and DY [M, N] are expert-grouped rows (row strides x_stride / dy_stride, unit column stride);
+ * DW is a strided view [E, K, N] (element strides dw_stride_e/k/n, one of k/n being 1).  Every element
+ * of DW is written: experts with no rows receive zeros, so the caller need not clear DW first.
+ * ------------------------------------------------------------------------------------------- */
+int ck_group_bwd_W(const void* DY, int64_t dy_stride, const void* X, int64_t x_stride,
+                   const int64_t* expert_offsets, void* DW, int64_t dw_stride_e, int64_t dw_stride_k,
+                   int64_t dw_stride_n, int64_t M, int64_t K, int64_t N, int64_t E, int dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Row gather with optional per-row coefficient ("group")
+ * replaces scattermoe/triton_implementation/ops.py:98-130 (cute::group).
+ *   out[i, :] = A[idx[i] / fan_out, :] * (coeff ? coeff[idx[i]] : 1)     i in [0, num_rows)
+ * ------------------------------------------------------------------------------------------- */
+int ck_group(const void* A, int64_t a_stride, const int64_t* idx, const void* coeff, void* out,
+             int64_t out_stride, int64_t num_rows, int64_t K, int64_t fan_out, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CUTE_HIP_H */

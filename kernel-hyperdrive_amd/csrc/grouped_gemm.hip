@@ -1,0 +1,532 @@
+// Grouped GEMMs of the scattermoe layer for gfx950:
+//   ck_scatter2scatter : out[out_row(i)] = X[in_row(i)] @ W[e(i)]        (forward and dX)
+//       cute_kernels/kernels/scattermoe/triton_implementation/kernels.py:8-149
+//   ck_group_bwd_W     : DW[e] = X_e^T @ DY_e                            (dW)
+//       cute_kernels/kernels/scattermoe/triton_implementation/kernels.py:152-240
+//   ck_group           : out[i] = A[idx[i] / fan_out] * coeff[idx[i]]    (row gather)
+//       cute_kernels/kernels/scattermoe/triton_implementation/kernels.py:243-298
+//
+// 16-bit types run on the matrix cores: v_mfma_f32_32x32x16_{bf16,f16}, fp32 accumulators, operand tiles
+// staged through double-buffered LDS.  Tiles are scheduled per expert from expert_offsets, so a tile
+// never mixes rows of two experts (the reference lets a 128-row block straddle experts and repeats the
+// product once per expert present in it).  fp32, and shapes whose contiguous dimensions are not
+// multiples of 8 elements, go through a plain fp32-FMA kernel.
+#include "ck_device.h"
+
+namespace ck {
+
+// ---- MFMA wrappers ---------------------------------------------------------------------------
+template <typename T>
+struct Mma;
+template <>
+struct Mma<BF16> {
+    typedef bf16x8_t frag_t;
+    static __device__ __forceinline__ f32x16_t mma(frag_t a, frag_t b, f32x16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+};
+template <>
+struct Mma<F16> {
+    typedef f16x8_t frag_t;
+    static __device__ __forceinline__ f32x16_t mma(frag_t a, frag_t b, f32x16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
+
+struct GemmParams {
+    const void* A;  // S2S: X [*, K]            XTY: P [rows, I]  (C = P^T Q)
+    const void* B;  // S2S: W view              XTY: Q [rows, J]
+    void* C;        // S2S: out [slots, N]      XTY: C [E, I, J], J contiguous
+    int64_t lda, ldb, ldc;
+    int64_t b_stride_e, c_stride_e;
+    const int64_t* row_idx;  // S2S: sorted_scattered_idxs
+    const int64_t* offsets;  // inclusive expert ends, [E]
+    int M, N, K, E;          // S2S: slots, N, K.  XTY: rows, J (= N), I (= K)
+    int fan_out, x_grouped, y_grouped;
+    int m_tiles, n_tiles;    // S2S: upper bound of row tiles; XTY: tiles along I
+};
+
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+// Expert tile lookup: row tile `mt` (counted over all experts, each expert's rows cut into BM-row tiles)
+// -> expert, first row, valid rows.  Executed by the first wave; result broadcast through LDS.
+template <int BM>
+__device__ __forceinline__ void find_tile(const int64_t* __restrict__ offsets, int E, int mt, int* sh_info) {
+    if (threadIdx.x < CK_WAVE) {
+        const int lane = lane_id();
+        int base_tiles = 0;
+        int found_e = -1, found_start = 0, found_rows = 0;
+        for (int e0 = 0; e0 < E && found_e < 0; e0 += CK_WAVE) {
+            const int e = e0 + lane;
+            int begin = 0, end = 0;
+            if (e < E) {
+                end = (int)offsets[e];
+                begin = e == 0 ? 0 : (int)offsets[e - 1];
+            }
+            const int tiles = (end - begin + BM - 1) / BM;
+            const int incl = wave_inclusive_scan_i(tiles) + base_tiles;
+            const uint64_t hit = __ballot(e < E && incl > mt);
+            if (hit != 0) {
+                const int src = __ffsll((unsigned long long)hit) - 1;
+                const int excl = __shfl(incl - tiles, src, CK_WAVE);
+                const int b = __shfl(begin, src, CK_WAVE);
+                const int en = __shfl(end, src, CK_WAVE);
+                found_e = e0 + src;
+                found_start = b + (mt - excl) * BM;
+                found_rows = min(BM, en - found_start);
+            }
+            base_tiles = __shfl(incl, CK_WAVE - 1, CK_WAVE);
+        }
+        if (lane == 0) {
+            sh_info[0] = found_e;
+            sh_info[1] = found_start;
+            sh_info[2] = found_rows;
+        }
+    }
+    __syncthreads();
+}
+
+// XCD-aware tile order: consecutive workgroup ids land on different XCDs (8 of them, one L2 each), so
+// give every XCD a contiguous range of logical tile ids; inside the range, walk GROUP_M row tiles for
+// one column tile before moving to the next column tile, so concurrent tiles share operands in L2.
+__device__ __forceinline__ bool logical_tile(int m_tiles, int n_tiles, int& mt, int& nt) {
+    constexpr int XCDS = 8, GROUP_M = 8;
+    const int total = m_tiles * n_tiles;
+    const int per_xcd = (total + XCDS - 1) / XCDS;
+    const int bid = blockIdx.x;
+    const int L = (bid % XCDS) * per_xcd + bid / XCDS;
+    if (L >= total) return false;
+    const int group_span = GROUP_M * n_tiles;
+    const int group = L / group_span;
+    const int first_m = group * GROUP_M;
+    const int gm = min(GROUP_M, m_tiles - first_m);
+    const int in_group = L - group * group_span;
+    mt = first_m + in_group % gm;
+    nt = in_group / gm;
+    return true;
+}
+
+// GROUP_K = false ("S2S"): C[row map] = A[row map] (k contiguous) x B, B k-contiguous (B_KC) or n-contiguous.
+// GROUP_K = true  ("XTY"): C[e] = P_e^T Q_e, both operands contiguous along the output dimension; the
+//                          contraction runs over the expert's rows.
+template <typename T, int BM, int BN, int BK, int WM, int WN, bool B_KC, bool GROUP_K>
+__global__ void __launch_bounds__(WM* WN* CK_WAVE) grouped_gemm_kernel(GemmParams p) {
+    typedef typename T::storage_t S;
+    typedef typename Mma<T>::frag_t frag_t;
+    constexpr int THREADS = WM * WN * CK_WAVE;
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    constexpr int PAD = 8;
+    constexpr bool A_KC = !GROUP_K;
+    constexpr bool B_KCC = GROUP_K ? false : B_KC;
+    // LDS tiles: k-contiguous operands as [rows][BK + PAD], others as [BK][rows + PAD]
+    constexpr int A_ROWS = A_KC ? BM : BK, A_COLS = (A_KC ? BK : BM) + PAD;
+    constexpr int B_ROWS = B_KCC ? BN : BK, B_COLS = (B_KCC ? BK : BN) + PAD;
+    __shared__ __attribute__((aligned(16))) S As[2][A_ROWS][A_COLS];
+    __shared__ __attribute__((aligned(16))) S Bs[2][B_ROWS][B_COLS];
+    __shared__ int sh_info[4];
+
+    int mt, nt;
+    if (!logical_tile(p.m_tiles, p.n_tiles, mt, nt)) return;
+
+    const int tid = threadIdx.x;
+    const int lane = lane_id();
+    const int wave = tid / CK_WAVE;
+    const int wm = wave / WN, wn = wave % WN;
+
+    // ---- which rows / which contraction range ------------------------------------------------
+    int expert, row_start, rows_valid;  // S2S: rows of this tile.  XTY: contraction rows of the expert
+    int k_begin, k_end;                 // contraction range
+    int i_base;                         // XTY: first output row of this tile
+    if (!GROUP_K) {
+        find_tile<BM>(p.offsets, p.E, mt, sh_info);
+        expert = sh_info[0];
+        row_start = sh_info[1];
+        rows_valid = sh_info[2];
+        if (expert < 0) return;
+        k_begin = 0;
+        k_end = p.K;
+        i_base = 0;
+    } else {
+        const int i_tiles = p.m_tiles / p.E;
+        expert = mt / i_tiles;
+        i_base = (mt % i_tiles) * BM;
+        k_begin = expert == 0 ? 0 : (int)p.offsets[expert - 1];
+        k_end = (int)p.offsets[expert];
+        row_start = 0;
+        rows_valid = min(BM, p.K - i_base);
+    }
+    const int n_base = nt * BN;
+
+    // ---- global -> register staging ------------------------------------------------------------
+    constexpr int A_CHUNKS_PER_ROW = (A_KC ? BK : BM) / 8;
+    constexpr int B_CHUNKS_PER_ROW = (B_KCC ? BK : BN) / 8;
+    constexpr int A_CH = A_ROWS * A_CHUNKS_PER_ROW / THREADS;
+    constexpr int B_CH = B_ROWS * B_CHUNKS_PER_ROW / THREADS;
+    static_assert(A_ROWS * A_CHUNKS_PER_ROW % THREADS == 0 && B_ROWS * B_CHUNKS_PER_ROW % THREADS == 0, "tile/threads");
+
+    const S* a_src[A_CH];  // S2S: row base pointers (nullptr = row outside the tile)
+    if (A_KC) {
+#pragma unroll
+        for (int i = 0; i < A_CH; ++i) {
+            const int c = tid + i * THREADS;
+            const int r = c / A_CHUNKS_PER_ROW;
+            a_src[i] = nullptr;
+            if (r < rows_valid) {
+                const int64_t slot = row_start + r;
+                const int64_t src_row = p.x_grouped ? slot : p.row_idx[slot] / p.fan_out;
+                a_src[i] = reinterpret_cast<const S*>(p.A) + src_row * p.lda;
+            }
+        }
+    }
+    const S* Bbase = reinterpret_cast<const S*>(p.B) + (GROUP_K ? 0 : (int64_t)expert * p.b_stride_e);
+
+    u32x4_t a_reg[A_CH], b_reg[B_CH];
+    auto load_tiles = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < A_CH; ++i) {
+            const int c = tid + i * THREADS;
+            const int r = c / A_CHUNKS_PER_ROW;
+            const int cc = (c % A_CHUNKS_PER_ROW) * 8;
+            u32x4_t v = {0u, 0u, 0u, 0u};
+            if (A_KC) {
+                // row r of the tile, k = k0 + cc .. +7
+                if (a_src[i] != nullptr && k0 + cc < k_end)
+                    v = *reinterpret_cast<const u32x4_t*>(a_src[i] + k0 + cc);
+            } else {
+                // contraction row k0 + r, output rows i_base + cc .. +7
+                if (k0 + r < k_end && i_base + cc < p.K)
+                    v = *reinterpret_cast<const u32x4_t*>(reinterpret_cast<const S*>(p.A) + (int64_t)(k0 + r) * p.lda +
+                                                          i_base + cc);
+            }
+            a_reg[i] = v;
+        }
+#pragma unroll
+        for (int i = 0; i < B_CH; ++i) {
+            const int c = tid + i * THREADS;
+            const int r = c / B_CHUNKS_PER_ROW;
+            const int cc = (c % B_CHUNKS_PER_ROW) * 8;
+            u32x4_t v = {0u, 0u, 0u, 0u};
+            if (B_KCC) {
+                // column n_base + r, k = k0 + cc .. +7
+                if (n_base + r < p.N && k0 + cc < k_end)
+                    v = *reinterpret_cast<const u32x4_t*>(Bbase + (int64_t)(n_base + r) * p.ldb + k0 + cc);
+            } else {
+                // contraction row k0 + r, columns n_base + cc .. +7
+                if (k0 + r < k_end && n_base + cc < p.N)
+                    v = *reinterpret_cast<const u32x4_t*>(Bbase + (int64_t)(k0 + r) * p.ldb + n_base + cc);
+            }
+            b_reg[i] = v;
+        }
+    };
+    auto store_tiles = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < A_CH; ++i) {
+            const int c = tid + i * THREADS;
+            *reinterpret_cast<u32x4_t*>(&As[buf][c / A_CHUNKS_PER_ROW][(c % A_CHUNKS_PER_ROW) * 8]) = a_reg[i];
+        }
+#pragma unroll
+        for (int i = 0; i < B_CH; ++i) {
+            const int c = tid + i * THREADS;
+            *reinterpret_cast<u32x4_t*>(&Bs[buf][c / B_CHUNKS_PER_ROW][(c % B_CHUNKS_PER_ROW) * 8]) = b_reg[i];
+        }
+    };
+
+    f32x16_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    const int frag_row = lane % 32;  // row (A) / column (B) inside a 32-wide MFMA tile
+    const int frag_k = (lane / 32) * 8;
+
+    const int k_tiles = (k_end - k_begin + BK - 1) / BK;
+    if (k_tiles > 0) {
+        load_tiles(k_begin);
+        store_tiles(0);
+    }
+    __syncthreads();
+    for (int kt = 0; kt < k_tiles; ++kt) {
+        const int buf = kt & 1;
+        if (kt + 1 < k_tiles) load_tiles(k_begin + (kt + 1) * BK);
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 16) {
+            frag_t af[TM], bf[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const int r = wm * (BM / WM) + i * 32 + frag_row;
+                if (A_KC) {
+                    af[i] = *reinterpret_cast<const frag_t*>(&As[buf][r][kk + frag_k]);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) af[i][j] = As[buf][kk + frag_k + j][r];
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int c = wn * (BN / WN) + j * 32 + frag_row;
+                if (B_KCC) {
+                    bf[j] = *reinterpret_cast<const frag_t*>(&Bs[buf][c][kk + frag_k]);
+                } else {
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) bf[j][q] = Bs[buf][kk + frag_k + q][c];
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) acc[i][j] = Mma<T>::mma(af[i], bf[j], acc[i][j]);
+        }
+        if (kt + 1 < k_tiles) store_tiles(buf ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: lane holds column (lane % 32), rows 8 * (r / 4) + 4 * (lane / 32) + r % 4 --------------
+    S* Cbase = reinterpret_cast<S*>(p.C) + (GROUP_K ? (int64_t)expert * p.c_stride_e : 0);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int row = wm * (BM / WM) + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
+            if (row >= rows_valid) continue;
+            int64_t out_row;
+            if (GROUP_K) {
+                out_row = i_base + row;
+            } else {
+                const int64_t slot = row_start + row;
+                out_row = p.y_grouped ? slot : p.row_idx[slot];
+            }
+            S* crow = Cbase + out_row * p.ldc;
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int col = n_base + wn * (BN / WN) + j * 32 + frag_row;
+                if (col < p.N) crow[col] = T::down(acc[i][j][r]);
+            }
+        }
+    }
+}
+
+// ---- plain kernels (fp32 and irregular shapes) ---------------------------------------------------
+// One lane per output element; fp32 FMA in ascending k.
+template <typename T>
+__global__ void __launch_bounds__(256)
+    s2s_plain_kernel(const typename T::storage_t* __restrict__ X, int64_t ldx, const typename T::storage_t* __restrict__ W,
+                     int64_t se, int64_t sk, int64_t sn, const int64_t* __restrict__ row_idx,
+                     const int64_t* __restrict__ offsets, typename T::storage_t* __restrict__ out, int64_t ldo,
+                     int64_t slots, int K, int N, int E, int fan_out, int x_grouped, int y_grouped) {
+    const int n = blockIdx.x * 64 + threadIdx.x % 64;
+    const int64_t slot = (int64_t)blockIdx.y * 4 + threadIdx.x / 64;
+    if (slot >= slots || n >= N) return;
+    // expert of this slot: first e with offsets[e] > slot (binary search)
+    int lo = 0, hi = E - 1;
+    while (lo < hi) {
+        const int mid = (lo + hi) / 2;
+        if (offsets[mid] > slot) hi = mid;
+        else lo = mid + 1;
+    }
+    const int64_t src_row = x_grouped ? slot : row_idx[slot] / fan_out;
+    const int64_t dst_row = y_grouped ? slot : row_idx[slot];
+    const typename T::storage_t* x = X + src_row * ldx;
+    const typename T::storage_t* w = W + (int64_t)lo * se + (int64_t)n * sn;
+    float acc = 0.f;
+    for (int k = 0; k < K; ++k) acc = fmaf(T::up(x[k]), T::up(w[(int64_t)k * sk]), acc);
+    out[dst_row * ldo + n] = T::down(acc);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+    xty_plain_kernel(const typename T::storage_t* __restrict__ DY, int64_t lddy, const typename T::storage_t* __restrict__ X,
+                     int64_t ldx, const int64_t* __restrict__ offsets, typename T::storage_t* __restrict__ DW, int64_t se,
+                     int64_t sk, int64_t sn, int K, int N, int E) {
+    // lanes run along the contiguous dimension of DW
+    const bool k_fast = sk == 1;
+    const int fast = blockIdx.x * 64 + threadIdx.x % 64;
+    const int slow = blockIdx.y * 4 + threadIdx.x / 64;
+    const int e = blockIdx.z;
+    const int k = k_fast ? fast : slow;
+    const int n = k_fast ? slow : fast;
+    if (k >= K || n >= N) return;
+    const int64_t begin = e == 0 ? 0 : offsets[e - 1];
+    const int64_t end = offsets[e];
+    float acc = 0.f;
+    for (int64_t m = begin; m < end; ++m) acc = fmaf(T::up(X[m * ldx + k]), T::up(DY[m * lddy + n]), acc);
+    DW[(int64_t)e * se + (int64_t)k * sk + (int64_t)n * sn] = T::down(acc);
+}
+
+// ---- row gather ------------------------------------------------------------------------------
+// One wave per output row, 4 rows per workgroup.
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256)
+    group_kernel(const typename T::storage_t* __restrict__ A, int64_t lda, const int64_t* __restrict__ idx,
+                 const typename T::storage_t* __restrict__ coeff, typename T::storage_t* __restrict__ out, int64_t ldo,
+                 int64_t rows, int64_t K, int64_t fan_out) {
+    typedef VPack<T, VEC> P;
+    const int64_t row = (int64_t)blockIdx.x * 4 + threadIdx.x / CK_WAVE;
+    if (row >= rows) return;
+    const int64_t id = idx[row];
+    const float c = coeff != nullptr ? T::up(coeff[id]) : 1.0f;
+    const P* src = reinterpret_cast<const P*>(A + (id / fan_out) * lda);
+    P* dst = reinterpret_cast<P*>(out + row * ldo);
+    const int64_t packs = K / VEC;
+    for (int64_t p = lane_id(); p < packs; p += CK_WAVE) {
+        P v = src[p];
+        if (coeff != nullptr) {
+            // the reference multiplies in the storage type (kernels.py:284-286): one rounding of the product
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v.v[j] = T::down(T::up(v.v[j]) * c);
+        }
+        nt_store(v, dst + p);
+    }
+}
+
+}  // namespace ck
+
+// ---- host side ------------------------------------------------------------------------------
+namespace {
+
+constexpr int kBM = 128, kBN = 128, kBK = 64, kWM = 2, kWN = 2;
+
+template <typename T, bool B_KC, bool GROUP_K>
+void launch_mfma(const ck::GemmParams& p, hipStream_t s) {
+    const int total = p.m_tiles * p.n_tiles;
+    const int grid = (total + 7) / 8 * 8;
+    hipLaunchKernelGGL((ck::grouped_gemm_kernel<T, kBM, kBN, kBK, kWM, kWN, B_KC, GROUP_K>), dim3((unsigned)grid),
+                       dim3(kWM * kWN * CK_WAVE), 0, s, p);
+}
+
+bool mult8(int64_t v) { return (v & 7) == 0; }
+
+}  // namespace
+
+extern "C" int ck_scatter2scatter(const void* X, int64_t x_stride, const void* W, int64_t w_stride_e,
+                                  int64_t w_stride_k, int64_t w_stride_n, const int64_t* sorted_scattered_idxs,
+                                  const int64_t* expert_offsets, void* out, int64_t out_stride, int64_t num_slots,
+                                  int64_t K, int64_t N, int64_t E, int64_t fan_out, int x_grouped, int y_grouped,
+                                  int dtype, void* stream) {
+    if (num_slots < 0 || K < 0 || N < 0 || E <= 0 || fan_out <= 0) return CK_ERR_SHAPE;
+    if (num_slots > 0x7fffffff || K > 0x7fffffff || N > 0x7fffffff || E > 0x7fffffff) return CK_ERR_SHAPE;
+    if (dtype != CK_F32 && dtype != CK_F16 && dtype != CK_BF16) return CK_ERR_DTYPE;
+    if (num_slots == 0 || N == 0) return CK_OK;
+    if (!out || !expert_offsets || (K > 0 && (!X || !W))) return CK_ERR_NULL;
+    if ((!x_grouped || !y_grouped) && !sorted_scattered_idxs) return CK_ERR_NULL;
+    if (!ck_aligned_elem(X, dtype) || !ck_aligned_elem(W, dtype) || !ck_aligned_elem(out, dtype)) return CK_ERR_ALIGN;
+    hipStream_t s = (hipStream_t)stream;
+
+    const bool b_kc = w_stride_k == 1, b_nc = w_stride_n == 1;
+    const bool fast = dtype != CK_F32 && K > 0 && (b_kc || b_nc) && ck_aligned16(X) && ck_aligned16(W) && mult8(K) &&
+                      mult8(x_stride) && mult8(w_stride_e) && mult8(b_kc ? w_stride_n : w_stride_k) &&
+                      (b_kc || mult8(N));
+    if (fast) {
+        ck::GemmParams p = {};
+        p.A = X;
+        p.B = W;
+        p.C = out;
+        p.lda = x_stride;
+        p.ldb = b_kc ? w_stride_n : w_stride_k;
+        p.ldc = out_stride;
+        p.b_stride_e = w_stride_e;
+        p.row_idx = sorted_scattered_idxs;
+        p.offsets = expert_offsets;
+        p.M = (int)num_slots;
+        p.N = (int)N;
+        p.K = (int)K;
+        p.E = (int)E;
+        p.fan_out = (int)fan_out;
+        p.x_grouped = x_grouped;
+        p.y_grouped = y_grouped;
+        p.m_tiles = (int)(num_slots / kBM + E);
+        p.n_tiles = (int)ck_ceil_div(N, kBN);
+        if ((int64_t)p.m_tiles * p.n_tiles > 0x7ffffff0) return CK_ERR_SHAPE;
+        if (dtype == CK_BF16) {
+            if (b_kc) launch_mfma<ck::BF16, true, false>(p, s);
+            else launch_mfma<ck::BF16, false, false>(p, s);
+        } else {
+            if (b_kc) launch_mfma<ck::F16, true, false>(p, s);
+            else launch_mfma<ck::F16, false, false>(p, s);
+        }
+        return ck_launch_status();
+    }
+    const dim3 grid((unsigned)ck_ceil_div(N, 64), (unsigned)ck_ceil_div(num_slots, 4));
+    if (grid.y > 65535u * 1024u) return CK_ERR_SHAPE;
+    CK_DISPATCH_DTYPE(dtype, {
+        typedef typename T::storage_t S;
+        hipLaunchKernelGGL((ck::s2s_plain_kernel<T>), grid, dim3(256), 0, s, (const S*)X, x_stride, (const S*)W,
+                           w_stride_e, w_stride_k, w_stride_n, sorted_scattered_idxs, expert_offsets, (S*)out,
+                           out_stride, num_slots, (int)K, (int)N, (int)E, (int)fan_out, x_grouped, y_grouped);
+    });
+    return ck_launch_status();
+}
+
+extern "C" int ck_group_bwd_W(const void* DY, int64_t dy_stride, const void* X, int64_t x_stride,
+                              const int64_t* expert_offsets, void* DW, int64_t dw_stride_e, int64_t dw_stride_k,
+                              int64_t dw_stride_n, int64_t M, int64_t K, int64_t N, int64_t E, int dtype, void* stream) {
+    if (M < 0 || K < 0 || N < 0 || E <= 0) return CK_ERR_SHAPE;
+    if (M > 0x7fffffff || K > 0x7fffffff || N > 0x7fffffff || E > 65535) return CK_ERR_SHAPE;
+    if (dtype != CK_F32 && dtype != CK_F16 && dtype != CK_BF16) return CK_ERR_DTYPE;
+    if (K == 0 || N == 0) return CK_OK;
+    if (!DW || !expert_offsets || (M > 0 && (!DY || !X))) return CK_ERR_NULL;
+    if (!ck_aligned_elem(DW, dtype) || !ck_aligned_elem(X, dtype) || !ck_aligned_elem(DY, dtype)) return CK_ERR_ALIGN;
+    hipStream_t s = (hipStream_t)stream;
+
+    const bool k_fast = dw_stride_k == 1, n_fast = dw_stride_n == 1;
+    const bool fast = dtype != CK_F32 && (k_fast || n_fast) && ck_aligned16(X) && ck_aligned16(DY) && mult8(K) &&
+                      mult8(N) && mult8(x_stride) && mult8(dy_stride);
+    if (fast) {
+        // C[e][i][j] = sum_r P[r][i] * Q[r][j] with j the contiguous dimension of DW
+        ck::GemmParams p = {};
+        const bool swap = k_fast;  // j = k: P = DY (i = n), Q = X
+        p.A = swap ? DY : X;
+        p.lda = swap ? dy_stride : x_stride;
+        p.B = swap ? X : DY;
+        p.ldb = swap ? x_stride : dy_stride;
+        p.C = DW;
+        p.ldc = swap ? dw_stride_n : dw_stride_k;
+        p.c_stride_e = dw_stride_e;
+        p.offsets = expert_offsets;
+        p.M = (int)M;
+        p.K = (int)(swap ? N : K);  // I
+        p.N = (int)(swap ? K : N);  // J
+        p.E = (int)E;
+        p.m_tiles = (int)(E * ck_ceil_div(p.K, kBM));
+        p.n_tiles = (int)ck_ceil_div(p.N, kBN);
+        if ((int64_t)p.m_tiles * p.n_tiles > 0x7ffffff0) return CK_ERR_SHAPE;
+        if (dtype == CK_BF16) launch_mfma<ck::BF16, false, true>(p, s);
+        else launch_mfma<ck::F16, false, true>(p, s);
+        return ck_launch_status();
+    }
+    const int64_t fast_dim = k_fast ? K : N, slow_dim = k_fast ? N : K;
+    const dim3 grid((unsigned)ck_ceil_div(fast_dim, 64), (unsigned)ck_ceil_div(slow_dim, 4), (unsigned)E);
+    CK_DISPATCH_DTYPE(dtype, {
+        typedef typename T::storage_t S;
+        hipLaunchKernelGGL((ck::xty_plain_kernel<T>), grid, dim3(256), 0, s, (const S*)DY, dy_stride, (const S*)X,
+                           x_stride, expert_offsets, (S*)DW, dw_stride_e, dw_stride_k, dw_stride_n, (int)K, (int)N,
+                           (int)E);
+    });
+    return ck_launch_status();
+}
+
+extern "C" int ck_group(const void* A, int64_t a_stride, const int64_t* idx, const void* coeff, void* out,
+                        int64_t out_stride, int64_t num_rows, int64_t K, int64_t fan_out, int dtype, void* stream) {
+    if (num_rows < 0 || K < 0 || fan_out <= 0) return CK_ERR_SHAPE;
+    if (num_rows == 0 || K == 0) return CK_OK;
+    if (!A || !idx || !out) return CK_ERR_NULL;
+    if (!ck_aligned_elem(A, dtype) || !ck_aligned_elem(out, dtype) || (coeff && !ck_aligned_elem(coeff, dtype)))
+        return CK_ERR_ALIGN;
+    const int64_t grid = ck_ceil_div(num_rows, 4);
+    if (grid > 0x7fffffff) return CK_ERR_SHAPE;
+    hipStream_t s = (hipStream_t)stream;
+    CK_DISPATCH_DTYPE(dtype, {
+        typedef typename T::storage_t S;
+        const bool vec = ck_aligned16(A) && ck_aligned16(out) && K % T::kVec == 0 && a_stride % T::kVec == 0 &&
+                         out_stride % T::kVec == 0;
+        if (vec)
+            hipLaunchKernelGGL((ck::group_kernel<T, T::kVec>), dim3((unsigned)grid), dim3(256), 0, s, (const S*)A,
+                               a_stride, idx, (const S*)coeff, (S*)out, out_stride, num_rows, K, fan_out);
+        else
+            hipLaunchKernelGGL((ck::group_kernel<T, 1>), dim3((unsigned)grid), dim3(256), 0, s, (const S*)A, a_stride,
+                               idx, (const S*)coeff, (S*)out, out_stride, num_rows, K, fan_out);
+    });
+    return ck_launch_status();
+}

@@ -1,0 +1,481 @@
+// RMSNorm forward / backward for gfx950 (math: cute_kernels/kernels/rmsnorm/README.md:3-25).
+//
+// Fast path (row length a multiple of the 16-byte packet, 16-byte aligned pointers):
+//   a "team" of TPR lanes (64, 256 or 1024) owns one row at a time and keeps it in registers, so x (and
+//   dy) are read from HBM exactly once.  Row sums use wave64 shuffles; teams wider than a wave finish
+//   through a few LDS floats.  Backward is persistent: each team walks rows team, team+teams, ... and
+//   accumulates its share of dweight in fp32 registers, writes one fp32 partial row to the workspace,
+//   and a second kernel sums the partial rows column-wise with shuffles.  No atomics anywhere, so
+//   dweight is deterministic for a given team count.
+// Generic path (any H, any element alignment): one 256-lane team per row re-reading the row from cache,
+//   and a column kernel for the dweight partials.
+#include "ck_device.h"
+
+namespace ck {
+
+constexpr int kMaxPacks = 8;        // packets a lane keeps per row on the fast path
+constexpr int kColSegments = 64;    // row segments of the generic dweight column kernel
+
+// sum over the TPR lanes that share a row; `red` is LDS scratch of (blockDim/64) floats per use
+template <int TPR>
+__device__ __forceinline__ float team_sum(float v, float* red) {
+    v = wave_sum(v);
+    if (TPR > CK_WAVE) {
+        const int wave = threadIdx.x / CK_WAVE;
+        __syncthreads();  // protect `red` from the previous use
+        if (lane_id() == 0) red[wave] = v;
+        __syncthreads();
+        float t = 0.f;
+#pragma unroll
+        for (int w = 0; w < TPR / CK_WAVE; ++w) t += red[w];
+        v = t;
+    }
+    return v;
+}
+
+template <typename T, int TPR>
+__global__ void __launch_bounds__(TPR > 256 ? TPR : 256)
+    rmsnorm_fwd_kernel(const typename T::storage_t* __restrict__ x, const typename T::storage_t* __restrict__ w,
+                       typename T::storage_t* __restrict__ y, float* __restrict__ rstd_out, int64_t B, int H,
+                       float eps) {
+    typedef VPack<T, T::kVec> P;
+    __shared__ float red[16];
+    const int teams_per_block = blockDim.x / TPR;
+    const int team = threadIdx.x / TPR;
+    const int t = threadIdx.x % TPR;
+    const int64_t row = (int64_t)blockIdx.x * teams_per_block + team;
+    const int packs = H / T::kVec;
+    // with TPR > 64 the whole block is one team, so `row < B` is uniform across the barriers below
+    if (row >= B) return;
+
+    const P* xr = reinterpret_cast<const P*>(x + row * H);
+    P xv[kMaxPacks];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < kMaxPacks; ++i) {
+        const int p = t + i * TPR;
+        if (p < packs) {
+            xv[i] = nt_load(xr + p);
+#pragma unroll
+            for (int j = 0; j < T::kVec; ++j) {
+                const float f = T::up(xv[i].v[j]);
+                ss += f * f;
+            }
+        }
+    }
+    ss = team_sum<TPR>(ss, red);
+    const float rstd = rsqrtf(ss / (float)H + eps);
+    if (rstd_out != nullptr && t == 0) rstd_out[row] = rstd;
+
+    P* yr = reinterpret_cast<P*>(y + row * H);
+#pragma unroll
+    for (int i = 0; i < kMaxPacks; ++i) {
+        const int p = t + i * TPR;
+        if (p < packs) {
+            P o;
+            if (w != nullptr) {
+                const P wv = reinterpret_cast<const P*>(w)[p];
+#pragma unroll
+                for (int j = 0; j < T::kVec; ++j) o.v[j] = T::down(T::up(xv[i].v[j]) * rstd * T::up(wv.v[j]));
+            } else {
+#pragma unroll
+                for (int j = 0; j < T::kVec; ++j) o.v[j] = T::down(T::up(xv[i].v[j]) * rstd);
+            }
+            nt_store(o, yr + p);
+        }
+    }
+}
+
+template <typename T, int TPR, bool HAS_W>
+__global__ void __launch_bounds__(TPR > 256 ? TPR : 256)
+    rmsnorm_bwd_kernel(const typename T::storage_t* __restrict__ x, const typename T::storage_t* __restrict__ w,
+                       const typename T::storage_t* __restrict__ dy, const float* __restrict__ rstd_in,
+                       typename T::storage_t* __restrict__ dx, float* __restrict__ dw_partial, int64_t B, int H,
+                       float eps) {
+    typedef VPack<T, T::kVec> P;
+    __shared__ float red[16];
+    const int teams_per_block = blockDim.x / TPR;
+    const int team = blockIdx.x * teams_per_block + threadIdx.x / TPR;
+    const int num_teams = gridDim.x * teams_per_block;
+    const int t = threadIdx.x % TPR;
+    const int packs = H / T::kVec;
+    const float inv_h = 1.0f / (float)H;
+
+    P wv[kMaxPacks];
+    float dw[kMaxPacks][T::kVec];
+    if (HAS_W) {
+#pragma unroll
+        for (int i = 0; i < kMaxPacks; ++i) {
+            const int p = t + i * TPR;
+            if (p < packs) wv[i] = reinterpret_cast<const P*>(w)[p];
+#pragma unroll
+            for (int j = 0; j < T::kVec; ++j) dw[i][j] = 0.f;
+        }
+    }
+
+    // rows are dealt round-robin; with TPR > 64 the block is one team so the trip count is block-uniform
+    for (int64_t row = team; row < B; row += num_teams) {
+        const P* xr = reinterpret_cast<const P*>(x + row * H);
+        const P* gr = reinterpret_cast<const P*>(dy + row * H);
+        P xv[kMaxPacks], gv[kMaxPacks];
+#pragma unroll
+        for (int i = 0; i < kMaxPacks; ++i) {
+            const int p = t + i * TPR;
+            if (p < packs) {
+                xv[i] = nt_load(xr + p);
+                gv[i] = nt_load(gr + p);
+            }
+        }
+        float ss = 0.f, dot = 0.f;
+#pragma unroll
+        for (int i = 0; i < kMaxPacks; ++i) {
+            const int p = t + i * TPR;
+            if (p < packs) {
+#pragma unroll
+                for (int j = 0; j < T::kVec; ++j) {
+                    const float xf = T::up(xv[i].v[j]);
+                    float g = T::up(gv[i].v[j]);
+                    if (HAS_W) g *= T::up(wv[i].v[j]);
+                    ss += xf * xf;
+                    dot += g * xf;
+                }
+            }
+        }
+        float rstd;
+        if (rstd_in != nullptr) {
+            rstd = rstd_in[row];
+        } else {
+            ss = team_sum<TPR>(ss, red);
+            rstd = rsqrtf(ss * inv_h + eps);
+        }
+        dot = team_sum<TPR>(dot, red);
+        const float c = rstd * rstd * rstd * inv_h * dot;
+
+        P* dr = reinterpret_cast<P*>(dx + row * H);
+#pragma unroll
+        for (int i = 0; i < kMaxPacks; ++i) {
+            const int p = t + i * TPR;
+            if (p < packs) {
+                P o;
+#pragma unroll
+                for (int j = 0; j < T::kVec; ++j) {
+                    const float xf = T::up(xv[i].v[j]);
+                    const float d = T::up(gv[i].v[j]);
+                    float g = d;
+                    if (HAS_W) {
+                        g *= T::up(wv[i].v[j]);
+                        dw[i][j] += d * (xf * rstd);
+                    }
+                    o.v[j] = T::down(rstd * g - c * xf);
+                }
+                nt_store(o, dr + p);
+            }
+        }
+    }
+
+    if (HAS_W) {
+        float* out = dw_partial + (int64_t)team * H;
+#pragma unroll
+        for (int i = 0; i < kMaxPacks; ++i) {
+            const int p = t + i * TPR;
+            if (p < packs) {
+#pragma unroll
+                for (int j = 0; j < T::kVec; j += 4) {
+                    float4 v = make_float4(dw[i][j], dw[i][j + 1], dw[i][j + 2], dw[i][j + 3]);
+                    *reinterpret_cast<float4*>(out + p * T::kVec + j) = v;
+                }
+            }
+        }
+    }
+}
+
+// dweight[j] = sum over `parts` partial rows of partial[r][j].  One wave per block owns 16 columns:
+// lane = 16 row-groups x 4 column-quads; each lane strides over the partial rows with float4 loads,
+// then the 16 row-groups are folded with shuffles.  Requires H % 4 == 0.
+template <typename T>
+__global__ void __launch_bounds__(64)
+    rmsnorm_dw_reduce_kernel(const float* __restrict__ partial, typename T::storage_t* __restrict__ dw, int parts,
+                             int H) {
+    const int lane = threadIdx.x;
+    const int quad = lane & 3;
+    const int group = lane >> 2;
+    const int col = blockIdx.x * 16 + quad * 4;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (col < H) {
+        for (int r = group; r < parts; r += 16) {
+            const float4 v = *reinterpret_cast<const float4*>(partial + (int64_t)r * H + col);
+            acc.x += v.x;
+            acc.y += v.y;
+            acc.z += v.z;
+            acc.w += v.w;
+        }
+    }
+#pragma unroll
+    for (int off = 4; off < CK_WAVE; off <<= 1) {
+        acc.x += __shfl_xor(acc.x, off, CK_WAVE);
+        acc.y += __shfl_xor(acc.y, off, CK_WAVE);
+        acc.z += __shfl_xor(acc.z, off, CK_WAVE);
+        acc.w += __shfl_xor(acc.w, off, CK_WAVE);
+    }
+    if (group == 0 && col < H) {
+        dw[col + 0] = T::down(acc.x);
+        dw[col + 1] = T::down(acc.y);
+        dw[col + 2] = T::down(acc.z);
+        dw[col + 3] = T::down(acc.w);
+    }
+}
+
+// ---- generic path ---------------------------------------------------------------------------
+__device__ __forceinline__ float block_sum_256(float v, float* red) {
+    v = wave_sum(v);
+    __syncthreads();
+    if (lane_id() == 0) red[threadIdx.x / CK_WAVE] = v;
+    __syncthreads();
+    return red[0] + red[1] + red[2] + red[3];
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+    rmsnorm_fwd_generic_kernel(const typename T::storage_t* __restrict__ x, const typename T::storage_t* __restrict__ w,
+                               typename T::storage_t* __restrict__ y, float* __restrict__ rstd_out, int64_t B, int H,
+                               float eps) {
+    __shared__ float red[4];
+    for (int64_t row = blockIdx.x; row < B; row += gridDim.x) {
+        const typename T::storage_t* xr = x + row * H;
+        float ss = 0.f;
+        for (int j = threadIdx.x; j < H; j += 256) {
+            const float f = T::up(xr[j]);
+            ss += f * f;
+        }
+        ss = block_sum_256(ss, red);
+        const float rstd = rsqrtf(ss / (float)H + eps);
+        if (rstd_out != nullptr && threadIdx.x == 0) rstd_out[row] = rstd;
+        for (int j = threadIdx.x; j < H; j += 256) {
+            float v = T::up(xr[j]) * rstd;
+            if (w != nullptr) v *= T::up(w[j]);
+            y[row * H + j] = T::down(v);
+        }
+    }
+}
+
+// dx for one row per block; also leaves rstd of every row in `rstd_ws` for the column kernel
+template <typename T>
+__global__ void __launch_bounds__(256)
+    rmsnorm_bwd_generic_kernel(const typename T::storage_t* __restrict__ x, const typename T::storage_t* __restrict__ w,
+                               const typename T::storage_t* __restrict__ dy, const float* __restrict__ rstd_in,
+                               typename T::storage_t* __restrict__ dx, float* __restrict__ rstd_ws, int64_t B, int H,
+                               float eps) {
+    __shared__ float red[4];
+    const float inv_h = 1.0f / (float)H;
+    for (int64_t row = blockIdx.x; row < B; row += gridDim.x) {
+        const typename T::storage_t* xr = x + row * H;
+        const typename T::storage_t* gr = dy + row * H;
+        float ss = 0.f, dot = 0.f;
+        for (int j = threadIdx.x; j < H; j += 256) {
+            const float xf = T::up(xr[j]);
+            float g = T::up(gr[j]);
+            if (w != nullptr) g *= T::up(w[j]);
+            ss += xf * xf;
+            dot += g * xf;
+        }
+        float rstd;
+        if (rstd_in != nullptr) {
+            rstd = rstd_in[row];
+        } else {
+            ss = block_sum_256(ss, red);
+            rstd = rsqrtf(ss * inv_h + eps);
+        }
+        dot = block_sum_256(dot, red);
+        if (rstd_ws != nullptr && threadIdx.x == 0) rstd_ws[row] = rstd;
+        const float c = rstd * rstd * rstd * inv_h * dot;
+        for (int j = threadIdx.x; j < H; j += 256) {
+            const float xf = T::up(xr[j]);
+            float g = T::up(gr[j]);
+            if (w != nullptr) g *= T::up(w[j]);
+            dx[row * H + j] = T::down(rstd * g - c * xf);
+        }
+    }
+}
+
+// partial[seg][j] = sum over the rows of segment `seg` of dy[b][j] * x[b][j] * rstd[b]; lane per column
+template <typename T>
+__global__ void __launch_bounds__(256)
+    rmsnorm_dw_columns_kernel(const typename T::storage_t* __restrict__ x, const typename T::storage_t* __restrict__ dy,
+                              const float* __restrict__ rstd, float* __restrict__ partial, int64_t B, int H,
+                              int H_padded) {
+    const int j = blockIdx.x * 256 + threadIdx.x;
+    const int seg = blockIdx.y;
+    const int64_t rows_per_seg = (B + kColSegments - 1) / kColSegments;
+    const int64_t b0 = seg * rows_per_seg;
+    const int64_t b1 = (b0 + rows_per_seg < B) ? b0 + rows_per_seg : B;
+    if (j >= H_padded) return;
+    float acc = 0.f;
+    if (j < H)
+        for (int64_t b = b0; b < b1; ++b) acc += T::up(dy[b * H + j]) * (T::up(x[b * H + j]) * rstd[b]);
+    partial[(int64_t)seg * H_padded + j] = acc;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+    rmsnorm_dw_reduce_generic_kernel(const float* __restrict__ partial, typename T::storage_t* __restrict__ dw,
+                                     int parts, int H, int H_padded) {
+    const int j = blockIdx.x * 256 + threadIdx.x;
+    if (j >= H) return;
+    float acc = 0.f;
+    for (int r = 0; r < parts; ++r) acc += partial[(int64_t)r * H_padded + j];
+    dw[j] = T::down(acc);
+}
+
+}  // namespace ck
+
+// ---- host side ------------------------------------------------------------------------------
+static int cu_count() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
+// threads per row on the fast path, 0 when the row does not fit the register budget
+static int fast_tpr(int64_t H, int dtype) {
+    const int vec = dtype == CK_F32 ? 4 : 8;
+    if (H % vec != 0) return 0;
+    const int64_t packs = H / vec;
+    if (packs <= 64 * ck::kMaxPacks) return 64;
+    if (packs <= 256 * ck::kMaxPacks) return 256;
+    if (packs <= 1024 * ck::kMaxPacks) return 1024;
+    return 0;
+}
+
+// teams of the persistent backward kernel (also the number of fp32 partial rows)
+static int bwd_teams(int64_t B, int tpr) {
+    const int block = tpr > 256 ? tpr : 256;
+    const int teams_per_block = block / tpr;
+    int64_t blocks = (int64_t)cu_count() * (tpr == 1024 ? 1 : 2);
+    const int64_t need = ck_ceil_div(B, teams_per_block);
+    if (blocks > need) blocks = need;
+    if (blocks < 1) blocks = 1;
+    return (int)(blocks * teams_per_block);
+}
+
+extern "C" int ck_rmsnorm_forward(const void* x, const void* weight, void* output, float* rstd, int64_t B, int64_t H,
+                                  float eps, int dtype, void* stream) {
+    if (B < 0 || H < 0 || H > 65536) return CK_ERR_SHAPE;
+    if (B == 0 || H == 0) return CK_OK;
+    if (!x || !output) return CK_ERR_NULL;
+    if (!ck_aligned_elem(x, dtype) || !ck_aligned_elem(output, dtype) || (weight && !ck_aligned_elem(weight, dtype)))
+        return CK_ERR_ALIGN;
+    hipStream_t s = (hipStream_t)stream;
+    const bool aligned = ck_aligned16(x) && ck_aligned16(output) && (!weight || ck_aligned16(weight));
+    const int tpr = aligned ? fast_tpr(H, dtype) : 0;
+    CK_DISPATCH_DTYPE(dtype, {
+        typedef typename T::storage_t S;
+        if (tpr == 64) {
+            hipLaunchKernelGGL((ck::rmsnorm_fwd_kernel<T, 64>), dim3((unsigned)ck_ceil_div(B, 4)), dim3(256), 0, s,
+                               (const S*)x, (const S*)weight, (S*)output, rstd, B, (int)H, eps);
+        } else if (tpr == 256) {
+            hipLaunchKernelGGL((ck::rmsnorm_fwd_kernel<T, 256>), dim3((unsigned)B), dim3(256), 0, s, (const S*)x,
+                               (const S*)weight, (S*)output, rstd, B, (int)H, eps);
+        } else if (tpr == 1024) {
+            hipLaunchKernelGGL((ck::rmsnorm_fwd_kernel<T, 1024>), dim3((unsigned)B), dim3(1024), 0, s, (const S*)x,
+                               (const S*)weight, (S*)output, rstd, B, (int)H, eps);
+        } else {
+            const int64_t grid = B < 65536 ? B : 65536;
+            hipLaunchKernelGGL((ck::rmsnorm_fwd_generic_kernel<T>), dim3((unsigned)grid), dim3(256), 0, s, (const S*)x,
+                               (const S*)weight, (S*)output, rstd, B, (int)H, eps);
+        }
+    });
+    return ck_launch_status();
+}
+
+// Workspace layout.  Fast path: teams x H fp32 partial rows.  Generic path: B fp32 rstd values, then
+// kColSegments x H_padded fp32 partial rows.  The query returns the larger of the two.
+static int64_t padded_h(int64_t H) { return (H + 3) / 4 * 4; }
+
+extern "C" int64_t ck_rmsnorm_backward_workspace_size(int64_t B, int64_t H) {
+    if (B <= 0 || H <= 0) return 0;
+    int64_t teams = 1;
+    for (int tpr : {64, 256, 1024}) {
+        const int64_t t = bwd_teams(B, tpr);
+        if (t > teams) teams = t;
+    }
+    const int64_t fast = teams * H * 4;
+    const int64_t generic = (B + 3) / 4 * 16 + (int64_t)ck::kColSegments * padded_h(H) * 4;
+    return fast > generic ? fast : generic;
+}
+
+template <typename T, int TPR>
+static void launch_bwd(unsigned grid, int block, hipStream_t s, const void* x, const void* weight, const void* dy,
+                       const float* rstd, void* dx, float* ws, int64_t B, int H, float eps) {
+    typedef typename T::storage_t S;
+    if (weight)
+        hipLaunchKernelGGL((ck::rmsnorm_bwd_kernel<T, TPR, true>), dim3(grid), dim3(block), 0, s, (const S*)x,
+                           (const S*)weight, (const S*)dy, rstd, (S*)dx, ws, B, H, eps);
+    else
+        hipLaunchKernelGGL((ck::rmsnorm_bwd_kernel<T, TPR, false>), dim3(grid), dim3(block), 0, s, (const S*)x,
+                           (const S*)weight, (const S*)dy, rstd, (S*)dx, ws, B, H, eps);
+}
+
+extern "C" int ck_rmsnorm_backward(const void* x, const void* weight, const void* output_grad, const float* rstd,
+                                   void* x_grad, void* weight_grad, void* workspace, int64_t workspace_bytes, int64_t B,
+                                   int64_t H, float eps, int dtype, void* stream) {
+    if (B < 0 || H < 0 || H > 65536) return CK_ERR_SHAPE;
+    if (dtype != CK_F32 && dtype != CK_F16 && dtype != CK_BF16) return CK_ERR_DTYPE;
+    hipStream_t s = (hipStream_t)stream;
+    if (B == 0 || H == 0) {
+        // an empty batch still defines dweight = 0
+        if (weight && weight_grad && H > 0)
+            if (hipMemsetAsync(weight_grad, 0, (size_t)H * ck_elem_size(dtype), s) != hipSuccess) return CK_ERR_LAUNCH;
+        return CK_OK;
+    }
+    if (!x || !output_grad || !x_grad) return CK_ERR_NULL;
+    if (weight && !weight_grad) return CK_ERR_NULL;
+    const void* ptrs[5] = {x, output_grad, x_grad, weight, weight_grad};
+    bool aligned = true;
+    for (const void* p : ptrs) {
+        if (!p) continue;
+        if (!ck_aligned_elem(p, dtype)) return CK_ERR_ALIGN;
+        aligned = aligned && ck_aligned16(p);
+    }
+    if (weight) {
+        if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 15u)) return CK_ERR_WORKSPACE;
+        if (workspace_bytes < ck_rmsnorm_backward_workspace_size(B, H)) return CK_ERR_WORKSPACE;
+    }
+    const int tpr = aligned ? fast_tpr(H, dtype) : 0;
+    float* ws = (float*)workspace;
+
+    CK_DISPATCH_DTYPE(dtype, {
+        typedef typename T::storage_t S;
+        if (tpr != 0) {
+            const int teams = bwd_teams(B, tpr);
+            const int block = tpr > 256 ? tpr : 256;
+            const unsigned grid = (unsigned)(teams / (block / tpr));
+            if (tpr == 64) launch_bwd<T, 64>(grid, block, s, x, weight, output_grad, rstd, x_grad, ws, B, (int)H, eps);
+            else if (tpr == 256) launch_bwd<T, 256>(grid, block, s, x, weight, output_grad, rstd, x_grad, ws, B, (int)H, eps);
+            else launch_bwd<T, 1024>(grid, block, s, x, weight, output_grad, rstd, x_grad, ws, B, (int)H, eps);
+            if (weight)
+                hipLaunchKernelGGL((ck::rmsnorm_dw_reduce_kernel<T>), dim3((unsigned)ck_ceil_div(H, 16)), dim3(64), 0, s,
+                                   ws, (S*)weight_grad, teams, (int)H);
+        } else {
+            const int64_t grid = B < 65536 ? B : 65536;
+            float* rstd_ws = weight ? ws : nullptr;
+            hipLaunchKernelGGL((ck::rmsnorm_bwd_generic_kernel<T>), dim3((unsigned)grid), dim3(256), 0, s, (const S*)x,
+                               (const S*)weight, (const S*)output_grad, rstd, (S*)x_grad, rstd_ws, B, (int)H, eps);
+            if (weight) {
+                const int hp = (int)padded_h(H);
+                float* partial = ws + (B + 3) / 4 * 4;
+                hipLaunchKernelGGL((ck::rmsnorm_dw_columns_kernel<T>),
+                                   dim3((unsigned)ck_ceil_div(hp, 256), ck::kColSegments), dim3(256), 0, s, (const S*)x,
+                                   (const S*)output_grad, rstd_ws, partial, B, (int)H, hp);
+                hipLaunchKernelGGL((ck::rmsnorm_dw_reduce_generic_kernel<T>), dim3((unsigned)ck_ceil_div(H, 256)),
+                                   dim3(256), 0, s, partial, (S*)weight_grad, ck::kColSegments, (int)H, hp);
+            }
+        }
+    });
+    return ck_launch_status();
+}

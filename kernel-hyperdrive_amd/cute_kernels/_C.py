@@ -1,0 +1,332 @@
+"""ctypes binding of ``libcute_hip.so`` (C ABI declared in ``include/cute_hip.h``).
+
+This is the only module that touches the native library.  It plays the part of the reference's
+``cpp_jit`` (cute_kernels/jit.py:63-89): kernel launchers elsewhere in the package call
+``_C.<function>(tensor, ...)`` and get a kernel launch on torch's current stream.  There is no
+fallback: if the library cannot be loaded the first call raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+
+import torch
+
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libcute_hip.so")
+_ABI_VERSION = 1
+
+_lib = None
+_lock = threading.Lock()
+
+CK_F32, CK_F16, CK_BF16 = 0, 1, 2
+_DTYPE_CODE = {torch.float32: CK_F32, torch.float16: CK_F16, torch.bfloat16: CK_BF16}
+
+_p = ctypes.c_void_p
+_i64 = ctypes.c_int64
+_i32 = ctypes.c_int
+_f32 = ctypes.c_float
+
+# name -> (restype, argtypes); mirrors include/cute_hip.h declaration by declaration
+_SIGNATURES = {
+    "ck_status_string": (ctypes.c_char_p, [_i32]),
+    "ck_abi_version": (_i32, []),
+    "ck_swiglu_forward": (_i32, [_p, _p, _p, _i64, _i32, _i32, _p]),
+    "ck_swiglu_backward": (_i32, [_p, _p, _p, _p, _p, _i64, _i32, _i32, _p]),
+    "ck_swiglu_unchunked_forward": (_i32, [_p, _p, _i64, _i64, _i32, _i32, _p]),
+    "ck_swiglu_unchunked_backward": (_i32, [_p, _p, _p, _i64, _i64, _i32, _i32, _p]),
+    "ck_rmsnorm_forward": (_i32, [_p, _p, _p, _p, _i64, _i64, _f32, _i32, _p]),
+    "ck_rmsnorm_backward_workspace_size": (_i64, [_i64, _i64]),
+    "ck_rmsnorm_backward": (_i32, [_p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _f32, _i32, _p]),
+    "ck_embedding_forward": (_i32, [_p, _i32, _p, _p, _i64, _i64, _i64, _i32, _p]),
+    "ck_embedding_backward_workspace_size": (_i64, [_i64, _i64, _i64]),
+    "ck_embedding_backward": (_i32, [_p, _i32, _p, _p, _p, _i64, _i64, _i64, _i64, _i32, _p]),
+    "ck_contiguous_count": (_i32, [_p, _i32, _p, _i64, _i64, _p]),
+    "ck_moe_sort_workspace_size": (_i64, [_i64, _i64]),
+    "ck_moe_sort": (_i32, [_p, _i32, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
+    "ck_scatter2scatter": (
+        _i32,
+        [_p, _i64, _p, _i64, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _p],
+    ),
+    "ck_offsets_from_sorted": (_i32, [_p, _p, _i64, _i64, _p]),
+    "ck_group_bwd_W": (_i32, [_p, _i64, _p, _i64, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _p]),
+    "ck_group": (_i32, [_p, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _i32, _p]),
+}
+
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+
+def library_path() -> str:
+    return _LIB_PATH
+
+
+def load_library() -> ctypes.CDLL:
+    """Load (building first if nothing is built) and type the native library."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not os.path.exists(_LIB_PATH):
+            from ._build import build
+
+            build()
+        lib = ctypes.CDLL(_LIB_PATH)
+        for name, (restype, argtypes) in _SIGNATURES.items():
+            fn = getattr(lib, name)  # AttributeError here = library older than this binding
+            fn.restype = restype
+            fn.argtypes = argtypes
+        if lib.ck_abi_version() != _ABI_VERSION:
+            raise RuntimeError(
+                f"libcute_hip.so has ABI version {lib.ck_abi_version()}, this package needs {_ABI_VERSION}: rebuild it"
+            )
+        _lib = lib
+    return _lib
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise ValueError(f"unsupported dtype ({dtype}); the HIP kernels take float32, float16 and bfloat16") from None
+
+
+def _ptr(t: torch.Tensor | None):
+    return None if t is None else t.data_ptr()
+
+
+def _require_gpu(*tensors: torch.Tensor | None) -> torch.device:
+    device = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError("cute_kernels HIP kernels need GPU tensors; got a tensor on " + str(t.device))
+        if device is None:
+            device = t.device
+        elif t.device != device:
+            raise RuntimeError(f"tensors on different devices ({device} and {t.device})")
+    if device is None:
+        raise RuntimeError("no tensor argument")
+    return device
+
+
+class _Launch:
+    """Context for one native call: the tensors' device made current, its stream fetched."""
+
+    __slots__ = ("device", "guard", "stream")
+
+    def __init__(self, *tensors):
+        self.device = _require_gpu(*tensors)
+        self.guard = None
+
+    def __enter__(self):
+        if self.device.index != torch.cuda.current_device():
+            self.guard = torch.cuda.device(self.device)
+            self.guard.__enter__()
+        self.stream = torch.cuda.current_stream().cuda_stream
+        return self
+
+    def __exit__(self, *exc):
+        if self.guard is not None:
+            self.guard.__exit__(*exc)
+        return False
+
+
+def _check(status: int, name: str) -> None:
+    if status != 0:
+        text = load_library().ck_status_string(status).decode()
+        raise RuntimeError(f"{name} failed: {text} (status {status})")
+
+
+def _ids_are_i32(ids: torch.Tensor) -> int:
+    if ids.dtype == torch.int32:
+        return 1
+    if ids.dtype == torch.int64:
+        return 0
+    raise ValueError(f"index tensor must be int32 or int64, got {ids.dtype}")
+
+
+# ---- one Python function per C entry point ----------------------------------------------------------
+# All tensors must be contiguous unless a stride is passed explicitly.
+
+
+def swiglu_forward(gate, up, output, block_size: int) -> None:
+    lib = load_library()
+    with _Launch(gate, up, output) as L:
+        _check(
+            lib.ck_swiglu_forward(_ptr(gate), _ptr(up), _ptr(output), gate.numel(), dtype_code(gate.dtype),
+                                  block_size, L.stream),
+            "ck_swiglu_forward",
+        )
+
+
+def swiglu_backward(gate, up, output_grad, gate_grad, up_grad, block_size: int) -> None:
+    lib = load_library()
+    with _Launch(gate, up, output_grad, gate_grad, up_grad) as L:
+        _check(
+            lib.ck_swiglu_backward(_ptr(gate), _ptr(up), _ptr(output_grad), _ptr(gate_grad), _ptr(up_grad),
+                                   gate.numel(), dtype_code(gate.dtype), block_size, L.stream),
+            "ck_swiglu_backward",
+        )
+
+
+def swiglu_unchunked_forward(x, output, block_size: int) -> None:
+    lib = load_library()
+    H = x.size(-1)
+    B = x.numel() // H if H > 0 else 0
+    with _Launch(x, output) as L:
+        _check(
+            lib.ck_swiglu_unchunked_forward(_ptr(x), _ptr(output), B, H, dtype_code(x.dtype), block_size, L.stream),
+            "ck_swiglu_unchunked_forward",
+        )
+
+
+def swiglu_unchunked_backward(x, output_grad, x_grad, block_size: int) -> None:
+    lib = load_library()
+    H = x.size(-1)
+    B = x.numel() // H if H > 0 else 0
+    with _Launch(x, output_grad, x_grad) as L:
+        _check(
+            lib.ck_swiglu_unchunked_backward(_ptr(x), _ptr(output_grad), _ptr(x_grad), B, H, dtype_code(x.dtype),
+                                             block_size, L.stream),
+            "ck_swiglu_unchunked_backward",
+        )
+
+
+def rmsnorm_forward(x, weight, output, rstd, eps: float) -> None:
+    lib = load_library()
+    H = x.size(-1)
+    B = x.numel() // H if H > 0 else 0
+    with _Launch(x, weight, output, rstd) as L:
+        _check(
+            lib.ck_rmsnorm_forward(_ptr(x), _ptr(weight), _ptr(output), _ptr(rstd), B, H, eps, dtype_code(x.dtype),
+                                   L.stream),
+            "ck_rmsnorm_forward",
+        )
+
+
+def rmsnorm_backward_workspace_size(B: int, H: int, device: torch.device) -> int:
+    lib = load_library()
+    with torch.cuda.device(device):
+        return lib.ck_rmsnorm_backward_workspace_size(B, H)
+
+
+def rmsnorm_backward(x, weight, output_grad, rstd, x_grad, weight_grad, workspace, eps: float) -> None:
+    lib = load_library()
+    H = x.size(-1)
+    B = x.numel() // H if H > 0 else 0
+    with _Launch(x, weight, output_grad, rstd, x_grad, weight_grad, workspace) as L:
+        _check(
+            lib.ck_rmsnorm_backward(_ptr(x), _ptr(weight), _ptr(output_grad), _ptr(rstd), _ptr(x_grad),
+                                    _ptr(weight_grad), _ptr(workspace),
+                                    0 if workspace is None else workspace.numel() * workspace.element_size(), B, H,
+                                    eps, dtype_code(x.dtype), L.stream),
+            "ck_rmsnorm_backward",
+        )
+
+
+def embedding_forward(input_ids, weight, output) -> None:
+    lib = load_library()
+    with _Launch(input_ids, weight, output) as L:
+        _check(
+            lib.ck_embedding_forward(_ptr(input_ids), _ids_are_i32(input_ids), _ptr(weight), _ptr(output),
+                                     input_ids.numel(), weight.size(0), weight.size(1), dtype_code(weight.dtype),
+                                     L.stream),
+            "ck_embedding_forward",
+        )
+
+
+def embedding_backward_workspace_size(num_ids: int, V: int, H: int) -> int:
+    return load_library().ck_embedding_backward_workspace_size(num_ids, V, H)
+
+
+def embedding_backward(input_ids, output_grad, weight_grad, workspace) -> None:
+    lib = load_library()
+    with _Launch(input_ids, output_grad, weight_grad, workspace) as L:
+        _check(
+            lib.ck_embedding_backward(_ptr(input_ids), _ids_are_i32(input_ids), _ptr(output_grad), _ptr(weight_grad),
+                                      _ptr(workspace), workspace.numel() * workspace.element_size(),
+                                      input_ids.numel(), weight_grad.size(0), weight_grad.size(1),
+                                      dtype_code(weight_grad.dtype), L.stream),
+            "ck_embedding_backward",
+        )
+
+
+def contiguous_count(x, output, size: int) -> None:
+    lib = load_library()
+    with _Launch(x, output) as L:
+        _check(
+            lib.ck_contiguous_count(_ptr(x), _ids_are_i32(x), _ptr(output), x.numel(), size, L.stream),
+            "ck_contiguous_count",
+        )
+
+
+def moe_sort_workspace_size(M: int, E: int) -> int:
+    return load_library().ck_moe_sort_workspace_size(M, E)
+
+
+def moe_sort(expert_ids, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, workspace, E: int) -> None:
+    lib = load_library()
+    with _Launch(expert_ids, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, workspace) as L:
+        _check(
+            lib.ck_moe_sort(_ptr(expert_ids), _ids_are_i32(expert_ids), _ptr(sorted_expert_idxs),
+                            _ptr(sorted_scattered_idxs), _ptr(expert_offsets), _ptr(workspace),
+                            0 if workspace is None else workspace.numel() * workspace.element_size(),
+                            expert_ids.numel(), E, L.stream),
+            "ck_moe_sort",
+        )
+
+
+def offsets_from_sorted(sorted_expert_idxs, expert_offsets) -> None:
+    lib = load_library()
+    with _Launch(sorted_expert_idxs, expert_offsets) as L:
+        _check(
+            lib.ck_offsets_from_sorted(_ptr(sorted_expert_idxs), _ptr(expert_offsets), sorted_expert_idxs.numel(),
+                                       expert_offsets.numel(), L.stream),
+            "ck_offsets_from_sorted",
+        )
+
+
+def scatter2scatter(X, W, sorted_scattered_idxs, expert_offsets, out, fan_out: int, x_grouped: bool,
+                    y_grouped: bool) -> None:
+    """X [*, K] (unit column stride), W strided view [E, K, N], out [slots, N] (unit column stride)."""
+    lib = load_library()
+    if X.stride(1) != 1 or out.stride(1) != 1:
+        raise ValueError("scatter2scatter needs unit column stride for X and out")
+    with _Launch(X, W, sorted_scattered_idxs, expert_offsets, out) as L:
+        _check(
+            lib.ck_scatter2scatter(_ptr(X), X.stride(0), _ptr(W), W.stride(0), W.stride(1), W.stride(2),
+                                   _ptr(sorted_scattered_idxs), _ptr(expert_offsets), _ptr(out), out.stride(0),
+                                   out.size(0), X.size(1), out.size(1), W.size(0), fan_out, int(x_grouped),
+                                   int(y_grouped), dtype_code(X.dtype), L.stream),
+            "ck_scatter2scatter",
+        )
+
+
+def group_bwd_W(DY, X, expert_offsets, DW, E: int) -> None:
+    lib = load_library()
+    if X.stride(1) != 1 or DY.stride(1) != 1:
+        raise ValueError("group_bwd_W needs unit column stride for X and DY")
+    with _Launch(DY, X, expert_offsets, DW) as L:
+        _check(
+            lib.ck_group_bwd_W(_ptr(DY), DY.stride(0), _ptr(X), X.stride(0), _ptr(expert_offsets), _ptr(DW),
+                               DW.stride(0), DW.stride(1), DW.stride(2), X.size(0), X.size(1), DY.size(1), E,
+                               dtype_code(X.dtype), L.stream),
+            "ck_group_bwd_W",
+        )
+
+
+def group(A, idx, coeff, out, fan_out: int) -> None:
+    lib = load_library()
+    if A.stride(1) != 1 or out.stride(1) != 1:
+        raise ValueError("group needs unit column stride for A and out")
+    with _Launch(A, idx, coeff, out) as L:
+        _check(
+            lib.ck_group(_ptr(A), A.stride(0), _ptr(idx), _ptr(coeff), _ptr(out), out.stride(0), idx.numel(),
+                         A.size(1), fan_out, dtype_code(A.dtype), L.stream),
+            "ck_group",
+        )

@@ -1,0 +1,78 @@
+"""Builds ``lib/libcute_hip.so`` from the HIP sources in ``../csrc`` with hipcc for gfx950.
+
+One shared library, plain C ABI (declared in ``include/cute_hip.h`` at the repository root).  The
+reference compiles its CUDA sources lazily, per op, through ``torch.utils.cpp_extension.load``
+(cute_kernels/jit.py:16-49); here everything is compiled ahead of time in one step so that the built
+library can be shipped next to the Python package.
+"""
+
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+from concurrent.futures import ThreadPoolExecutor
+
+
+PACKAGE_DIR = os.path.dirname(os.path.abspath(__file__))
+CSRC_DIR = os.path.normpath(os.path.join(PACKAGE_DIR, "..", "csrc"))
+LIB_DIR = os.path.join(PACKAGE_DIR, "lib")
+LIB_PATH = os.path.join(LIB_DIR, "libcute_hip.so")
+
+SOURCES = ["status.hip", "swiglu.hip", "rmsnorm.hip", "embedding.hip", "moe_sort.hip", "grouped_gemm.hip"]
+
+# -packed-fp32-ops off: the packed fp32 VALU forms are not wanted in any kernel of this library
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-Wall",
+    "-Wno-unused-function",
+    "-Xclang",
+    "-target-feature",
+    "-Xclang",
+    "-packed-fp32-ops",
+]
+
+
+def find_hipcc() -> str:
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        raise RuntimeError("hipcc not found: the HIP kernels of cute_kernels cannot be built")
+    return hipcc
+
+
+def _compile(hipcc: str, source: str, obj_dir: str, verbose: bool) -> str:
+    obj = os.path.join(obj_dir, os.path.splitext(source)[0] + ".o")
+    cmd = [hipcc, *HIPCC_FLAGS, "-c", os.path.join(CSRC_DIR, source), "-o", obj]
+    result = subprocess.run(cmd, capture_output=True, text=True)
+    # hipcc's host pass warns that it does not know the packed-fp32 feature; that line is noise
+    stderr = "\n".join(line for line in result.stderr.splitlines() if "packed-fp32-ops" not in line)
+    if result.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {source}:\n{stderr}")
+    if verbose and stderr.strip():
+        print(stderr)
+    return obj
+
+
+def build(verbose: bool = False, jobs: int | None = None) -> str:
+    """Compile every source and link the shared library; returns its path."""
+    hipcc = find_hipcc()
+    obj_dir = os.path.join(PACKAGE_DIR, "..", "build", "obj")
+    os.makedirs(obj_dir, exist_ok=True)
+    os.makedirs(LIB_DIR, exist_ok=True)
+    jobs = jobs or min(len(SOURCES), os.cpu_count() or 1, 16)
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        objects = list(pool.map(lambda src: _compile(hipcc, src, obj_dir, verbose), SOURCES))
+    tmp = LIB_PATH + ".tmp"
+    link = subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objects, "-o", tmp],
+                          capture_output=True, text=True)
+    if link.returncode != 0:
+        raise RuntimeError(f"linking libcute_hip.so failed:\n{link.stderr}")
+    os.replace(tmp, LIB_PATH)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

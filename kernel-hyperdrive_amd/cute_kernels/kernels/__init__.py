@@ -1,0 +1,6 @@
+from .contiguous_count import contiguous_count_cute
+from .embedding import embedding_cute, embedding_torch
+from .rmsnorm import rmsnorm_cute, rmsnorm_torch
+from .scattermoe import MoE_HIP, MoE_Torch, MoE_Triton, scattered_experts
+from .swiglu import swiglu_cute, swiglu_torch
+from .swiglu_unchunked import swiglu_unchunked_cute, swiglu_unchunked_torch

@@ -1,0 +1,206 @@
+"""RMSNorm over the last dimension, forward and backward.
+
+Public function and autograd signature follow cute_kernels/kernels/rmsnorm/__init__.py:11-106 (1-D input,
+``eps=None`` -> ``torch.finfo(dtype).eps``, optional weight, ``memory_efficient`` recomputation of 1/rms).
+The HIP kernels choose their own row tiling from the row length, so the BLOCK_SIZE_B / BLOCK_SIZE_H
+arguments of the reference are accepted for call compatibility and do not change the launch.
+"""
+
+import torch
+import torch.nn.functional as F
+
+from .. import _C
+from ..constants import LIBRARY_NAME, MAX_ROW_LENGTH
+from ..cutotune import CutoTuneConfig, CutoTuneParameter, cutotune
+from ..enums import KernelBackend
+from ..utils import cute_op, ensure_contiguous
+from ._common import check_backend
+
+
+def rmsnorm_torch(x: torch.Tensor, weight: torch.Tensor | None, eps: float | None) -> torch.Tensor:
+    return F.rms_norm(x, (x.size(-1),), weight=weight, eps=eps)
+
+
+@cute_op(f"{LIBRARY_NAME}::rmsnorm_forward_hip", mutates_args={"output", "rmsnorm_denominator"})
+def rmsnorm_forward_hip(
+    x: torch.Tensor,
+    weight: torch.Tensor | None,
+    output: torch.Tensor,
+    eps: float,
+    rmsnorm_denominator: torch.Tensor | None,
+) -> None:
+    _C.rmsnorm_forward(x, weight, output, rmsnorm_denominator, eps)
+
+
+@cute_op(f"{LIBRARY_NAME}::rmsnorm_backward_hip", mutates_args={"x_grad", "weight_grad", "workspace"})
+def rmsnorm_backward_hip(
+    x: torch.Tensor,
+    weight: torch.Tensor | None,
+    output_grad: torch.Tensor,
+    rmsnorm_denominator: torch.Tensor | None,
+    x_grad: torch.Tensor,
+    weight_grad: torch.Tensor | None,
+    workspace: torch.Tensor | None,
+    eps: float,
+) -> None:
+    _C.rmsnorm_backward(x, weight, output_grad, rmsnorm_denominator, x_grad, weight_grad, workspace, eps)
+
+
+_ONLY_CONFIG = CutoTuneConfig({"kernel_backend": KernelBackend.hip})
+
+
+def _check_row_length(hidden_size: int) -> None:
+    if hidden_size > MAX_ROW_LENGTH:
+        raise ValueError(f"hidden size ({hidden_size}) is larger than the longest supported row ({MAX_ROW_LENGTH})")
+
+
+@cutotune(configs=[_ONLY_CONFIG], default_config=_ONLY_CONFIG, triggers={"x.dtype"})
+def _forward(
+    x: torch.Tensor,
+    weight: torch.Tensor | None,
+    eps: float,
+    memory_efficient: bool,
+    kernel_backend: KernelBackend,
+    BLOCK_SIZE_B: int,
+    BLOCK_SIZE_H: int,
+) -> tuple[torch.Tensor, torch.Tensor | None]:
+    check_backend(kernel_backend)
+    hidden_size = x.size(-1)
+    _check_row_length(hidden_size)
+    num_rows = x.numel() // hidden_size if hidden_size > 0 else 0
+
+    output = torch.empty_like(x)
+    rmsnorm_denominator = None if memory_efficient else torch.empty(num_rows, device=x.device, dtype=torch.float32)
+    rmsnorm_forward_hip(x=x, weight=weight, output=output, eps=eps, rmsnorm_denominator=rmsnorm_denominator)
+    return output, rmsnorm_denominator
+
+
+@cutotune(configs=[_ONLY_CONFIG], default_config=_ONLY_CONFIG, triggers={"x.dtype"})
+def _backward(
+    x: torch.Tensor,
+    weight: torch.Tensor | None,
+    eps: float,
+    rmsnorm_denominator: torch.Tensor | None,
+    output_grad: torch.Tensor,
+    kernel_backend: KernelBackend,
+    BLOCK_SIZE_B: int,
+    BLOCK_SIZE_H: int,
+) -> tuple[torch.Tensor, torch.Tensor | None]:
+    check_backend(kernel_backend)
+    hidden_size = x.size(-1)
+    _check_row_length(hidden_size)
+    num_rows = x.numel() // hidden_size if hidden_size > 0 else 0
+
+    x_grad = torch.empty_like(x)
+    weight_grad = None
+    workspace = None
+    if weight is not None:
+        weight_grad = torch.empty_like(weight)
+        nbytes = _C.rmsnorm_backward_workspace_size(num_rows, hidden_size, x.device)
+        workspace = torch.empty(max(nbytes, 16), device=x.device, dtype=torch.uint8)
+    rmsnorm_backward_hip(
+        x=x,
+        weight=weight,
+        output_grad=output_grad,
+        rmsnorm_denominator=rmsnorm_denominator,
+        x_grad=x_grad,
+        weight_grad=weight_grad,
+        workspace=workspace,
+        eps=eps,
+    )
+    return x_grad, weight_grad
+
+
+class _RMSNorm_Cute(torch.autograd.Function):
+    @staticmethod
+    @ensure_contiguous
+    def forward(
+        ctx,
+        x: torch.Tensor,
+        weight: torch.Tensor | None,
+        eps: float | None,
+        memory_efficient: bool,
+        kernel_backend_forward: KernelBackend,
+        kernel_backend_backward: KernelBackend,
+        BLOCK_SIZE_B_forward: int,
+        BLOCK_SIZE_B_backward: int,
+        BLOCK_SIZE_H_forward: int,
+        BLOCK_SIZE_H_backward: int,
+    ) -> torch.Tensor:
+        if weight is not None:
+            assert weight.dim() == 1, "weight should be 1D"
+            assert weight.size(-1) == x.size(-1), "hidden size for x and weight tensor is different"
+            assert weight.type() == x.type(), "tensors weight and y should have same dtype"
+
+        is_x_1d = x.dim() == 1
+        if is_x_1d:
+            x = x.unsqueeze(0)
+        if eps is None:
+            eps = torch.finfo(x.dtype).eps
+
+        output, rmsnorm_denominator = _forward(
+            x=x,
+            weight=weight,
+            eps=eps,
+            memory_efficient=memory_efficient,
+            kernel_backend=kernel_backend_forward,
+            BLOCK_SIZE_B=BLOCK_SIZE_B_forward,
+            BLOCK_SIZE_H=BLOCK_SIZE_H_forward,
+        )
+        if is_x_1d:
+            output = output.squeeze(0)
+
+        ctx.save_for_backward(x, weight, rmsnorm_denominator)
+        ctx.is_x_1d = is_x_1d
+        ctx.eps = eps
+        ctx.kernel_backend_backward = kernel_backend_backward
+        ctx.BLOCK_SIZE_B_backward = BLOCK_SIZE_B_backward
+        ctx.BLOCK_SIZE_H_backward = BLOCK_SIZE_H_backward
+        return output
+
+    @staticmethod
+    @ensure_contiguous
+    def backward(ctx, output_grad: torch.Tensor):
+        x, weight, rmsnorm_denominator = ctx.saved_tensors
+        if ctx.is_x_1d:
+            output_grad = output_grad.unsqueeze(0)
+
+        x_grad, weight_grad = _backward(
+            x=x,
+            weight=weight,
+            eps=ctx.eps,
+            rmsnorm_denominator=rmsnorm_denominator,
+            output_grad=output_grad,
+            kernel_backend=ctx.kernel_backend_backward,
+            BLOCK_SIZE_B=ctx.BLOCK_SIZE_B_backward,
+            BLOCK_SIZE_H=ctx.BLOCK_SIZE_H_backward,
+        )
+        if ctx.is_x_1d:
+            x_grad = x_grad.squeeze(0)
+        return x_grad, weight_grad, None, None, None, None, None, None, None, None
+
+
+def rmsnorm_cute(
+    x: torch.Tensor,
+    weight: torch.Tensor | None,
+    eps: float | None,
+    memory_efficient: bool = False,
+    kernel_backend_forward: KernelBackend = CutoTuneParameter(),
+    kernel_backend_backward: KernelBackend = CutoTuneParameter(),
+    BLOCK_SIZE_B_forward: int = CutoTuneParameter(),
+    BLOCK_SIZE_B_backward: int = CutoTuneParameter(),
+    BLOCK_SIZE_H_forward: int = CutoTuneParameter(),
+    BLOCK_SIZE_H_backward: int = CutoTuneParameter(),
+) -> torch.Tensor:
+    return _RMSNorm_Cute.apply(
+        x,
+        weight,
+        eps,
+        memory_efficient,
+        kernel_backend_forward,
+        kernel_backend_backward,
+        BLOCK_SIZE_B_forward,
+        BLOCK_SIZE_B_backward,
+        BLOCK_SIZE_H_forward,
+        BLOCK_SIZE_H_backward,
+    )

@@ -1,0 +1,219 @@
+"""ScatterMoE operators on the HIP grouped-GEMM kernels.
+
+``scatter2scatter``, ``group_bwd_W`` and ``group`` keep the names, argument order and ``cute::`` custom-op
+registration of cute_kernels/kernels/scattermoe/triton_implementation/ops.py:16-130, and
+``_ScatteredExperts`` / ``scattered_experts`` the autograd contract of ops.py:133-301 (same inputs, same
+saved tensors, same nine gradient slots).  Differences that do not change results:
+  * ``scatter2scatter`` takes the expert offsets as an optional trailing argument (the tile scheduler works
+    per expert); without it they are recomputed from the sorted expert ids;
+  * the weight gradient is written completely by the kernel (zeros for experts without rows), so it is
+    allocated with ``empty_like`` instead of ``zeros_like`` (ops.py:237).
+"""
+
+import torch
+
+from ... import _C
+from ...constants import LIBRARY_NAME
+from ...utils import cute_op
+
+
+torch._dynamo.config.capture_scalar_outputs = True
+
+
+@cute_op(f"{LIBRARY_NAME}::scatter2scatter", mutates_args={"out"})
+def scatter2scatter(
+    X: torch.Tensor,
+    W: torch.Tensor,
+    sorted_expert_idxs: torch.Tensor,
+    sorted_scattered_idxs: torch.Tensor,
+    out: torch.Tensor,
+    FAN_OUT: int,
+    x_grouped: bool = False,
+    y_grouped: bool = False,
+    expert_offsets: torch.Tensor | None = None,
+) -> None:
+    assert sorted_scattered_idxs.size(0) == sorted_expert_idxs.size(0)
+    assert sorted_scattered_idxs.size(0) == X.size(0) * FAN_OUT
+    assert out.size(0) == sorted_expert_idxs.size(0)
+    assert out.size(1) == W.size(-1)
+    assert X.size(1) == W.size(1)
+
+    if expert_offsets is None:
+        expert_offsets = torch.empty(W.size(0), dtype=torch.int64, device=X.device)
+        _C.offsets_from_sorted(sorted_expert_idxs.contiguous(), expert_offsets)
+    if X.stride(1) != 1:
+        X = X.contiguous()
+    _C.scatter2scatter(X, W, sorted_scattered_idxs, expert_offsets, out, FAN_OUT, x_grouped, y_grouped)
+
+
+@cute_op(f"{LIBRARY_NAME}::group_bwd_W", mutates_args={"DW"})
+def group_bwd_W(DY: torch.Tensor, X: torch.Tensor, expert_offsets: torch.Tensor, DW: torch.Tensor, E: int) -> None:
+    assert DY.size(0) == X.size(0)
+    assert DW.size(0) == E and DW.size(1) == X.size(1) and DW.size(2) == DY.size(1)
+    if DY.stride(1) != 1:
+        DY = DY.contiguous()
+    if X.stride(1) != 1:
+        X = X.contiguous()
+    _C.group_bwd_W(DY, X, expert_offsets, DW, E)
+
+
+@cute_op(f"{LIBRARY_NAME}::group", mutates_args={"out"})
+def group(
+    A: torch.Tensor,
+    sorted_expert_idxs: torch.Tensor,
+    out: torch.Tensor,
+    coeff: torch.Tensor | None = None,
+    fan_out: int = 1,
+) -> None:
+    # (the reference names the index argument `sorted_expert_idxs`; callers pass sorted_scattered_idxs)
+    assert A.size(0) * fan_out == sorted_expert_idxs.size(0)
+    assert out.size(0) == sorted_expert_idxs.size(0) and out.size(1) == A.size(1)
+    if A.stride(1) != 1:
+        A = A.contiguous()
+    _C.group(A, sorted_expert_idxs, coeff, out, fan_out)
+
+
+class _ScatteredExperts(torch.autograd.Function):
+    @staticmethod
+    def forward(
+        ctx,
+        x,
+        expert_weights,
+        k,
+        sorted_expert_idxs,
+        sorted_scattered_idxs,
+        expert_offsets,
+        gates=None,
+        grouped_in=False,
+        grouped_out=False,
+    ):
+        # expert_weights: view [E, in, out] of the [E, out, in] parameter
+        output = torch.empty(sorted_expert_idxs.size(0), expert_weights.size(-1), device=x.device, dtype=x.dtype)
+        scatter2scatter(
+            X=x,
+            W=expert_weights,
+            sorted_expert_idxs=sorted_expert_idxs,
+            sorted_scattered_idxs=sorted_scattered_idxs,
+            out=output,
+            FAN_OUT=k,
+            x_grouped=grouped_in,
+            y_grouped=grouped_out,
+            expert_offsets=expert_offsets,
+        )
+
+        if gates is None:
+            output_expanded = None
+        else:
+            # rows are back in (token, slot) order: mix each token's k expert outputs with its routing weights
+            output_expanded = output.view(gates.size(0), gates.size(1), output.size(-1))
+            output = torch.bmm(gates.unsqueeze(1), output_expanded).squeeze(1)
+
+        ctx.save_for_backward(
+            x, expert_weights, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, gates, output_expanded
+        )
+        ctx.grouped_in = grouped_in
+        ctx.grouped_out = grouped_out
+        ctx.k = k
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        (
+            x,
+            expert_weights,
+            sorted_expert_idxs,
+            sorted_scattered_idxs,
+            expert_offsets,
+            gates,
+            output_expanded,
+        ) = ctx.saved_tensors
+        k = ctx.k
+        grouped_in = ctx.grouped_in
+        grouped_out = ctx.grouped_out
+        num_slots = sorted_expert_idxs.size(0)
+        grad_out = grad_out.contiguous()
+
+        # --- gradient of the routing weights, and grad_out brought into expert-grouped row order ---------
+        if gates is None:
+            d_gates = None
+            gates_flat = None
+            gate_fan = 1
+            grouped_grad_out = None
+        else:
+            d_gates = torch.bmm(output_expanded, grad_out.unsqueeze(2)).squeeze(-1)
+            gates_flat = gates.flatten()
+            gate_fan = gates.size(1)
+            grouped_grad_out = output_expanded.flatten(0, 1)  # saved buffer, overwritten below
+
+        if grouped_out:
+            grouped_grad_out = grad_out
+        else:
+            if grouped_grad_out is None:
+                grouped_grad_out = torch.empty(num_slots, grad_out.size(1), dtype=grad_out.dtype, device=grad_out.device)
+            group(
+                A=grad_out,
+                sorted_expert_idxs=sorted_scattered_idxs,
+                out=grouped_grad_out,
+                coeff=gates_flat,
+                fan_out=gate_fan,
+            )
+
+        # --- expert-grouped input rows ----------------------------------------------------------------
+        if grouped_in:
+            grouped_x = x
+            d_expanded_input = torch.empty(num_slots, expert_weights.size(1), device=x.device, dtype=x.dtype)
+        else:
+            grouped_x = torch.empty(num_slots, x.size(1), dtype=x.dtype, device=x.device)
+            group(A=x, sorted_expert_idxs=sorted_scattered_idxs, out=grouped_x, fan_out=k)
+            d_expanded_input = grouped_x  # reused once the weight gradient has consumed it
+
+        # --- weight gradient: DW[e] = X_e^T DY_e, laid out like the parameter view --------------------
+        d_weights = torch.empty_like(expert_weights)
+        group_bwd_W(
+            DY=grouped_grad_out, X=grouped_x, expert_offsets=expert_offsets, DW=d_weights, E=expert_weights.size(0)
+        )
+
+        # --- input gradient: DY_e W_e^T, scattered back unless the input was grouped --------------------
+        scatter2scatter(
+            X=grouped_grad_out,
+            W=expert_weights.permute(0, 2, 1),
+            sorted_expert_idxs=sorted_expert_idxs,
+            sorted_scattered_idxs=sorted_scattered_idxs,
+            out=d_expanded_input,
+            FAN_OUT=1,
+            x_grouped=True,
+            y_grouped=grouped_in,
+            expert_offsets=expert_offsets,
+        )
+
+        if k == 1:
+            d_input = d_expanded_input
+        else:
+            d_input = d_expanded_input.view(x.size(0), k, d_expanded_input.size(-1)).sum(-2)
+
+        # x, expert_weights, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, gates, grouped_in, grouped_out
+        return d_input, d_weights, None, None, None, None, d_gates, None, None
+
+
+def scattered_experts(
+    inputs,
+    expert_weights,
+    k,
+    sorted_expert_idxs,
+    sorted_scattered_idxs,
+    expert_offsets,
+    gates=None,
+    grouped_in=False,
+    grouped_out=False,
+):
+    return _ScatteredExperts.apply(
+        inputs,
+        expert_weights,
+        k,
+        sorted_expert_idxs,
+        sorted_scattered_idxs,
+        expert_offsets,
+        gates,
+        grouped_in,
+        grouped_out,
+    )

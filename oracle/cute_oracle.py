@@ -1,0 +1,340 @@
+"""CPU oracle for the cute_kernels hot path.  TEST INFRASTRUCTURE ONLY.
+
+This module restates, with plain torch / numpy on the CPU, what the reference computes on the hot path, so
+that the HIP kernels can be checked against it.  Only tests, ``__graft_entry__.smoke()`` and the
+``cpu_baseline`` leg of ``bench.py`` may import it; nothing in the shipped package does.
+
+How each function is pinned (the reference holds no golden vectors for this path; its tests compare against
+stock torch ops on random inputs):
+  swiglu_*            closed form cute_kernels/kernels/swiglu/README.md:3-13; checked against autograd of
+                      ``up * F.silu(gate)`` in fp64 and the limits g -> +-inf, g = 0
+  rmsnorm_*           closed form cute_kernels/kernels/rmsnorm/README.md:3-25; checked against autograd of
+                      ``F.rms_norm`` in fp64, scale invariance and the dx.x identity
+  embedding_*         one_hot(ids)^T @ dy (cute_kernels/kernels/embedding/README.md:7-15); checked against a
+                      dense one-hot matmul and ``F.embedding`` autograd in fp64
+  contiguous_count    numpy.bincount(minlength) (tests/kernels/contiguous_count_test.py:35)
+  moe_sort            stable argsort; checked against a brute-force insertion on tiny inputs
+  scatter2scatter, group_bwd_W, group
+                      per-slot / per-expert loops straight from the kernel docstrings
+                      (scattermoe/triton_implementation/kernels.py:66-102, 152-240, 243-298)
+  moe_forward_backward
+                      restatement of MoE_Torch (scattermoe/torch_implementation.py:101-199) with bincount in
+                      place of the Triton histogram; checked against an independent per-token dense
+                      formulation (y_t = sum_j softmax_j * FFN_{e_j}(x_t)) and its autograd in fp64
+No function here is "parity unpinned".
+
+Precision policy: inputs are values of the storage dtype (bf16 / fp16 / fp32).  ``compute_dtype=float32``
+gives the expectation "fp32 accumulation, one rounding at the end"; passing the storage dtype runs the
+same torch ops natively in that dtype, which is the reference's own torch implementation.
+"""
+
+from __future__ import annotations
+
+import math
+
+import numpy as np
+import torch
+import torch.nn.functional as F
+
+
+# =====================================================================================================
+# tolerances (BASELINE.json north_star)
+# =====================================================================================================
+TOLERANCE = {
+    torch.float32: dict(rtol=1e-5, atol=1e-5),
+    torch.bfloat16: dict(rtol=2e-2, atol=1e-2),
+    torch.float16: dict(rtol=2e-2, atol=1e-2),
+}
+
+
+def tolerance(dtype: torch.dtype) -> dict:
+    return TOLERANCE[dtype]
+
+
+def fraction_outside(actual: torch.Tensor, expected: torch.Tensor, rtol: float, atol: float) -> float:
+    """Fraction of elements with |actual - expected| > atol + rtol * |expected| (computed in fp64)."""
+    a = actual.detach().double().cpu()
+    e = expected.detach().double().cpu()
+    bad = (a - e).abs() > atol + rtol * e.abs()
+    return bad.double().mean().item() if bad.numel() else 0.0
+
+
+# =====================================================================================================
+# SwiGLU   (cute_kernels/kernels/swiglu/torch_implementation.py:5-6, README.md:3-13)
+# =====================================================================================================
+def _sigmoid(x: torch.Tensor) -> torch.Tensor:
+    # overflow-free form, as cute_kernels/include/activations.h:5-17
+    e = torch.exp(-x.abs())
+    s = 1.0 / (1.0 + e)
+    return torch.where(x >= 0, s, 1.0 - s)
+
+
+def swiglu_forward(gate: torch.Tensor, up: torch.Tensor, compute_dtype=torch.float32) -> torch.Tensor:
+    g, u = gate.to(compute_dtype), up.to(compute_dtype)
+    return (u * g * _sigmoid(g)).to(gate.dtype)
+
+
+def swiglu_backward(gate, up, output_grad, compute_dtype=torch.float32):
+    g, u, dy = gate.to(compute_dtype), up.to(compute_dtype), output_grad.to(compute_dtype)
+    s = _sigmoid(g)
+    gate_grad = dy * u * (s + g * s * (1 - s))
+    up_grad = dy * g * s
+    return gate_grad.to(gate.dtype), up_grad.to(up.dtype)
+
+
+def swiglu_unchunked_forward(x: torch.Tensor, compute_dtype=torch.float32) -> torch.Tensor:
+    # up = first half, gate = second half (swiglu_unchunked/torch_implementation.py:5-7)
+    up, gate = x.chunk(2, dim=-1)
+    return swiglu_forward(gate, up, compute_dtype)
+
+
+def swiglu_unchunked_backward(x, output_grad, compute_dtype=torch.float32) -> torch.Tensor:
+    up, gate = x.chunk(2, dim=-1)
+    gate_grad, up_grad = swiglu_backward(gate, up, output_grad, compute_dtype)
+    return torch.cat([up_grad, gate_grad], dim=-1)
+
+
+# =====================================================================================================
+# RMSNorm   (cute_kernels/kernels/rmsnorm/torch_implementation.py:5-6, README.md:3-25)
+# =====================================================================================================
+def resolve_eps(eps: float | None, dtype: torch.dtype) -> float:
+    # cute_kernels/kernels/rmsnorm/__init__.py:36-37
+    return torch.finfo(dtype).eps if eps is None else eps
+
+
+def rmsnorm_forward(x, weight, eps, compute_dtype=torch.float32):
+    """Returns (y, rstd) with rstd = 1 / sqrt(mean(x^2) + eps) in compute_dtype."""
+    eps = resolve_eps(eps, x.dtype)
+    xf = x.to(compute_dtype)
+    rstd = torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + eps)
+    y = xf * rstd
+    if weight is not None:
+        y = y * weight.to(compute_dtype)
+    return y.to(x.dtype), rstd.squeeze(-1)
+
+
+def rmsnorm_backward(x, weight, output_grad, eps, compute_dtype=torch.float32):
+    """dx = rstd * g - x * rstd^3 / H * sum_h(g x), g = dy * w;  dw = sum_b dy * x * rstd."""
+    eps = resolve_eps(eps, x.dtype)
+    H = x.size(-1)
+    xf = x.to(compute_dtype).reshape(-1, H)
+    dy = output_grad.to(compute_dtype).reshape(-1, H)
+    rstd = torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + eps)
+    g = dy if weight is None else dy * weight.to(compute_dtype)
+    dx = rstd * g - xf * rstd.pow(3) / H * (g * xf).sum(dim=-1, keepdim=True)
+    dw = None if weight is None else (dy * xf * rstd).sum(dim=0).to(weight.dtype)
+    return dx.reshape(x.shape).to(x.dtype), dw
+
+
+# =====================================================================================================
+# Embedding   (cute_kernels/kernels/embedding/torch_implementation.py:5-6, README.md:7-15)
+# =====================================================================================================
+def embedding_forward(input_ids: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    return weight[input_ids.reshape(-1).long()].reshape(*input_ids.shape, weight.size(-1))
+
+
+def embedding_backward(input_ids, output_grad, vocab_size: int, compute_dtype=torch.float32) -> torch.Tensor:
+    H = output_grad.size(-1)
+    dw = torch.zeros(vocab_size, H, dtype=compute_dtype)
+    dw.index_add_(0, input_ids.reshape(-1).long(), output_grad.reshape(-1, H).to(compute_dtype))
+    return dw.to(output_grad.dtype)
+
+
+# =====================================================================================================
+# integer front end of the MoE layer
+# =====================================================================================================
+def contiguous_count(x: torch.Tensor, size: int) -> torch.Tensor:
+    # tests/kernels/contiguous_count_test.py:35: equals x.bincount(minlength=size); int32 like the kernel
+    counts = np.bincount(x.cpu().numpy().astype(np.int64), minlength=size)[:size]
+    return torch.from_numpy(counts.astype(np.int32))
+
+
+def moe_sort(expert_ids: torch.Tensor, num_experts: int):
+    """(sorted_expert_idxs, sorted_scattered_idxs, expert_offsets), all int64.
+
+    scattermoe/triton_implementation/__init__.py:80-81.  The reference's ``sort()`` leaves the order of equal
+    ids unspecified; the contract here is the stable order, which makes the answer unique.
+    """
+    ids = expert_ids.reshape(-1).cpu().numpy().astype(np.int64)
+    order = np.argsort(ids, kind="stable")
+    counts = np.bincount(ids, minlength=num_experts)[:num_experts]
+    return (
+        torch.from_numpy(ids[order]),
+        torch.from_numpy(order.astype(np.int64)),
+        torch.from_numpy(np.cumsum(counts).astype(np.int64)),
+    )
+
+
+def _expert_of_slot(expert_offsets: torch.Tensor, num_slots: int) -> np.ndarray:
+    ends = expert_offsets.cpu().numpy()
+    return np.searchsorted(ends, np.arange(num_slots), side="right")
+
+
+def scatter2scatter(X, W, sorted_scattered_idxs, expert_offsets, fan_out, x_grouped, y_grouped,
+                    compute_dtype=torch.float32):
+    """out[out_row(i)] = X[in_row(i)] @ W[e(i)];  W is [E, K, N]  (kernels.py:66-102)."""
+    num_slots = sorted_scattered_idxs.numel()
+    expert = _expert_of_slot(expert_offsets, num_slots)
+    idx = sorted_scattered_idxs.cpu().numpy()
+    out = torch.zeros(num_slots, W.size(-1), dtype=compute_dtype)
+    Xc, Wc = X.to(compute_dtype), W.to(compute_dtype)
+    for i in range(num_slots):
+        src = i if x_grouped else idx[i] // fan_out
+        dst = i if y_grouped else idx[i]
+        out[dst] = Xc[src] @ Wc[expert[i]]
+    return out.to(X.dtype)
+
+
+def group_bwd_W(DY, X, expert_offsets, num_experts, compute_dtype=torch.float32):
+    """DW[e] = X_e^T @ DY_e over rows [offsets[e-1], offsets[e])  (kernels.py:152-240); [E, K, N]."""
+    ends = [0] + expert_offsets.tolist()
+    DW = torch.zeros(num_experts, X.size(1), DY.size(1), dtype=compute_dtype)
+    for e in range(num_experts):
+        rows = slice(ends[e], ends[e + 1])
+        DW[e] = X[rows].to(compute_dtype).T @ DY[rows].to(compute_dtype)
+    return DW.to(X.dtype)
+
+
+def group(A, idx, coeff, fan_out):
+    """out[i] = A[idx[i] // fan_out] * coeff[idx[i]]  (kernels.py:243-298), product rounded once."""
+    rows = A[(idx // fan_out).long()]
+    if coeff is None:
+        return rows.clone()
+    return (rows.float() * coeff[idx.long()].float().unsqueeze(-1)).to(A.dtype)
+
+
+# =====================================================================================================
+# the MoE layer   (scattermoe/torch_implementation.py:101-199)
+# =====================================================================================================
+def _acc_dtype(x: torch.Tensor) -> torch.dtype:
+    """fp32 for 16- and 32-bit inputs; fp64 stays fp64 (used when the oracle itself is being pinned)."""
+    return torch.float64 if x.dtype == torch.float64 else torch.float32
+
+
+def swiglu_unchunked_activation(x: torch.Tensor) -> torch.Tensor:
+    """Differentiable activation used between c_fc and c_proj in the BASELINE configs: fp32 math, one rounding."""
+    up, gate = x.chunk(2, dim=-1)
+    acc = _acc_dtype(x)
+    return (up.to(acc) * F.silu(gate.to(acc))).to(x.dtype)
+
+
+def moe_forward(x, w_gate, w_fc, w_proj, top_k: int, activation=swiglu_unchunked_activation, selected=None):
+    """Forward of MoE_Torch on tensors of one dtype; returns (y [T, H], router_logits [T, E]).
+
+    x [T, H]; w_gate [E, H]; w_fc [E, F, H] (F = 2I for a GLU activation); w_proj [E, H, I].
+    ``selected`` ([T, k] expert ids) replaces the top-k decision: logits rounded to 16 bits tie often, and
+    two correct implementations may break a tie differently, so a test passes the decision of the run under
+    test.  The values at the selected positions still come from this function's own logits.
+    """
+    T, H = x.shape
+    E = w_gate.size(0)
+    router_logits = F.linear(x, w_gate)                                       # :122
+    if selected is not None:
+        top_vals = router_logits.gather(1, selected)
+    elif top_k == 1:                                                          # :193-199
+        top_vals, selected = router_logits.max(dim=-1, keepdim=True)
+    else:
+        top_vals, selected = router_logits.topk(top_k, dim=-1)
+    router_weights = F.softmax(top_vals.to(_acc_dtype(x)), dim=-1).type_as(x)  # :130-131 (softmax in fp32)
+
+    flat = selected.flatten()                                                 # :172-191
+    expert_frequency = torch.bincount(flat, minlength=E)
+    order = torch.argsort(flat, stable=True)
+    fan_in_index = order // top_k
+    batch_gates = router_weights.flatten()[order]
+
+    grouped = x[fan_in_index]                                                 # :150
+    splits = expert_frequency.tolist()
+    outs = []
+    for e, rows in enumerate(grouped.split(splits, dim=0)):                   # :36-43, 154-158
+        h = F.linear(rows, w_fc[e])
+        h = activation(h)
+        outs.append(F.linear(h, w_proj[e]))
+    grouped = torch.cat(outs) * batch_gates.unsqueeze(-1)                     # :161
+    # :162-163; the accumulation is done in fp32 and rounded once
+    acc = _acc_dtype(x)
+    y = torch.zeros(T, H, dtype=acc).index_add(0, fan_in_index, grouped.to(acc)).to(x.dtype)
+    return y, router_logits
+
+
+def moe_forward_backward(x, w_gate, w_fc, w_proj, dy, top_k: int, compute_dtype=torch.float32,
+                         activation=swiglu_unchunked_activation, selected=None) -> dict:
+    """Forward and all gradients for loss = sum(y * dy), torch ops run in ``compute_dtype``.
+
+    Results are returned in the dtype of ``x``.
+    """
+    leaves = [t.detach().to(compute_dtype).clone().requires_grad_(True) for t in (x, w_gate, w_fc, w_proj)]
+    y, router_logits = moe_forward(*leaves, top_k=top_k, activation=activation, selected=selected)
+    (y * dy.to(compute_dtype)).sum().backward()
+    out_dtype = x.dtype
+    return {
+        "y": y.detach().to(out_dtype),
+        "router_logits": router_logits.detach().to(out_dtype),
+        "dx": leaves[0].grad.to(out_dtype),
+        "dw_gate": leaves[1].grad.to(out_dtype),
+        "dw_fc": leaves[2].grad.to(out_dtype),
+        "dw_proj": leaves[3].grad.to(out_dtype),
+    }
+
+
+def moe_dense_per_token(x, w_gate, w_fc, w_proj, top_k: int, activation=swiglu_unchunked_activation):
+    """Independent formulation used to pin ``moe_forward``: no sorting, no grouping.
+
+    y_t = sum_j softmax(top-k logits)_j * W_proj[e_j] act(W_fc[e_j] x_t)
+    """
+    logits = x @ w_gate.T
+    vals, sel = logits.topk(top_k, dim=-1) if top_k > 1 else logits.max(dim=-1, keepdim=True)
+    p = torch.softmax(vals.to(_acc_dtype(x)), dim=-1).type_as(x)
+    rows = []
+    for t in range(x.size(0)):
+        acc = torch.zeros(x.size(1), dtype=x.dtype)
+        for j in range(top_k):
+            e = int(sel[t, j])
+            acc = acc + p[t, j] * (w_proj[e] @ activation((w_fc[e] @ x[t]).unsqueeze(0)).squeeze(0))
+        rows.append(acc)
+    return torch.stack(rows), logits
+
+
+# =====================================================================================================
+# seeded inputs of the BASELINE configs
+# =====================================================================================================
+def _gen(seed: int) -> torch.Generator:
+    return torch.Generator().manual_seed(seed)
+
+
+def zipf_ids(shape, vocab_size: int, s: float, seed: int) -> torch.Tensor:
+    """int64 ids with P(rank r) ~ 1 / r^s, ranks mapped through a fixed random permutation of the vocabulary."""
+    g = _gen(seed)
+    ranks = torch.arange(1, vocab_size + 1, dtype=torch.float64)
+    cdf = torch.cumsum(ranks.pow(-s), 0)
+    cdf = cdf / cdf[-1]
+    u = torch.rand(math.prod(shape), generator=g, dtype=torch.float64)
+    rank = torch.searchsorted(cdf, u).clamp_(max=vocab_size - 1)
+    perm = torch.randperm(vocab_size, generator=g)
+    return perm[rank].reshape(shape)
+
+
+def moe_inputs(T: int, H: int, I: int, E: int, dtype, seed: int = 0):
+    """x ~ N(0,1); router and expert weights ~ N(0, 0.02); upstream grad ~ N(0,1).  SwiGLU experts: c_fc has
+    2I output rows.  Returns (x [T,H], w_gate [E,H], w_fc [E,2I,H], w_proj [E,H,I], dy [T,H]) in ``dtype``."""
+    g = _gen(seed)
+    x = torch.randn(T, H, generator=g)
+    w_gate = torch.randn(E, H, generator=g) * 0.02
+    w_fc = torch.randn(E, 2 * I, H, generator=g) * 0.02
+    w_proj = torch.randn(E, H, I, generator=g) * 0.02
+    dy = torch.randn(T, H, generator=g)
+    return tuple(t.to(dtype) for t in (x, w_gate, w_fc, w_proj, dy))
+
+
+def skewed_router(w_gate: torch.Tensor, x: torch.Tensor, s: float, seed: int, scale: float = 1.0):
+    """Per-expert logit bias b_e = -scale * s * ln(rank_e) (rank from a seeded permutation), i.e. the log of a
+    Zipf(s) popularity, folded into the bias-free router without changing a shape: feature 0 of every token
+    is set to 1 and b_e is written into w_gate[e, 0].  Returns (w_gate', x')."""
+    E = w_gate.size(0)
+    rank = torch.randperm(E, generator=_gen(seed)) + 1
+    bias = -scale * s * torch.log(rank.double())
+    w = w_gate.clone()
+    xx = x.clone()
+    xx[:, 0] = 1.0
+    w[:, 0] = bias.to(w.dtype)
+    return w, xx

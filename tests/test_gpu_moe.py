@@ -1,0 +1,224 @@
+"""GPU parity of the scattermoe path: grouped GEMM operators against brute-force oracle loops, then the whole
+layer (forward and every gradient) against the oracle restatement of MoE_Torch and against MoE_Torch itself."""
+
+import pytest
+import torch
+import torch.nn as nn
+
+from helpers import announce, assert_close, randn
+from oracle import cute_oracle as O
+
+
+pytestmark = pytest.mark.gpu
+
+
+def routing(T, k, E, seed, empty=()):
+    g = torch.Generator().manual_seed(seed)
+    allowed = torch.tensor([e for e in range(E) if e not in empty])
+    sel = torch.stack([allowed[torch.randperm(len(allowed), generator=g)[:k]] for _ in range(T)])
+    return O.moe_sort(sel, E)
+
+
+# ---- scatter2scatter ----------------------------------------------------------------------------------
+S2S_SHAPES = [
+    # T, k, E, K, N, empty experts
+    (16, 2, 4, 64, 128, ()),
+    (100, 2, 4, 72, 136, (1,)),
+    (300, 3, 7, 200, 40, (0, 6)),
+    (700, 2, 3, 256, 384, ()),
+    (64, 1, 2, 128, 128, ()),
+    (50, 2, 5, 30, 20, ()),  # contiguous sizes not multiples of 8: plain kernel
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("w_layout", ["k_contiguous", "n_contiguous"])
+@pytest.mark.parametrize("mode", ["gather_in", "scatter_out", "grouped_both"])
+@pytest.mark.parametrize("shape", S2S_SHAPES)
+def test_scatter2scatter(gpu, dtype, w_layout, mode, shape):
+    from cute_kernels.kernels.scattermoe import scatter2scatter
+
+    T, k, E, K, N, empty = shape
+    announce("scatter2scatter", dtype, w_layout, mode, shape)
+    s_e, s_idx, off = routing(T, k, E, 31, empty)
+    x_grouped = mode != "gather_in"
+    y_grouped = mode != "scatter_out"
+    fan_out = 1 if x_grouped else k
+    X = randn((T * k if x_grouped else T, K), dtype, 32)
+    if w_layout == "k_contiguous":
+        W = randn((E, N, K), dtype, 33, 0.05).permute(0, 2, 1)  # [E, K, N] view, K contiguous
+    else:
+        W = randn((E, K, N), dtype, 33, 0.05)
+    out = torch.full((T * k, N), float("nan"), dtype=dtype, device=gpu)
+    Wg = W.to(gpu) if w_layout == "n_contiguous" else W.permute(0, 2, 1).contiguous().to(gpu).permute(0, 2, 1)
+    assert Wg.stride() == W.stride()
+    scatter2scatter(X.to(gpu), Wg, s_e.to(gpu), s_idx.to(gpu), out, fan_out, x_grouped, y_grouped, off.to(gpu))
+    expected = O.scatter2scatter(X, W, s_idx, off, fan_out, x_grouped, y_grouped)
+    assert_close(out, expected, dtype, "out")
+    # without offsets (reference signature): recomputed from the sorted expert ids
+    out2 = torch.full_like(out, float("nan"))
+    scatter2scatter(X.to(gpu), Wg, s_e.to(gpu), s_idx.to(gpu), out2, fan_out, x_grouped, y_grouped)
+    assert torch.equal(out2, out)
+
+
+# ---- group_bwd_W --------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("dw_layout", ["k_contiguous", "n_contiguous"])
+@pytest.mark.parametrize("shape", [(16, 2, 4, 64, 128, ()), (100, 2, 4, 72, 136, (1,)), (300, 3, 7, 200, 40, (0, 6)),
+                                   (900, 2, 3, 256, 384, ()), (50, 2, 5, 30, 20, ())])
+def test_group_bwd_W(gpu, dtype, dw_layout, shape):
+    from cute_kernels.kernels.scattermoe import group_bwd_W
+
+    T, k, E, K, N, empty = shape
+    announce("group_bwd_W", dtype, dw_layout, shape)
+    _, _, off = routing(T, k, E, 41, empty)
+    X = randn((T * k, K), dtype, 42)
+    DY = randn((T * k, N), dtype, 43)
+    if dw_layout == "k_contiguous":
+        DW = torch.full((E, N, K), float("nan"), dtype=dtype, device=gpu).permute(0, 2, 1)
+    else:
+        DW = torch.full((E, K, N), float("nan"), dtype=dtype, device=gpu)
+    group_bwd_W(DY.to(gpu), X.to(gpu), off.to(gpu), DW, E)
+    expected = O.group_bwd_W(DY, X, off, E)
+    # the sums run over up to a few hundred rows of N(0,1) products: same tolerance, applied to O(10) values
+    assert_close(DW, expected, dtype, "DW")
+    for e in empty:
+        assert torch.count_nonzero(DW[e]) == 0
+
+
+# ---- group --------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("K", [8, 100, 4096, 30])
+@pytest.mark.parametrize("with_coeff", [False, True])
+def test_group(gpu, dtype, K, with_coeff):
+    from cute_kernels.kernels.scattermoe import group
+
+    announce("group", dtype, K, with_coeff)
+    T, k, E = 77, 2, 4
+    _, s_idx, _ = routing(T, k, E, 51)
+    A = randn((T, K), dtype, 52)
+    coeff = randn((T * k,), dtype, 53) if with_coeff else None
+    out = torch.empty(T * k, K, dtype=dtype, device=gpu)
+    group(A.to(gpu), s_idx.to(gpu), out, None if coeff is None else coeff.to(gpu), k)
+    expected = O.group(A, s_idx, coeff, k)
+    if with_coeff:
+        assert_close(out, expected, dtype, "out")
+    else:
+        assert torch.equal(out.cpu(), expected)
+
+
+# ---- the whole layer ----------------------------------------------------------------------------------
+def build_moe(cls, gpu, dtype, E, k, H, I, w_gate, w_fc, w_proj):
+    from cute_kernels import swiglu_unchunked_cute
+
+    moe = cls(num_experts=E, num_experts_per_tok=k, hidden_size=H, intermediate_size=I,
+              activation_function=swiglu_unchunked_cute, is_glu=True, add_bias=False, std=0.02)
+    moe = moe.to(device=gpu, dtype=dtype)
+    with torch.no_grad():
+        moe.gate.weight.copy_(w_gate)
+        moe.c_fc.weight.copy_(w_fc)
+        moe.c_proj.weight.copy_(w_proj)
+    return moe
+
+
+def run_moe(moe, x, dy, gpu):
+    xg = x.to(gpu).requires_grad_(True)
+    y, logits = moe(xg)
+    (y * dy.to(gpu)).sum().backward()
+    with torch.no_grad():
+        _, _, selected = moe._compute_routing_weights(xg.view(-1, moe.hidden_size))
+    return {
+        "y": y.detach(), "router_logits": logits.detach(), "dx": xg.grad,
+        "dw_gate": moe.gate.weight.grad, "dw_fc": moe.c_fc.weight.grad, "dw_proj": moe.c_proj.weight.grad,
+    }, selected.cpu()
+
+
+MOE_CASES = [
+    # name, T, H, I, E, k, skew
+    ("config1", 1024, 512, 1024, 8, 2, None),
+    ("odd_rows", 333, 256, 384, 6, 3, None),
+    ("skewed_empty", 2048, 256, 128, 32, 4, 2.0),
+    ("top1", 200, 128, 128, 4, 1, None),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case", MOE_CASES, ids=[c[0] for c in MOE_CASES])
+def test_moe_layer_against_oracle(gpu, dtype, case):
+    from cute_kernels import MoE_Triton
+
+    name, T, H, I, E, k, skew = case
+    announce("moe layer", dtype, case)
+    x, w_gate, w_fc, w_proj, dy = O.moe_inputs(T, H, I, E, dtype, seed=61)
+    if skew is not None:
+        w_gate, x = O.skewed_router(w_gate, x, 1.2, seed=62, scale=skew)
+    moe = build_moe(MoE_Triton, gpu, dtype, E, k, H, I, w_gate, w_fc, w_proj)
+    got, selected = run_moe(moe, x, dy, gpu)
+    if skew is not None:
+        assert (selected.flatten().bincount(minlength=E) == 0).any(), "case is meant to leave experts empty"
+
+    # the reference's torch implementation run in the storage dtype (fp32 accumulation inside each op)
+    expected = O.moe_forward_backward(x, w_gate, w_fc, w_proj, dy, k, compute_dtype=dtype, selected=selected)
+    for key in ("router_logits", "y", "dx", "dw_fc", "dw_proj", "dw_gate"):
+        assert_close(got[key], expected[key], dtype, f"{name}/{key}")
+
+    if dtype != torch.float32:
+        # against exact fp32 math on the same 16-bit inputs nearly every element is within tolerance too;
+        # the remainder is the rounding of 16-bit intermediates, which both implementations above share
+        exact = O.moe_forward_backward(x, w_gate, w_fc, w_proj, dy, k, compute_dtype=torch.float32, selected=selected)
+        tol = O.tolerance(dtype)
+        for key in ("y", "dx", "dw_fc", "dw_proj"):
+            assert O.fraction_outside(got[key], exact[key], **tol) < 2e-3, key
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("E,k", [(2, 2), (4, 2), (6, 4), (8, 4)])
+@pytest.mark.parametrize("is_glu", [True, False])
+def test_moe_like_the_reference_test(gpu, dtype, E, k, is_glu):
+    """The reference's own check (tests/kernels/scattermoe_test.py:14-139): one token, H=2048, I=8192,
+    nn.GLU or tanh-GELU, shared state dict, output and x.grad within its tolerances."""
+    from cute_kernels import MoE_Torch, MoE_Triton
+
+    announce("moe reference-style", dtype, E, k, is_glu)
+    torch.manual_seed(42)
+    act = nn.GLU() if is_glu else nn.GELU(approximate="tanh")
+    kwargs = dict(num_experts=E, num_experts_per_tok=k, hidden_size=2048, intermediate_size=8192,
+                  activation_function=act, is_glu=is_glu, add_bias=False, std=0.02)
+    with torch.device(gpu):
+        moe_custom = MoE_Triton(**kwargs).to(dtype=dtype)
+        moe_torch = MoE_Torch(**kwargs).to(dtype=dtype)
+    moe_torch.load_state_dict(moe_custom.state_dict())
+
+    x_torch = torch.randn(2048, device=gpu, dtype=dtype, requires_grad=True)
+    x_custom = x_torch.clone().detach().requires_grad_()
+    y_torch = moe_torch(x_torch)[0]
+    y_custom = moe_custom(x_custom)[0]
+    atol = {torch.float16: 4e-3, torch.bfloat16: 2e-2, torch.float32: 6e-3}[dtype]
+    torch.testing.assert_close(y_custom, y_torch, atol=atol, rtol=0)
+    y_torch.sum().backward()
+    y_custom.sum().backward()
+    atol = {torch.float16: 4e-3, torch.bfloat16: 4e-2, torch.float32: 6e-3}[dtype]
+    torch.testing.assert_close(x_custom.grad, x_torch.grad, atol=atol, rtol=0)
+
+
+def test_moe_3d_input_and_weight_grad_layout(gpu):
+    from cute_kernels import MoE_Triton, MoE_Torch
+
+    announce("moe 3d input")
+    dtype = torch.bfloat16
+    x, w_gate, w_fc, w_proj, dy = O.moe_inputs(6 * 50, 128, 64, 4, dtype, seed=71)
+    moe = build_moe(MoE_Triton, gpu, dtype, 4, 2, 128, 64, w_gate, w_fc, w_proj)
+    ref = build_moe(MoE_Torch, gpu, dtype, 4, 2, 128, 64, w_gate, w_fc, w_proj)
+    xg = x.view(6, 50, 128).to(gpu).requires_grad_(True)
+    xr = x.view(6, 50, 128).to(gpu).requires_grad_(True)
+    y, logits = moe(xg)
+    yr, logits_r = ref(xr)
+    assert y.shape == (6, 50, 128) and logits.shape == (300, 4)
+    (y * dy.view(6, 50, 128).to(gpu)).sum().backward()
+    (yr * dy.view(6, 50, 128).to(gpu)).sum().backward()
+    assert_close(y, yr, dtype, "y")
+    assert_close(xg.grad, xr.grad, dtype, "dx")
+    for name in ("c_fc", "c_proj"):
+        g, gr = getattr(moe, name).weight.grad, getattr(ref, name).weight.grad
+        assert g.shape == gr.shape and g.is_contiguous()
+        assert_close(g, gr, dtype, name)

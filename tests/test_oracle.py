@@ -1,0 +1,253 @@
+"""Pins the CPU oracle: every function of oracle/cute_oracle.py is checked against something it does not
+share code with - closed-form limits, autograd of the stock torch op in fp64, brute force on tiny inputs,
+algebraic invariants - chosen so that a dropped term, a wrong sign or a swapped operand fails."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import cute_oracle as O
+
+
+torch.manual_seed(0)
+F64 = torch.float64
+
+
+# ---- swiglu -------------------------------------------------------------------------------------------
+def test_swiglu_matches_autograd_fp64():
+    g = torch.randn(37, 19, dtype=F64, requires_grad=True)
+    u = torch.randn(37, 19, dtype=F64, requires_grad=True)
+    dy = torch.randn(37, 19, dtype=F64)
+    y = u * F.silu(g)
+    y.backward(dy)
+    assert torch.allclose(O.swiglu_forward(g.detach(), u.detach(), F64), y.detach(), rtol=1e-12, atol=1e-12)
+    dg, du = O.swiglu_backward(g.detach(), u.detach(), dy, F64)
+    assert torch.allclose(dg, g.grad, rtol=1e-11, atol=1e-12)
+    assert torch.allclose(du, u.grad, rtol=1e-11, atol=1e-12)
+
+
+def test_swiglu_known_values_and_limits():
+    g = torch.tensor([0.0, 100.0, -100.0, 1.0], dtype=F64)
+    u = torch.tensor([3.0, 2.0, 2.0, -1.5], dtype=F64)
+    y = O.swiglu_forward(g, u, F64)
+    # g = 0: silu = 0; g -> +inf: silu = g; g -> -inf: silu = 0; g = 1: 1 / (1 + e^-1)
+    expected = torch.tensor([0.0, 200.0, 0.0, -1.5 / (1 + math.exp(-1.0))], dtype=F64)
+    assert torch.allclose(y, expected, rtol=1e-12, atol=1e-30)
+    dg, du = O.swiglu_backward(g, u, torch.ones(4, dtype=F64), F64)
+    # g = 0: d silu / dg = 1/2, so dg = u / 2 and du = 0
+    assert dg[0].item() == pytest.approx(1.5) and du[0].item() == 0.0
+    assert dg[1].item() == pytest.approx(2.0) and du[1].item() == pytest.approx(100.0)
+    assert abs(dg[2].item()) < 1e-30 and abs(du[2].item()) < 1e-30
+    assert torch.isfinite(y).all() and torch.isfinite(dg).all()
+
+
+def test_swiglu_unchunked_halves():
+    x = torch.randn(5, 12, dtype=F64, requires_grad=True)
+    dy = torch.randn(5, 6, dtype=F64)
+    # the FIRST half is `up`, the SECOND half goes through silu
+    y = x[:, :6] * F.silu(x[:, 6:])
+    y.backward(dy)
+    assert torch.allclose(O.swiglu_unchunked_forward(x.detach(), F64), y.detach(), atol=1e-13)
+    assert torch.allclose(O.swiglu_unchunked_backward(x.detach(), dy, F64), x.grad, atol=1e-12)
+    # swapping the halves must change the answer (guards against a silently symmetric check)
+    swapped = torch.cat([x.detach()[:, 6:], x.detach()[:, :6]], dim=-1)
+    assert not torch.allclose(O.swiglu_unchunked_forward(swapped, F64), y.detach(), atol=1e-6)
+
+
+def test_swiglu_rounds_once():
+    g = torch.randn(4096).bfloat16()
+    u = torch.randn(4096).bfloat16()
+    exact = (u.double() * g.double() * torch.sigmoid(g.double()))
+    assert torch.equal(O.swiglu_forward(g, u), exact.float().bfloat16())
+
+
+# ---- rmsnorm ------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("has_weight", [True, False])
+def test_rmsnorm_matches_autograd_fp64(has_weight):
+    x = torch.randn(11, 24, dtype=F64, requires_grad=True)
+    w = torch.randn(24, dtype=F64, requires_grad=True) if has_weight else None
+    dy = torch.randn(11, 24, dtype=F64)
+    eps = 1e-5
+    y = F.rms_norm(x, (24,), weight=w, eps=eps)
+    y.backward(dy)
+    yo, rstd = O.rmsnorm_forward(x.detach(), None if w is None else w.detach(), eps, F64)
+    assert torch.allclose(yo, y.detach(), rtol=1e-12, atol=1e-13)
+    assert torch.allclose(rstd, torch.rsqrt(x.detach().pow(2).mean(-1) + eps), rtol=1e-13)
+    dx, dw = O.rmsnorm_backward(x.detach(), None if w is None else w.detach(), dy, eps, F64)
+    assert torch.allclose(dx, x.grad, rtol=1e-10, atol=1e-12)
+    if has_weight:
+        assert torch.allclose(dw, w.grad, rtol=1e-10, atol=1e-12)
+    else:
+        assert dw is None
+
+
+def test_rmsnorm_invariants():
+    x = torch.randn(7, 64, dtype=F64)
+    w = torch.randn(64, dtype=F64)
+    dy = torch.randn(7, 64, dtype=F64)
+    eps = 1e-6
+    # unit row: x = (1, ..., 1) -> rstd = 1/sqrt(1 + eps), y = w * rstd
+    ones = torch.ones(1, 64, dtype=F64)
+    y, rstd = O.rmsnorm_forward(ones, w, eps, F64)
+    assert rstd.item() == pytest.approx(1 / math.sqrt(1 + eps), rel=1e-14)
+    assert torch.allclose(y[0], w / math.sqrt(1 + eps), rtol=1e-14)
+    # scale invariance as eps -> 0
+    y1, _ = O.rmsnorm_forward(x, w, 0.0, F64)
+    y2, _ = O.rmsnorm_forward(3.7 * x, w, 0.0, F64)
+    assert torch.allclose(y1, y2, rtol=1e-12, atol=1e-13)
+    # sum_h dx_h x_h = rstd * sum_h(g_h x_h) * eps / (mean(x^2) + eps)
+    dx, _ = O.rmsnorm_backward(x, w, dy, eps, F64)
+    ms = x.pow(2).mean(-1)
+    rstd = torch.rsqrt(ms + eps)
+    lhs = (dx * x).sum(-1)
+    rhs = rstd * (dy * w * x).sum(-1) * eps / (ms + eps)
+    assert torch.allclose(lhs, rhs, rtol=1e-8, atol=1e-12)
+
+
+def test_rmsnorm_eps_default_and_1d():
+    assert O.resolve_eps(None, torch.bfloat16) == torch.finfo(torch.bfloat16).eps
+    assert O.resolve_eps(None, torch.float32) == torch.finfo(torch.float32).eps
+    x = torch.randn(33, dtype=F64)
+    y, rstd = O.rmsnorm_forward(x, None, 1e-5, F64)
+    assert y.shape == x.shape and rstd.shape == ()
+    assert torch.allclose(y, F.rms_norm(x, (33,), eps=1e-5), rtol=1e-12)
+
+
+# ---- embedding ----------------------------------------------------------------------------------------
+def test_embedding_forward_and_backward_against_one_hot():
+    V, H = 23, 8
+    ids = torch.randint(0, V, (3, 17))
+    ids[0, :5] = 4  # duplicates
+    w = torch.randn(V, H, dtype=F64, requires_grad=True)
+    dy = torch.randn(3, 17, H, dtype=F64)
+    out = F.embedding(ids, w)
+    out.backward(dy)
+    assert torch.equal(O.embedding_forward(ids, w.detach()), out.detach())
+    one_hot = F.one_hot(ids.reshape(-1), V).to(F64)
+    dense = one_hot.T @ dy.reshape(-1, H)
+    dw = O.embedding_backward(ids, dy, V, F64)
+    assert torch.allclose(dw, dense, rtol=1e-13, atol=1e-13)
+    assert torch.allclose(dw, w.grad, rtol=1e-13, atol=1e-13)
+    untouched = sorted(set(range(V)) - set(ids.reshape(-1).tolist()))
+    assert untouched and torch.count_nonzero(dw[untouched]) == 0
+    assert torch.allclose(dw.sum(0), dy.reshape(-1, H).sum(0), rtol=1e-12)
+
+
+def test_embedding_backward_accumulates_in_fp32():
+    # 4096 copies of one row in bf16: sequential bf16 accumulation stalls, fp32 accumulation does not
+    ids = torch.zeros(4096, dtype=torch.long)
+    dy = torch.full((4096, 4), 0.01).bfloat16()
+    dw = O.embedding_backward(ids, dy, 2)
+    assert dw[0, 0].item() == pytest.approx(4096 * dy[0, 0].item(), rel=4e-3)
+
+
+# ---- integer front end --------------------------------------------------------------------------------
+def test_contiguous_count_matches_bincount():
+    x = torch.randint(0, 72, (5000,))
+    c = O.contiguous_count(x, 72)
+    assert c.dtype == torch.int32 and torch.equal(c.long(), x.bincount(minlength=72))
+    assert torch.equal(O.contiguous_count(torch.tensor([3, 3, 0]), 5), torch.tensor([1, 0, 0, 2, 0], dtype=torch.int32))
+
+
+def test_moe_sort_is_the_stable_sort():
+    ids = torch.tensor([2, 0, 2, 1, 0, 2, 5])
+    s, idx, off = O.moe_sort(ids, 6)
+    assert s.tolist() == [0, 0, 1, 2, 2, 2, 5]
+    assert idx.tolist() == [1, 4, 3, 0, 2, 5, 6]  # ties keep input order
+    assert off.tolist() == [2, 3, 6, 6, 6, 7]  # inclusive ends; experts 3 and 4 are empty
+    # brute force on a random case: insertion into per-expert buckets in input order
+    ids = torch.randint(0, 9, (300,))
+    buckets = [[] for _ in range(9)]
+    for pos, e in enumerate(ids.tolist()):
+        buckets[e].append(pos)
+    s, idx, off = O.moe_sort(ids, 9)
+    assert idx.tolist() == [p for b in buckets for p in b]
+    assert s.tolist() == [e for e, b in enumerate(buckets) for _ in b]
+    assert off.tolist() == np.cumsum([len(b) for b in buckets]).tolist()
+
+
+# ---- grouped GEMM pieces ------------------------------------------------------------------------------
+def _routing(T, k, E, seed):
+    g = torch.Generator().manual_seed(seed)
+    sel = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)])
+    return O.moe_sort(sel, E)
+
+
+@pytest.mark.parametrize("x_grouped,y_grouped", [(False, True), (True, False), (True, True), (False, False)])
+def test_scatter2scatter_against_dense_per_expert(x_grouped, y_grouped):
+    T, k, E, K, N = 13, 2, 4, 6, 5
+    s_e, s_idx, off = _routing(T, k, E, 1)
+    W = torch.randn(E, K, N, dtype=F64)
+    fan_out = 1 if x_grouped else k
+    X = torch.randn(T * k if x_grouped else T, K, dtype=F64)
+    out = O.scatter2scatter(X, W, s_idx, off, fan_out, x_grouped, y_grouped, F64)
+    # dense statement: gather all rows into grouped order, multiply each expert's block, scatter back
+    src = torch.arange(T * k) if x_grouped else s_idx // fan_out
+    grouped = X[src]
+    dense = torch.cat([grouped[s_e == e] @ W[e] for e in range(E)])
+    expected = dense if y_grouped else torch.zeros_like(dense).index_copy(0, s_idx, dense)
+    assert torch.allclose(out, expected, rtol=1e-13, atol=1e-13)
+
+
+def test_group_bwd_w_and_group():
+    T, k, E, K, N = 11, 2, 5, 4, 3
+    s_e, s_idx, off = _routing(T, k, E, 2)
+    X = torch.randn(T * k, K, dtype=F64)
+    DY = torch.randn(T * k, N, dtype=F64)
+    DW = O.group_bwd_W(DY, X, off, E, F64)
+    for e in range(E):
+        rows = s_e == e
+        expected = sum((torch.outer(X[i], DY[i]) for i in torch.nonzero(rows).flatten()), torch.zeros(K, N, dtype=F64))
+        assert torch.allclose(DW[e], expected, rtol=1e-12, atol=1e-13)
+    # an expert without rows gets zeros
+    off2 = off.clone()
+    off2[1] = off2[0]
+    assert torch.count_nonzero(O.group_bwd_W(DY, X, off2, E, F64)[1]) == 0
+
+    A = torch.randn(T, K, dtype=F64)
+    coeff = torch.randn(T * k, dtype=F64)
+    out = O.group(A, s_idx, coeff, k)
+    for i in range(T * k):
+        j = int(s_idx[i])
+        assert torch.allclose(out[i], A[j // k] * coeff[j], rtol=1e-6)
+    assert torch.equal(O.group(A, s_idx, None, k), A[s_idx // k])
+
+
+# ---- the MoE layer ------------------------------------------------------------------------------------
+@pytest.mark.parametrize("top_k", [1, 2, 3])
+def test_moe_restatement_against_dense_per_token(top_k):
+    T, H, I, E = 9, 8, 6, 4
+    x, wg, wfc, wproj, dy = (t.double() for t in O.moe_inputs(T, H, I, E, torch.float32, seed=3))
+    wg = wg * 20  # spread the logits so that top-k is far from ties
+    res = O.moe_forward_backward(x, wg, wfc, wproj, dy, top_k, compute_dtype=F64)
+
+    leaves = [t.clone().requires_grad_(True) for t in (x, wg, wfc, wproj)]
+    y, logits = O.moe_dense_per_token(*leaves, top_k=top_k)
+    (y * dy).sum().backward()
+    assert torch.allclose(res["y"], y.detach(), rtol=1e-10, atol=1e-12)
+    assert torch.allclose(res["router_logits"], logits.detach(), rtol=1e-12, atol=1e-13)
+    for name, leaf in zip(("dx", "dw_gate", "dw_fc", "dw_proj"), leaves):
+        assert torch.allclose(res[name], leaf.grad, rtol=1e-9, atol=1e-11), name
+    if top_k == 1:
+        # one expert per token with weight softmax([v]) = 1: the router gets no gradient through the weights
+        assert torch.count_nonzero(res["dw_gate"]) == 0
+
+
+def test_moe_single_expert_is_a_plain_mlp():
+    T, H, I = 7, 8, 5
+    x, wg, wfc, wproj, dy = (t.double() for t in O.moe_inputs(T, H, I, 1, torch.float32, seed=4))
+    res = O.moe_forward_backward(x, wg, wfc, wproj, dy, 1, compute_dtype=F64)
+    h = x @ wfc[0].T
+    expected = (h[:, :I] * F.silu(h[:, I:])) @ wproj[0].T
+    assert torch.allclose(res["y"], expected, rtol=1e-11, atol=1e-13)
+
+
+def test_zipf_ids_and_skewed_router():
+    ids = O.zipf_ids((8, 4096), 128256, 1.1, seed=0)
+    assert ids.shape == (8, 4096) and ids.min() >= 0 and ids.max() < 128256
+    top = ids.flatten().bincount().max().item()
+    assert top > 0.02 * ids.numel()  # heavy duplicates
+    assert torch.equal(ids, O.zipf_ids((8, 4096), 128256, 1.1, seed=0))
