@@ -22,6 +22,16 @@ namespace ck {
 constexpr int kChunk = 32;      // slots of one run summed by one wave
 constexpr int kRowPacks = 8;    // packets per lane per column tile (tile = 64 lanes * 8 packets)
 
+// accumulator of the backward sums
+template <typename T>
+struct AccOf {
+    typedef float type;
+};
+template <>
+struct AccOf<F32> {
+    typedef double type;
+};
+
 template <bool I32>
 __device__ __forceinline__ int64_t load_tok(const void* p, int64_t i) {
     return I32 ? (int64_t) reinterpret_cast<const int32_t*>(p)[i] : reinterpret_cast<const int64_t*>(p)[i];
@@ -197,12 +207,14 @@ __global__ void __launch_bounds__(256)
 
     const int64_t packs = H / VEC;
     const int64_t tile = (int64_t)CK_WAVE * kRowPacks;
+    // fp32 tables sum in fp64 so that the result is the correctly rounded sum whatever the order
+    typedef typename AccOf<T>::type acc_t;
     for (int64_t p0 = 0; p0 < packs; p0 += tile) {
-        float acc[kRowPacks][VEC];
+        acc_t acc[kRowPacks][VEC];
 #pragma unroll
         for (int q = 0; q < kRowPacks; ++q)
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) acc[q][j] = 0.f;
+            for (int j = 0; j < VEC; ++j) acc[q][j] = 0;
         for (int r = 0; r < cnt; ++r) {
             const uint32_t pos = __shfl(my_pos, r, CK_WAVE);
             const P* src = reinterpret_cast<const P*>(dy + (int64_t)pos * H);
@@ -217,7 +229,7 @@ __global__ void __launch_bounds__(256)
                 const int64_t p = p0 + lane + (int64_t)q * CK_WAVE;
                 if (p < packs) {
 #pragma unroll
-                    for (int j = 0; j < VEC; ++j) acc[q][j] += T::up(v[q].v[j]);
+                    for (int j = 0; j < VEC; ++j) acc[q][j] += (acc_t)T::up(v[q].v[j]);
                 }
             }
         }
@@ -229,7 +241,7 @@ __global__ void __launch_bounds__(256)
                 if (p < packs) {
                     P o;
 #pragma unroll
-                    for (int j = 0; j < VEC; ++j) o.v[j] = T::down(acc[q][j]);
+                    for (int j = 0; j < VEC; ++j) o.v[j] = T::down((float)acc[q][j]);
                     nt_store(o, dst + p);
                 }
             }
@@ -245,11 +257,11 @@ __global__ void __launch_bounds__(256)
                     if (VEC % 4 == 0) {
 #pragma unroll
                         for (int j = 0; j + 3 < VEC; j += 4)
-                            *reinterpret_cast<float4*>(dst + p * VEC + j) =
-                                make_float4(acc[q][j], acc[q][j + 1], acc[q][j + 2], acc[q][j + 3]);
+                            *reinterpret_cast<float4*>(dst + p * VEC + j) = make_float4(
+                                (float)acc[q][j], (float)acc[q][j + 1], (float)acc[q][j + 2], (float)acc[q][j + 3]);
                     } else {
 #pragma unroll
-                        for (int j = 0; j < VEC; ++j) dst[p * VEC + j] = acc[q][j];
+                        for (int j = 0; j < VEC; ++j) dst[p * VEC + j] = (float)acc[q][j];
                     }
                 }
             }
@@ -269,13 +281,14 @@ __global__ void __launch_bounds__(256)
     if ((int64_t)id >= V) return;
     if ((int)run_head[i] != i) return;
     if (!(i + kChunk < n && skeys[i + kChunk] == id)) return;
+    typedef typename AccOf<T>::type acc_t;
     for (int64_t c = threadIdx.x; c < H; c += blockDim.x) {
-        float acc = 0.f;
+        acc_t acc = 0;
         for (int s = i; s < n && skeys[s] == id; s += kChunk) {
             const int64_t slot = 2 * (int64_t)(s / kChunk) + (s == i ? 1 : 0);
-            acc += partial[slot * H + c];
+            acc += (acc_t)partial[slot * H + c];
         }
-        dw[(int64_t)id * H + c] = T::down(acc);
+        dw[(int64_t)id * H + c] = T::down((float)acc);
     }
 }
 

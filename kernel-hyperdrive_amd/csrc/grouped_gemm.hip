@@ -10,7 +10,7 @@
 // staged through double-buffered LDS.  Tiles are scheduled per expert from expert_offsets, so a tile
 // never mixes rows of two experts (the reference lets a 128-row block straddle experts and repeats the
 // product once per expert present in it).  fp32, and shapes whose contiguous dimensions are not
-// multiples of 8 elements, go through a plain fp32-FMA kernel.
+// multiples of 8 elements, go through a plain kernel with exact (fp64) accumulation.
 #include "ck_device.h"
 
 namespace ck {
@@ -309,7 +309,8 @@ __global__ void __launch_bounds__(WM* WN* CK_WAVE) grouped_gemm_kernel(GemmParam
 }
 
 // ---- plain kernels (fp32 and irregular shapes) ---------------------------------------------------
-// One lane per output element; fp32 FMA in ascending k.
+// One lane per output element, fp64 accumulation: the fp32 path promises 1e-5, which an fp32 sum of a few
+// hundred O(1) terms does not keep in any order, so the sum is made exact and rounded once.
 template <typename T>
 __global__ void __launch_bounds__(256)
     s2s_plain_kernel(const typename T::storage_t* __restrict__ X, int64_t ldx, const typename T::storage_t* __restrict__ W,
@@ -330,9 +331,9 @@ __global__ void __launch_bounds__(256)
     const int64_t dst_row = y_grouped ? slot : row_idx[slot];
     const typename T::storage_t* x = X + src_row * ldx;
     const typename T::storage_t* w = W + (int64_t)lo * se + (int64_t)n * sn;
-    float acc = 0.f;
-    for (int k = 0; k < K; ++k) acc = fmaf(T::up(x[k]), T::up(w[(int64_t)k * sk]), acc);
-    out[dst_row * ldo + n] = T::down(acc);
+    double acc = 0.0;
+    for (int k = 0; k < K; ++k) acc = fma((double)T::up(x[k]), (double)T::up(w[(int64_t)k * sk]), acc);
+    out[dst_row * ldo + n] = T::down((float)acc);
 }
 
 template <typename T>
@@ -350,9 +351,10 @@ __global__ void __launch_bounds__(256)
     if (k >= K || n >= N) return;
     const int64_t begin = e == 0 ? 0 : offsets[e - 1];
     const int64_t end = offsets[e];
-    float acc = 0.f;
-    for (int64_t m = begin; m < end; ++m) acc = fmaf(T::up(X[m * ldx + k]), T::up(DY[m * lddy + n]), acc);
-    DW[(int64_t)e * se + (int64_t)k * sk + (int64_t)n * sn] = T::down(acc);
+    double acc = 0.0;
+    for (int64_t m = begin; m < end; ++m)
+        acc = fma((double)T::up(X[m * ldx + k]), (double)T::up(DY[m * lddy + n]), acc);
+    DW[(int64_t)e * se + (int64_t)k * sk + (int64_t)n * sn] = T::down((float)acc);
 }
 
 // ---- row gather ------------------------------------------------------------------------------

@@ -27,10 +27,11 @@ def embedding_forward_hip(input_ids: torch.Tensor, weight: torch.Tensor, output:
     _C.embedding_forward(input_ids, weight, output)
 
 
-@cute_op(f"{LIBRARY_NAME}::embedding_backward_hip", mutates_args={"weight_grad", "workspace"})
-def embedding_backward_hip(
-    input_ids: torch.Tensor, output_grad: torch.Tensor, weight_grad: torch.Tensor, workspace: torch.Tensor
-) -> None:
+@cute_op(f"{LIBRARY_NAME}::embedding_backward_hip", mutates_args={"weight_grad"})
+def embedding_backward_hip(input_ids: torch.Tensor, output_grad: torch.Tensor, weight_grad: torch.Tensor) -> None:
+    # sorted ids, run heads, row marks and fp32 partial rows; taken from torch's caching allocator
+    nbytes = _C.embedding_backward_workspace_size(input_ids.numel(), weight_grad.size(0), weight_grad.size(1))
+    workspace = torch.empty(max(nbytes, 256), device=weight_grad.device, dtype=torch.uint8)
     _C.embedding_backward(input_ids, output_grad, weight_grad, workspace)
 
 
@@ -60,9 +61,7 @@ def _backward(
     check_backend(kernel_backend)
     # every row is written by the kernels (selected rows once, the rest as zeros): no zero-fill first
     weight_grad = torch.empty_like(weight)
-    nbytes = _C.embedding_backward_workspace_size(input_ids.numel(), weight.size(0), weight.size(1))
-    workspace = torch.empty(max(nbytes, 256), device=weight.device, dtype=torch.uint8)
-    embedding_backward_hip(input_ids=input_ids, output_grad=output_grad, weight_grad=weight_grad, workspace=workspace)
+    embedding_backward_hip(input_ids=input_ids, output_grad=output_grad, weight_grad=weight_grad)
     return weight_grad
 
 

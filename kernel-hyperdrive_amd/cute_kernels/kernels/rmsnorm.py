@@ -32,7 +32,7 @@ def rmsnorm_forward_hip(
     _C.rmsnorm_forward(x, weight, output, rmsnorm_denominator, eps)
 
 
-@cute_op(f"{LIBRARY_NAME}::rmsnorm_backward_hip", mutates_args={"x_grad", "weight_grad", "workspace"})
+@cute_op(f"{LIBRARY_NAME}::rmsnorm_backward_hip", mutates_args={"x_grad", "weight_grad"})
 def rmsnorm_backward_hip(
     x: torch.Tensor,
     weight: torch.Tensor | None,
@@ -40,9 +40,15 @@ def rmsnorm_backward_hip(
     rmsnorm_denominator: torch.Tensor | None,
     x_grad: torch.Tensor,
     weight_grad: torch.Tensor | None,
-    workspace: torch.Tensor | None,
     eps: float,
 ) -> None:
+    workspace = None
+    if weight is not None:
+        # fp32 partial rows of the two-stage dweight reduction; taken from torch's caching allocator
+        hidden_size = x.size(-1)
+        num_rows = x.numel() // hidden_size if hidden_size > 0 else 0
+        nbytes = _C.rmsnorm_backward_workspace_size(num_rows, hidden_size, x.device)
+        workspace = torch.empty(max(nbytes, 16), device=x.device, dtype=torch.uint8)
     _C.rmsnorm_backward(x, weight, output_grad, rmsnorm_denominator, x_grad, weight_grad, workspace, eps)
 
 
@@ -89,15 +95,9 @@ def _backward(
     check_backend(kernel_backend)
     hidden_size = x.size(-1)
     _check_row_length(hidden_size)
-    num_rows = x.numel() // hidden_size if hidden_size > 0 else 0
 
     x_grad = torch.empty_like(x)
-    weight_grad = None
-    workspace = None
-    if weight is not None:
-        weight_grad = torch.empty_like(weight)
-        nbytes = _C.rmsnorm_backward_workspace_size(num_rows, hidden_size, x.device)
-        workspace = torch.empty(max(nbytes, 16), device=x.device, dtype=torch.uint8)
+    weight_grad = None if weight is None else torch.empty_like(weight)
     rmsnorm_backward_hip(
         x=x,
         weight=weight,
@@ -105,7 +105,6 @@ def _backward(
         rmsnorm_denominator=rmsnorm_denominator,
         x_grad=x_grad,
         weight_grad=weight_grad,
-        workspace=workspace,
         eps=eps,
     )
     return x_grad, weight_grad

@@ -22,3 +22,18 @@ def assert_close(actual, expected, dtype, what=""):
 def announce(*parts):
     """Name the case before the GPU step runs, flushed, so a lost box still tells which case it was."""
     print("[case]", *parts, flush=True)
+
+
+def acc_dtype(dtype):
+    """Accumulation dtype of the expectation: the correctly rounded result.  fp32 accumulation is exact
+    enough for 16-bit data; fp32 data needs fp64, because an fp32 sum of a few hundred O(1) terms is itself
+    off by more than the 1e-5 tolerance, in any order."""
+    return torch.float64 if dtype == torch.float32 else torch.float32
+
+
+def assert_norm_close(actual, expected, rel, what=""):
+    """||actual - expected||_F <= rel * ||expected||_F, for quantities that are long sums of O(1) terms."""
+    a, e = actual.detach().double().cpu(), expected.detach().double().cpu()
+    err = (a - e).norm().item()
+    ref = e.norm().item()
+    assert err <= rel * max(ref, 1e-30), f"{what}: relative Frobenius error {err / max(ref, 1e-30):.3e} > {rel:.1e}"

@@ -4,7 +4,7 @@ cute_kernels functions (autograd.Function -> cute op -> C ABI -> HIP kernel)."""
 import pytest
 import torch
 
-from helpers import DTYPES, announce, assert_close, randn
+from helpers import DTYPES, acc_dtype, announce, assert_close, randn
 from oracle import cute_oracle as O
 
 
@@ -151,7 +151,7 @@ def test_embedding(gpu, dtype, ids_shape, table):
     out.backward(dy.to(gpu))
     assert out.shape == ids_shape + (H,)
     assert torch.equal(out.cpu(), O.embedding_forward(ids, w)), "forward must be a bit-exact copy"
-    assert_close(wg.grad, O.embedding_backward(ids, dy, V), dtype, "weight_grad")
+    assert_close(wg.grad, O.embedding_backward(ids, dy, V, acc_dtype(dtype)), dtype, "weight_grad")
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
@@ -175,7 +175,7 @@ def test_embedding_duplicates(gpu, dtype, case):
     out = embedding_cute(ids.to(gpu), wg)
     out.backward(dy.to(gpu))
     assert torch.equal(out.cpu(), O.embedding_forward(ids, w))
-    expected = O.embedding_backward(ids, dy, V)
+    expected = O.embedding_backward(ids, dy, V, acc_dtype(dtype))
     assert_close(wg.grad, expected, dtype, "weight_grad")
     touched = torch.zeros(V, dtype=torch.bool)
     touched[ids.reshape(-1).long()] = True
