@@ -1,0 +1,271 @@
+"""Benchmark of the hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One step = one forward + backward of the Mixtral-shape scattermoe layer (BASELINE.json configs[3]: T=8192,
+H=4096, I=14336, E=8 SwiGLU experts, top-2, bf16) on synthetic, seeded data that is resident in HBM before the
+timed region.  Prints ONE JSON line:
+  value        TFLOP/s of the whole step, counting 18*M*H*I flops (M = T*k routed rows); router, top-k, sort,
+               activation and gate mixing are inside the timed region but not in the flop count
+  roofline     the grouped GEMM (6 launches per step: forward, dX and dW of c_fc and c_proj), timed inside the
+               timed region with GPU events on the launch stream, against the 2.5 PFLOP/s dense bf16 MFMA peak
+  cpu_baseline the oracle's torch restatement of the reference layer on the host cores, on a bounded sample
+  extras       HBM GB/s of SwiGLU, RMSNorm and embedding at their BASELINE shapes (buffers rotated so that the
+               256 MB last-level cache cannot serve them)
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _path in (ROOT, os.path.join(ROOT, "kernel-hyperdrive_amd")):
+    if _path not in sys.path:
+        sys.path.insert(0, _path)
+
+import torch  # noqa: E402
+
+BF16_MFMA_PEAK_TFLOPS = 2500.0
+HBM_PEAK_GBS = 8000.0
+
+
+def parse_args():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=10)
+    p.add_argument("--warmup", type=int, default=3)
+    p.add_argument("--no-extras", action="store_true", help="skip the SwiGLU / RMSNorm / embedding bandwidth figures")
+    p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    p.add_argument("--tokens", type=int, default=8192, help="T of the MoE workload (default: the BASELINE shape)")
+    return p.parse_args()
+
+
+# ---- the MoE step ---------------------------------------------------------------------------------------
+def build_moe(device, T, H, I, E, k, dtype):
+    import cute_kernels as ck
+
+    g = torch.Generator(device=device).manual_seed(0)
+    moe = ck.MoE_Triton(num_experts=E, num_experts_per_tok=k, hidden_size=H, intermediate_size=I,
+                        activation_function=ck.swiglu_unchunked_cute, is_glu=True, add_bias=False, std=0.02)
+    moe = moe.to(device=device, dtype=dtype)
+    with torch.no_grad():
+        for prm in moe.parameters():
+            prm.copy_(torch.randn(prm.shape, generator=g, device=device, dtype=torch.float32).mul_(0.02))
+    x = torch.randn(T, H, generator=g, device=device, dtype=torch.float32).to(dtype).requires_grad_(True)
+    dy = torch.randn(T, H, generator=g, device=device, dtype=torch.float32).to(dtype)
+    return moe, x, dy
+
+
+def moe_step(moe, x, dy):
+    for prm in moe.parameters():
+        prm.grad = None
+    x.grad = None
+    y, _ = moe(x)
+    y.backward(dy)
+
+
+def bench_moe(device, args):
+    from cute_kernels import _C
+
+    T, H, I, E, k = args.tokens, 4096, 14336, 8, 2
+    dtype = torch.bfloat16
+    moe, x, dy = build_moe(device, T, H, I, E, k, dtype)
+    for _ in range(args.warmup):
+        moe_step(moe, x, dy)
+    torch.cuda.synchronize()
+
+    trace = []
+    _C.set_launch_trace(trace)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        moe_step(moe, x, dy)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    _C.set_launch_trace(None)
+
+    M = T * k
+    flop_per_step = 18.0 * M * H * I
+    ms_per_step = elapsed / args.steps * 1e3
+    gemm_ms = sum(s.elapsed_time(e) for _, _, s, e in trace)
+    gemm_flop = sum(f for _, f, _, _ in trace)
+    launches = len(trace)
+    per_kind = {}
+    for name, f, s, e in trace:
+        d = per_kind.setdefault(name, [0.0, 0.0, 0])
+        d[0] += f
+        d[1] += s.elapsed_time(e)
+        d[2] += 1
+    achieved = gemm_flop / (gemm_ms * 1e-3) / 1e12
+    roofline = {
+        "bound": "mfma",
+        "kernel": "grouped_gemm_kernel (scatter2scatter + group_bwd_W launches)",
+        "achieved": round(achieved, 2),
+        "peak": BF16_MFMA_PEAK_TFLOPS,
+        "unit": "TFLOP/s",
+        "frac": round(achieved / BF16_MFMA_PEAK_TFLOPS, 4),
+        "traffic": None,
+        "launches_per_step": launches // args.steps,
+        "avg_launch_ms": round(gemm_ms / max(launches, 1), 4),
+        "gemm_ms_per_step": round(gemm_ms / args.steps, 3),
+        "per_entry_point_tflops": {n: round(d[0] / (d[1] * 1e-3) / 1e12, 2) for n, d in per_kind.items()},
+    }
+    result = {
+        "value": round(flop_per_step / (ms_per_step * 1e-3) / 1e12, 2),
+        "ms_per_step": round(ms_per_step, 3),
+        "frac_of_mfma_peak": round(flop_per_step / (ms_per_step * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS, 4),
+    }
+    config = {"workload": f"Mixtral-shape scattermoe fwd+bwd (BASELINE configs[3]): T={T} H={H} I={I} E={E} top-{k} SwiGLU bf16",
+              "routed_rows": M, "flop_per_step": flop_per_step}
+    del moe, x, dy
+    torch.cuda.empty_cache()
+    return result, roofline, config
+
+
+# ---- HBM-bound ops ----------------------------------------------------------------------------------------
+def _time_rotating(fn, sets, iters=20, warmup=3):
+    """Median-free simple timing: `fn(i)` uses buffer set i % sets; returns ms per call."""
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(iters):
+        fn(i)
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / iters
+
+
+def bench_extras(device):
+    from cute_kernels import KernelBackend
+    from cute_kernels.kernels import embedding as EM
+    from cute_kernels.kernels import rmsnorm as RN
+    from cute_kernels.kernels import swiglu as SW
+    from oracle import cute_oracle as O
+
+    dtype = torch.bfloat16
+    hip = KernelBackend.hip
+    out = {}
+
+    def gbs(nbytes, ms):
+        v = nbytes / (ms * 1e-3) / 1e9
+        return {"GB/s": round(v, 1), "frac_of_hbm_peak": round(v / HBM_PEAK_GBS, 4), "ms": round(ms, 4)}
+
+    # RMSNorm, BASELINE configs[1]: x [16384, 4096]; 4 buffer sets of 134 MB
+    B, H = 16384, 4096
+    sets = 4
+    xs = [torch.randn(B, H, device=device, dtype=dtype) for _ in range(sets)]
+    dys = [torch.randn(B, H, device=device, dtype=dtype) for _ in range(sets)]
+    w = (torch.randn(H, device=device) * 0.1 + 1).to(dtype)
+    rstd = RN._forward(x=xs[0], weight=w, eps=1e-5, memory_efficient=False, kernel_backend=hip, BLOCK_SIZE_B=1, BLOCK_SIZE_H=H)[1]
+    ms = _time_rotating(lambda i: RN._forward(x=xs[i % sets], weight=w, eps=1e-5, memory_efficient=False,
+                                              kernel_backend=hip, BLOCK_SIZE_B=1, BLOCK_SIZE_H=H), sets)
+    out["rmsnorm_fwd"] = gbs(2 * B * H * 2 + H * 2 + B * 4, ms)
+    ms = _time_rotating(lambda i: RN._backward(x=xs[i % sets], weight=w, eps=1e-5, rmsnorm_denominator=rstd,
+                                               output_grad=dys[i % sets], kernel_backend=hip, BLOCK_SIZE_B=1, BLOCK_SIZE_H=H), sets)
+    out["rmsnorm_bwd"] = gbs(3 * B * H * 2 + 2 * H * 2 + B * 4, ms)
+    del xs, dys
+
+    # SwiGLU, BASELINE configs[2]: gate, up [16384, 14336]; 470 MB per tensor already exceeds the cache
+    N = 16384 * 14336
+    gate = torch.randn(N, device=device, dtype=dtype)
+    up = torch.randn(N, device=device, dtype=dtype)
+    dy = torch.randn(N, device=device, dtype=dtype)
+    ms = _time_rotating(lambda i: SW._forward(gate=gate, up=up, kernel_backend=hip, BLOCK_SIZE=256), 1)
+    out["swiglu_fwd"] = gbs(3 * N * 2, ms)
+    ms = _time_rotating(lambda i: SW._backward(gate=gate, up=up, output_grad=dy, kernel_backend=hip, BLOCK_SIZE=256), 1)
+    out["swiglu_bwd"] = gbs(5 * N * 2, ms)
+    del gate, up, dy
+    torch.cuda.empty_cache()
+
+    # Embedding, BASELINE configs[2]: table [128256, 4096], ids [8, 4096]; (a) uniform ids, (b) Zipf(1.1) ids
+    V, H = 128256, 4096
+    table = (torch.randn(V, H, device=device) * 0.02).to(dtype)
+    n = 8 * 4096
+    dys = [torch.randn(8, 4096, H, device=device, dtype=dtype) for _ in range(2)]
+    for label, ids in (("uniform", torch.randint(0, V, (8, 4096), generator=torch.Generator().manual_seed(0))),
+                       ("zipf", O.zipf_ids((8, 4096), V, 1.1, seed=0))):
+        ids = ids.to(device)
+        ms = _time_rotating(lambda i: EM._forward(input_ids=ids, weight=table, kernel_backend=hip, BLOCK_SIZE_B=4, BLOCK_SIZE_H=512), 1)
+        out[f"embedding_fwd_{label}"] = gbs(2 * n * H * 2 + 8 * n, ms)
+        ms = _time_rotating(lambda i: EM._backward(input_ids=ids, weight=table, output_grad=dys[i % 2], kernel_backend=hip,
+                                                   BLOCK_SIZE_B=4, BLOCK_SIZE_H=512), 2, iters=10)
+        out[f"embedding_bwd_{label}"] = gbs(n * H * 2 + V * H * 2 + 8 * n, ms)
+    del table, dys
+    torch.cuda.empty_cache()
+    return out
+
+
+# ---- CPU baseline -----------------------------------------------------------------------------------------
+def bench_cpu():
+    """The oracle's restatement of the reference torch layer, fp32, on the host cores: the Mixtral shape with
+    T=512 of the 8192 tokens (same H, I, E, k).  About 1.1e12 flop per step."""
+    from oracle import cute_oracle as O
+
+    threads = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(threads)
+    T, H, I, E, k = 512, 4096, 14336, 8, 2
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(T, H, generator=g)
+    w_gate = torch.randn(E, H, generator=g) * 0.02
+    w_fc = torch.empty(E, 2 * I, H).normal_(0, 0.02, generator=g)
+    w_proj = torch.empty(E, H, I).normal_(0, 0.02, generator=g)
+    dy = torch.randn(T, H, generator=g)
+    flop = 18.0 * T * k * H * I
+    O.moe_forward_backward(x, w_gate, w_fc, w_proj, dy, k)  # warm-up
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 5 and time.perf_counter() - t_start < 20.0:
+        t0 = time.perf_counter()
+        O.moe_forward_backward(x, w_gate, w_fc, w_proj, dy, k)
+        times.append(time.perf_counter() - t0)
+    best = sorted(times)[len(times) // 2]
+    return {
+        "value": round(flop / best / 1e12, 4),
+        "unit": "TFLOP/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"Mixtral shape with T={T} of 8192 tokens (H={H} I={I} E={E} top-{k}), fp32 fwd+bwd, "
+                  f"median of {len(times)} runs, {best * 1e3:.0f} ms each; torch {torch.__version__}",
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: this build has no multi-GPU path (asked for --gpus {args.gpus})", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    device = torch.device("cuda", 0)
+    result, roofline, config = bench_moe(device, args)
+    line = {
+        "metric": "scattermoe_fwd_bwd_tflops",
+        "value": result["value"],
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": result["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": config,
+        "frac_of_mfma_peak": result["frac_of_mfma_peak"],
+        "roofline": roofline,
+    }
+    if not args.no_extras:
+        line["extras"] = bench_extras(device)
+    if not args.no_cpu:
+        line["cpu_baseline"] = bench_cpu()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -136,6 +136,36 @@ class _Launch:
         return False
 
 
+# Optional per-launch timing: while a list is installed here, the grouped-GEMM entry points bracket their
+# launch with GPU events recorded on the launch stream and append (name, flop, start, end) to it.
+_launch_trace: list | None = None
+
+
+def set_launch_trace(trace: list | None) -> None:
+    global _launch_trace
+    _launch_trace = trace
+
+
+class _Timed:
+    __slots__ = ("name", "flop", "start")
+
+    def __init__(self, name: str, flop: float):
+        self.name, self.flop = name, flop
+
+    def __enter__(self):
+        if _launch_trace is not None:
+            self.start = torch.cuda.Event(enable_timing=True)
+            self.start.record()
+        return self
+
+    def __exit__(self, *exc):
+        if _launch_trace is not None:
+            end = torch.cuda.Event(enable_timing=True)
+            end.record()
+            _launch_trace.append((self.name, self.flop, self.start, end))
+        return False
+
+
 def _check(status: int, name: str) -> None:
     if status != 0:
         text = load_library().ck_status_string(status).decode()
@@ -297,7 +327,8 @@ def scatter2scatter(X, W, sorted_scattered_idxs, expert_offsets, out, fan_out: i
     lib = load_library()
     if X.stride(1) != 1 or out.stride(1) != 1:
         raise ValueError("scatter2scatter needs unit column stride for X and out")
-    with _Launch(X, W, sorted_scattered_idxs, expert_offsets, out) as L:
+    flop = 2.0 * out.size(0) * X.size(1) * out.size(1)
+    with _Launch(X, W, sorted_scattered_idxs, expert_offsets, out) as L, _Timed("scatter2scatter", flop):
         _check(
             lib.ck_scatter2scatter(_ptr(X), X.stride(0), _ptr(W), W.stride(0), W.stride(1), W.stride(2),
                                    _ptr(sorted_scattered_idxs), _ptr(expert_offsets), _ptr(out), out.stride(0),
@@ -311,7 +342,8 @@ def group_bwd_W(DY, X, expert_offsets, DW, E: int) -> None:
     lib = load_library()
     if X.stride(1) != 1 or DY.stride(1) != 1:
         raise ValueError("group_bwd_W needs unit column stride for X and DY")
-    with _Launch(DY, X, expert_offsets, DW) as L:
+    flop = 2.0 * X.size(0) * X.size(1) * DY.size(1)
+    with _Launch(DY, X, expert_offsets, DW) as L, _Timed("group_bwd_W", flop):
         _check(
             lib.ck_group_bwd_W(_ptr(DY), DY.stride(0), _ptr(X), X.stride(0), _ptr(expert_offsets), _ptr(DW),
                                DW.stride(0), DW.stride(1), DW.stride(2), X.size(0), X.size(1), DY.size(1), E,
