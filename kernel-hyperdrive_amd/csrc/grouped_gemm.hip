@@ -106,23 +106,67 @@ __device__ __forceinline__ bool logical_tile(int m_tiles, int n_tiles, int& mt, 
     return true;
 }
 
+// Tile shape of the MFMA kernel.  BM x BN outputs per workgroup, BK of the contraction per step,
+// WM x WN wavefronts each owning a (BM/WM) x (BN/WN) block of 32x32 MFMA tiles.
+template <int BM_, int BN_, int BK_, int WM_, int WN_>
+struct Tile {
+    static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
+    static constexpr int THREADS = WM * WN * CK_WAVE;
+    static constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+};
+
+typedef short v4i16_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) v4i16_t* lds_v4i16_ptr;
+
+// Operand tile in LDS.
+//   KC = true : [ROWS][BK + 8]  (contraction contiguous); an MFMA fragment is one 16-byte read per lane; the
+//               8-element pad makes consecutive rows fall 36 dwords apart, which spreads 16 lanes over all banks
+//   KC = false: [BK][ROWS + 32] (output dimension contiguous); fragments come from two transposing reads
+//               (ds_read_b64_tr_b16): inside each group of 16 lanes, 4 lanes fetch one contraction row of 16
+//               elements and lane i receives element i of each of the 4 rows
+template <typename S, int ROWS, int BK, bool KC>
+struct OperandTile {
+    static constexpr int LD = KC ? BK + 8 : ROWS + 32;
+    static constexpr int LINES = KC ? ROWS : BK;
+    static constexpr int ELEMS = LINES * LD;
+    static constexpr int CHUNKS_PER_LINE = (KC ? BK : ROWS) / 8;
+
+    // fragment for the 32 rows starting at `r0`, contraction offset `kk` (multiple of 16)
+    template <typename frag_t>
+    static __device__ __forceinline__ frag_t fragment(const S* tile, int r0, int kk, int lane) {
+        if (KC) {
+            return *reinterpret_cast<const frag_t*>(tile + (r0 + lane % 32) * LD + kk + (lane / 32) * 8);
+        } else {
+            const int g = lane / 16, i = lane % 16;
+            const S* p = tile + (kk + (g / 2) * 8 + i / 4) * LD + r0 + (g % 2) * 16 + (i % 4) * 4;
+            union {
+                v4i16_t h[2];
+                frag_t f;
+            } u;
+            u.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(p));
+            u.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(p + 4 * LD));
+            return u.f;
+        }
+    }
+};
+
 // GROUP_K = false ("S2S"): C[row map] = A[row map] (k contiguous) x B, B k-contiguous (B_KC) or n-contiguous.
 // GROUP_K = true  ("XTY"): C[e] = P_e^T Q_e, both operands contiguous along the output dimension; the
 //                          contraction runs over the expert's rows.
-template <typename T, int BM, int BN, int BK, int WM, int WN, bool B_KC, bool GROUP_K>
-__global__ void __launch_bounds__(WM* WN* CK_WAVE) grouped_gemm_kernel(GemmParams p) {
+template <typename T, typename TL, bool B_KC, bool GROUP_K>
+__global__ void __launch_bounds__(TL::THREADS) grouped_gemm_kernel(GemmParams p) {
     typedef typename T::storage_t S;
     typedef typename Mma<T>::frag_t frag_t;
-    constexpr int THREADS = WM * WN * CK_WAVE;
-    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
-    constexpr int PAD = 8;
+    constexpr int BM = TL::BM, BN = TL::BN, BK = TL::BK, WM = TL::WM, WN = TL::WN;
+    constexpr int THREADS = TL::THREADS, TM = TL::TM, TN = TL::TN;
     constexpr bool A_KC = !GROUP_K;
     constexpr bool B_KCC = GROUP_K ? false : B_KC;
-    // LDS tiles: k-contiguous operands as [rows][BK + PAD], others as [BK][rows + PAD]
-    constexpr int A_ROWS = A_KC ? BM : BK, A_COLS = (A_KC ? BK : BM) + PAD;
-    constexpr int B_ROWS = B_KCC ? BN : BK, B_COLS = (B_KCC ? BK : BN) + PAD;
-    __shared__ __attribute__((aligned(16))) S As[2][A_ROWS][A_COLS];
-    __shared__ __attribute__((aligned(16))) S Bs[2][B_ROWS][B_COLS];
+    typedef OperandTile<S, BM, BK, A_KC> ATile;
+    typedef OperandTile<S, BN, BK, B_KCC> BTile;
+    constexpr int C_LD = BN + 8;  // staged output tile [BM][BN + 8]
+    constexpr int STAGE_ELEMS = ATile::ELEMS + BTile::ELEMS;
+    constexpr int LDS_ELEMS = (2 * STAGE_ELEMS > BM * C_LD) ? 2 * STAGE_ELEMS : BM * C_LD;
+    __shared__ __attribute__((aligned(16))) S lds[LDS_ELEMS];
     __shared__ int sh_info[4];
 
     int mt, nt;
@@ -134,7 +178,7 @@ __global__ void __launch_bounds__(WM* WN* CK_WAVE) grouped_gemm_kernel(GemmParam
     const int wm = wave / WN, wn = wave % WN;
 
     // ---- which rows / which contraction range ------------------------------------------------
-    int expert, row_start, rows_valid;  // S2S: rows of this tile.  XTY: contraction rows of the expert
+    int expert, row_start, rows_valid;  // S2S: rows of this tile.  XTY: output rows of this tile
     int k_begin, k_end;                 // contraction range
     int i_base;                         // XTY: first output row of this tile
     if (!GROUP_K) {
@@ -158,18 +202,16 @@ __global__ void __launch_bounds__(WM* WN* CK_WAVE) grouped_gemm_kernel(GemmParam
     const int n_base = nt * BN;
 
     // ---- global -> register staging ------------------------------------------------------------
-    constexpr int A_CHUNKS_PER_ROW = (A_KC ? BK : BM) / 8;
-    constexpr int B_CHUNKS_PER_ROW = (B_KCC ? BK : BN) / 8;
-    constexpr int A_CH = A_ROWS * A_CHUNKS_PER_ROW / THREADS;
-    constexpr int B_CH = B_ROWS * B_CHUNKS_PER_ROW / THREADS;
-    static_assert(A_ROWS * A_CHUNKS_PER_ROW % THREADS == 0 && B_ROWS * B_CHUNKS_PER_ROW % THREADS == 0, "tile/threads");
+    constexpr int A_CH = ATile::LINES * ATile::CHUNKS_PER_LINE / THREADS;
+    constexpr int B_CH = BTile::LINES * BTile::CHUNKS_PER_LINE / THREADS;
+    static_assert(ATile::LINES * ATile::CHUNKS_PER_LINE % THREADS == 0, "A tile / threads");
+    static_assert(BTile::LINES * BTile::CHUNKS_PER_LINE % THREADS == 0, "B tile / threads");
 
     const S* a_src[A_CH];  // S2S: row base pointers (nullptr = row outside the tile)
     if (A_KC) {
 #pragma unroll
         for (int i = 0; i < A_CH; ++i) {
-            const int c = tid + i * THREADS;
-            const int r = c / A_CHUNKS_PER_ROW;
+            const int r = (tid + i * THREADS) / ATile::CHUNKS_PER_LINE;
             a_src[i] = nullptr;
             if (r < rows_valid) {
                 const int64_t slot = row_start + r;
@@ -178,6 +220,7 @@ __global__ void __launch_bounds__(WM* WN* CK_WAVE) grouped_gemm_kernel(GemmParam
             }
         }
     }
+    const S* Abase = reinterpret_cast<const S*>(p.A);
     const S* Bbase = reinterpret_cast<const S*>(p.B) + (GROUP_K ? 0 : (int64_t)expert * p.b_stride_e);
 
     u32x4_t a_reg[A_CH], b_reg[B_CH];
@@ -185,26 +228,24 @@ __global__ void __launch_bounds__(WM* WN* CK_WAVE) grouped_gemm_kernel(GemmParam
 #pragma unroll
         for (int i = 0; i < A_CH; ++i) {
             const int c = tid + i * THREADS;
-            const int r = c / A_CHUNKS_PER_ROW;
-            const int cc = (c % A_CHUNKS_PER_ROW) * 8;
+            const int r = c / ATile::CHUNKS_PER_LINE;
+            const int cc = (c % ATile::CHUNKS_PER_LINE) * 8;
             u32x4_t v = {0u, 0u, 0u, 0u};
             if (A_KC) {
                 // row r of the tile, k = k0 + cc .. +7
-                if (a_src[i] != nullptr && k0 + cc < k_end)
-                    v = *reinterpret_cast<const u32x4_t*>(a_src[i] + k0 + cc);
+                if (a_src[i] != nullptr && k0 + cc < k_end) v = *reinterpret_cast<const u32x4_t*>(a_src[i] + k0 + cc);
             } else {
                 // contraction row k0 + r, output rows i_base + cc .. +7
                 if (k0 + r < k_end && i_base + cc < p.K)
-                    v = *reinterpret_cast<const u32x4_t*>(reinterpret_cast<const S*>(p.A) + (int64_t)(k0 + r) * p.lda +
-                                                          i_base + cc);
+                    v = *reinterpret_cast<const u32x4_t*>(Abase + (int64_t)(k0 + r) * p.lda + i_base + cc);
             }
             a_reg[i] = v;
         }
 #pragma unroll
         for (int i = 0; i < B_CH; ++i) {
             const int c = tid + i * THREADS;
-            const int r = c / B_CHUNKS_PER_ROW;
-            const int cc = (c % B_CHUNKS_PER_ROW) * 8;
+            const int r = c / BTile::CHUNKS_PER_LINE;
+            const int cc = (c % BTile::CHUNKS_PER_LINE) * 8;
             u32x4_t v = {0u, 0u, 0u, 0u};
             if (B_KCC) {
                 // column n_base + r, k = k0 + cc .. +7
@@ -219,15 +260,19 @@ __global__ void __launch_bounds__(WM* WN* CK_WAVE) grouped_gemm_kernel(GemmParam
         }
     };
     auto store_tiles = [&](int buf) {
+        S* At = lds + buf * STAGE_ELEMS;
+        S* Bt = At + ATile::ELEMS;
 #pragma unroll
         for (int i = 0; i < A_CH; ++i) {
             const int c = tid + i * THREADS;
-            *reinterpret_cast<u32x4_t*>(&As[buf][c / A_CHUNKS_PER_ROW][(c % A_CHUNKS_PER_ROW) * 8]) = a_reg[i];
+            *reinterpret_cast<u32x4_t*>(At + (c / ATile::CHUNKS_PER_LINE) * ATile::LD + (c % ATile::CHUNKS_PER_LINE) * 8) =
+                a_reg[i];
         }
 #pragma unroll
         for (int i = 0; i < B_CH; ++i) {
             const int c = tid + i * THREADS;
-            *reinterpret_cast<u32x4_t*>(&Bs[buf][c / B_CHUNKS_PER_ROW][(c % B_CHUNKS_PER_ROW) * 8]) = b_reg[i];
+            *reinterpret_cast<u32x4_t*>(Bt + (c / BTile::CHUNKS_PER_LINE) * BTile::LD + (c % BTile::CHUNKS_PER_LINE) * 8) =
+                b_reg[i];
         }
     };
 
@@ -239,9 +284,6 @@ __global__ void __launch_bounds__(WM* WN* CK_WAVE) grouped_gemm_kernel(GemmParam
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    const int frag_row = lane % 32;  // row (A) / column (B) inside a 32-wide MFMA tile
-    const int frag_k = (lane / 32) * 8;
-
     const int k_tiles = (k_end - k_begin + BK - 1) / BK;
     if (k_tiles > 0) {
         load_tiles(k_begin);
@@ -251,29 +293,17 @@ __global__ void __launch_bounds__(WM* WN* CK_WAVE) grouped_gemm_kernel(GemmParam
     for (int kt = 0; kt < k_tiles; ++kt) {
         const int buf = kt & 1;
         if (kt + 1 < k_tiles) load_tiles(k_begin + (kt + 1) * BK);
+        const S* At = lds + buf * STAGE_ELEMS;
+        const S* Bt = At + ATile::ELEMS;
 #pragma unroll
         for (int kk = 0; kk < BK; kk += 16) {
             frag_t af[TM], bf[TN];
 #pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                const int r = wm * (BM / WM) + i * 32 + frag_row;
-                if (A_KC) {
-                    af[i] = *reinterpret_cast<const frag_t*>(&As[buf][r][kk + frag_k]);
-                } else {
+            for (int i = 0; i < TM; ++i)
+                af[i] = ATile::template fragment<frag_t>(At, wm * (BM / WM) + i * 32, kk, lane);
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) af[i][j] = As[buf][kk + frag_k + j][r];
-                }
-            }
-#pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                const int c = wn * (BN / WN) + j * 32 + frag_row;
-                if (B_KCC) {
-                    bf[j] = *reinterpret_cast<const frag_t*>(&Bs[buf][c][kk + frag_k]);
-                } else {
-#pragma unroll
-                    for (int q = 0; q < 8; ++q) bf[j][q] = Bs[buf][kk + frag_k + q][c];
-                }
-            }
+            for (int j = 0; j < TN; ++j)
+                bf[j] = BTile::template fragment<frag_t>(Bt, wn * (BN / WN) + j * 32, kk, lane);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -283,14 +313,31 @@ __global__ void __launch_bounds__(WM* WN* CK_WAVE) grouped_gemm_kernel(GemmParam
         __syncthreads();
     }
 
-    // ---- epilogue: lane holds column (lane % 32), rows 8 * (r / 4) + 4 * (lane / 32) + r % 4 --------------
+    // ---- epilogue -------------------------------------------------------------------------------
+    // Accumulators (lane: column lane % 32, rows 8 * (r / 4) + 4 * (lane / 32) + r % 4 of each 32x32 tile) are
+    // rounded and staged in LDS, then written out as 16-byte packets along rows, rows going to their mapped
+    // position.  The loop above ended with a barrier, so the operand buffers can be reused.
+    S* Ct = lds;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = wm * (BM / WM) + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
+                const int col = wn * (BN / WN) + j * 32 + lane % 32;
+                Ct[row * C_LD + col] = T::down(acc[i][j][r]);
+            }
+    __syncthreads();
     S* Cbase = reinterpret_cast<S*>(p.C) + (GROUP_K ? (int64_t)expert * p.c_stride_e : 0);
+    constexpr int C_CHUNKS_PER_ROW = BN / 8;
+    constexpr int C_CH = BM * C_CHUNKS_PER_ROW / THREADS;
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int row = wm * (BM / WM) + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
-            if (row >= rows_valid) continue;
+    for (int i = 0; i < C_CH; ++i) {
+        const int c = tid + i * THREADS;
+        const int row = c / C_CHUNKS_PER_ROW;
+        const int col = (c % C_CHUNKS_PER_ROW) * 8;
+        if (row < rows_valid && n_base + col < p.N) {
             int64_t out_row;
             if (GROUP_K) {
                 out_row = i_base + row;
@@ -298,12 +345,8 @@ __global__ void __launch_bounds__(WM* WN* CK_WAVE) grouped_gemm_kernel(GemmParam
                 const int64_t slot = row_start + row;
                 out_row = p.y_grouped ? slot : p.row_idx[slot];
             }
-            S* crow = Cbase + out_row * p.ldc;
-#pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                const int col = n_base + wn * (BN / WN) + j * 32 + frag_row;
-                if (col < p.N) crow[col] = T::down(acc[i][j][r]);
-            }
+            *reinterpret_cast<u32x4_t*>(Cbase + out_row * p.ldc + n_base + col) =
+                *reinterpret_cast<const u32x4_t*>(Ct + row * C_LD + col);
         }
     }
 }
@@ -388,14 +431,15 @@ __global__ void __launch_bounds__(256)
 // ---- host side ------------------------------------------------------------------------------
 namespace {
 
-constexpr int kBM = 128, kBN = 128, kBK = 64, kWM = 2, kWN = 2;
+typedef ck::Tile<256, 256, 64, 2, 4> MainTile;
+constexpr int kBM = MainTile::BM, kBN = MainTile::BN;
 
 template <typename T, bool B_KC, bool GROUP_K>
 void launch_mfma(const ck::GemmParams& p, hipStream_t s) {
     const int total = p.m_tiles * p.n_tiles;
     const int grid = (total + 7) / 8 * 8;
-    hipLaunchKernelGGL((ck::grouped_gemm_kernel<T, kBM, kBN, kBK, kWM, kWN, B_KC, GROUP_K>), dim3((unsigned)grid),
-                       dim3(kWM * kWN * CK_WAVE), 0, s, p);
+    hipLaunchKernelGGL((ck::grouped_gemm_kernel<T, MainTile, B_KC, GROUP_K>), dim3((unsigned)grid),
+                       dim3(MainTile::THREADS), 0, s, p);
 }
 
 bool mult8(int64_t v) { return (v & 7) == 0; }
@@ -418,8 +462,8 @@ extern "C" int ck_scatter2scatter(const void* X, int64_t x_stride, const void* W
 
     const bool b_kc = w_stride_k == 1, b_nc = w_stride_n == 1;
     const bool fast = dtype != CK_F32 && K > 0 && (b_kc || b_nc) && ck_aligned16(X) && ck_aligned16(W) && mult8(K) &&
-                      mult8(x_stride) && mult8(w_stride_e) && mult8(b_kc ? w_stride_n : w_stride_k) &&
-                      (b_kc || mult8(N));
+                      mult8(x_stride) && mult8(w_stride_e) && mult8(b_kc ? w_stride_n : w_stride_k) && mult8(N) &&
+                      ck_aligned16(out) && mult8(out_stride);
     if (fast) {
         ck::GemmParams p = {};
         p.A = X;
@@ -474,7 +518,8 @@ extern "C" int ck_group_bwd_W(const void* DY, int64_t dy_stride, const void* X, 
 
     const bool k_fast = dw_stride_k == 1, n_fast = dw_stride_n == 1;
     const bool fast = dtype != CK_F32 && (k_fast || n_fast) && ck_aligned16(X) && ck_aligned16(DY) && mult8(K) &&
-                      mult8(N) && mult8(x_stride) && mult8(dy_stride);
+                      mult8(N) && mult8(x_stride) && mult8(dy_stride) && ck_aligned16(DW) && mult8(dw_stride_e) &&
+                      mult8(k_fast ? dw_stride_n : dw_stride_k);
     if (fast) {
         // C[e][i][j] = sum_r P[r][i] * Q[r][j] with j the contiguous dimension of DW
         ck::GemmParams p = {};
