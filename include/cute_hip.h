@@ -158,6 +158,18 @@ int ck_group_bwd_W(const void* DY, int64_t dy_stride, const void* X, int64_t x_s
 int ck_group(const void* A, int64_t a_stride, const int64_t* idx, const void* coeff, void* out,
              int64_t out_stride, int64_t num_rows, int64_t K, int64_t fan_out, int dtype, void* stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * Mixing of each token's k expert outputs with its routing weights, and the routing weights' gradient
+ * replaces the two torch.bmm calls of scattermoe/triton_implementation/ops.py:160-164 and :204.
+ *   forward : out[t, :]     = sum_j gates[t, j] * expanded[t, j, :]      expanded [T, k, H], gates [T, k]
+ *   backward: d_gates[t, j] = sum_h expanded[t, j, h] * grad_out[t, h]
+ * All tensors dense.
+ * ------------------------------------------------------------------------------------------- */
+int ck_moe_combine_forward(const void* expanded, const void* gates, void* out, int64_t tokens, int64_t k,
+                           int64_t H, int dtype, void* stream);
+int ck_moe_combine_backward_gates(const void* expanded, const void* grad_out, void* d_gates, int64_t tokens,
+                                  int64_t k, int64_t H, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

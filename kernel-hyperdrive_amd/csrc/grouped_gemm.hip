@@ -11,6 +11,8 @@
 // never mixes rows of two experts (the reference lets a 128-row block straddle experts and repeats the
 // product once per expert present in it).  fp32, and shapes whose contiguous dimensions are not
 // multiples of 8 elements, go through a plain kernel with exact (fp64) accumulation.
+#include <cstdlib>
+
 #include "ck_device.h"
 
 namespace ck {
@@ -44,6 +46,7 @@ struct GemmParams {
     int M, N, K, E;          // S2S: slots, N, K.  XTY: rows, J (= N), I (= K)
     int fan_out, x_grouped, y_grouped;
     int m_tiles, n_tiles;    // S2S: upper bound of row tiles; XTY: tiles along I
+    int debug;
 };
 
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -292,7 +295,7 @@ __global__ void __launch_bounds__(TL::THREADS) grouped_gemm_kernel(GemmParams p)
     __syncthreads();
     for (int kt = 0; kt < k_tiles; ++kt) {
         const int buf = kt & 1;
-        if (kt + 1 < k_tiles) load_tiles(k_begin + (kt + 1) * BK);
+        if (kt + 1 < k_tiles && !(p.debug & 1)) load_tiles(k_begin + (kt + 1) * BK);
         const S* At = lds + buf * STAGE_ELEMS;
         const S* Bt = At + ATile::ELEMS;
 #pragma unroll
@@ -307,9 +310,9 @@ __global__ void __launch_bounds__(TL::THREADS) grouped_gemm_kernel(GemmParams p)
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int j = 0; j < TN; ++j) acc[i][j] = Mma<T>::mma(af[i], bf[j], acc[i][j]);
+                for (int j = 0; j < TN; ++j) if (!(p.debug & 2)) acc[i][j] = Mma<T>::mma(af[i], bf[j], acc[i][j]);
         }
-        if (kt + 1 < k_tiles) store_tiles(buf ^ 1);
+        if (kt + 1 < k_tiles && !(p.debug & 4)) store_tiles(buf ^ 1);
         __syncthreads();
     }
 
@@ -482,6 +485,7 @@ extern "C" int ck_scatter2scatter(const void* X, int64_t x_stride, const void* W
         p.fan_out = (int)fan_out;
         p.x_grouped = x_grouped;
         p.y_grouped = y_grouped;
+        { const char* d = getenv("CK_GEMM_DEBUG"); p.debug = d ? atoi(d) : 0; }
         p.m_tiles = (int)(num_slots / kBM + E);
         p.n_tiles = (int)ck_ceil_div(N, kBN);
         if ((int64_t)p.m_tiles * p.n_tiles > 0x7ffffff0) return CK_ERR_SHAPE;
@@ -536,6 +540,7 @@ extern "C" int ck_group_bwd_W(const void* DY, int64_t dy_stride, const void* X, 
         p.K = (int)(swap ? N : K);  // I
         p.N = (int)(swap ? K : N);  // J
         p.E = (int)E;
+        { const char* d = getenv("CK_GEMM_DEBUG"); p.debug = d ? atoi(d) : 0; }
         p.m_tiles = (int)(E * ck_ceil_div(p.K, kBM));
         p.n_tiles = (int)ck_ceil_div(p.N, kBN);
         if ((int64_t)p.m_tiles * p.n_tiles > 0x7ffffff0) return CK_ERR_SHAPE;

@@ -53,6 +53,8 @@ _SIGNATURES = {
     "ck_offsets_from_sorted": (_i32, [_p, _p, _i64, _i64, _p]),
     "ck_group_bwd_W": (_i32, [_p, _i64, _p, _i64, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _p]),
     "ck_group": (_i32, [_p, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _i32, _p]),
+    "ck_moe_combine_forward": (_i32, [_p, _p, _p, _i64, _i64, _i64, _i32, _p]),
+    "ck_moe_combine_backward_gates": (_i32, [_p, _p, _p, _i64, _i64, _i64, _i32, _p]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
@@ -361,4 +363,28 @@ def group(A, idx, coeff, out, fan_out: int) -> None:
             lib.ck_group(_ptr(A), A.stride(0), _ptr(idx), _ptr(coeff), _ptr(out), out.stride(0), idx.numel(),
                          A.size(1), fan_out, dtype_code(A.dtype), L.stream),
             "ck_group",
+        )
+
+
+def moe_combine_forward(expanded, gates, out) -> None:
+    """expanded [T, k, H], gates [T, k], out [T, H]; all dense."""
+    lib = load_library()
+    T, k, H = expanded.shape
+    with _Launch(expanded, gates, out) as L:
+        _check(
+            lib.ck_moe_combine_forward(_ptr(expanded), _ptr(gates), _ptr(out), T, k, H, dtype_code(expanded.dtype),
+                                       L.stream),
+            "ck_moe_combine_forward",
+        )
+
+
+def moe_combine_backward_gates(expanded, grad_out, d_gates) -> None:
+    """expanded [T, k, H], grad_out [T, H], d_gates [T, k]; all dense."""
+    lib = load_library()
+    T, k, H = expanded.shape
+    with _Launch(expanded, grad_out, d_gates) as L:
+        _check(
+            lib.ck_moe_combine_backward_gates(_ptr(expanded), _ptr(grad_out), _ptr(d_gates), T, k, H,
+                                              dtype_code(expanded.dtype), L.stream),
+            "ck_moe_combine_backward_gates",
         )

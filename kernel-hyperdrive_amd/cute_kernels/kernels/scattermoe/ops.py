@@ -6,6 +6,8 @@ registration of cute_kernels/kernels/scattermoe/triton_implementation/ops.py:16-
 saved tensors, same nine gradient slots).  Differences that do not change results:
   * ``scatter2scatter`` takes the expert offsets as an optional trailing argument (the tile scheduler works
     per expert); without it they are recomputed from the sorted expert ids;
+  * the two ``torch.bmm`` calls that mix expert outputs with the routing weights (ops.py:160-164, 204) are
+    single-pass kernels (``moe_combine_forward`` / ``moe_combine_backward_gates``);
   * the weight gradient is written completely by the kernel (zeros for experts without rows), so it is
     allocated with ``empty_like`` instead of ``zeros_like`` (ops.py:237).
 """
@@ -73,6 +75,18 @@ def group(
     _C.group(A, sorted_expert_idxs, coeff, out, fan_out)
 
 
+@cute_op(f"{LIBRARY_NAME}::moe_combine_forward", mutates_args={"out"})
+def moe_combine_forward(expanded: torch.Tensor, gates: torch.Tensor, out: torch.Tensor) -> None:
+    """out[t] = sum_j gates[t, j] * expanded[t, j]  (the reference's bmm(gates[T,1,k], expanded[T,k,H]))."""
+    _C.moe_combine_forward(expanded.contiguous(), gates.contiguous(), out)
+
+
+@cute_op(f"{LIBRARY_NAME}::moe_combine_backward_gates", mutates_args={"d_gates"})
+def moe_combine_backward_gates(expanded: torch.Tensor, grad_out: torch.Tensor, d_gates: torch.Tensor) -> None:
+    """d_gates[t, j] = <expanded[t, j], grad_out[t]>  (the reference's bmm(expanded[T,k,H], grad_out[T,H,1]))."""
+    _C.moe_combine_backward_gates(expanded.contiguous(), grad_out.contiguous(), d_gates)
+
+
 class _ScatteredExperts(torch.autograd.Function):
     @staticmethod
     def forward(
@@ -106,7 +120,8 @@ class _ScatteredExperts(torch.autograd.Function):
         else:
             # rows are back in (token, slot) order: mix each token's k expert outputs with its routing weights
             output_expanded = output.view(gates.size(0), gates.size(1), output.size(-1))
-            output = torch.bmm(gates.unsqueeze(1), output_expanded).squeeze(1)
+            output = torch.empty(gates.size(0), output.size(-1), device=x.device, dtype=x.dtype)
+            moe_combine_forward(expanded=output_expanded, gates=gates, out=output)
 
         ctx.save_for_backward(
             x, expert_weights, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, gates, output_expanded
@@ -140,7 +155,8 @@ class _ScatteredExperts(torch.autograd.Function):
             gate_fan = 1
             grouped_grad_out = None
         else:
-            d_gates = torch.bmm(output_expanded, grad_out.unsqueeze(2)).squeeze(-1)
+            d_gates = torch.empty_like(gates)
+            moe_combine_backward_gates(expanded=output_expanded, grad_out=grad_out, d_gates=d_gates)
             gates_flat = gates.flatten()
             gate_fan = gates.size(1)
             grouped_grad_out = output_expanded.flatten(0, 1)  # saved buffer, overwritten below

@@ -14,6 +14,8 @@ stock torch ops on random inputs):
                       dense one-hot matmul and ``F.embedding`` autograd in fp64
   contiguous_count    numpy.bincount(minlength) (tests/kernels/contiguous_count_test.py:35)
   moe_sort            stable argsort; checked against a brute-force insertion on tiny inputs
+  moe_combine_*       the two torch.bmm calls of scattermoe/triton_implementation/ops.py:160-164, 204; checked
+                      against torch.bmm in fp64
   scatter2scatter, group_bwd_W, group
                       per-slot / per-expert loops straight from the kernel docstrings
                       (scattermoe/triton_implementation/kernels.py:66-102, 152-240, 243-298)
@@ -201,6 +203,16 @@ def group(A, idx, coeff, fan_out):
     if coeff is None:
         return rows.clone()
     return (rows.float() * coeff[idx.long()].float().unsqueeze(-1)).to(A.dtype)
+
+
+def moe_combine_forward(expanded, gates, compute_dtype=torch.float32):
+    """out[t] = sum_j gates[t, j] * expanded[t, j]: bmm(gates[T,1,k], expanded[T,k,H])  (ops.py:160-164)."""
+    return (gates.to(compute_dtype).unsqueeze(-1) * expanded.to(compute_dtype)).sum(dim=1).to(expanded.dtype)
+
+
+def moe_combine_backward_gates(expanded, grad_out, compute_dtype=torch.float32):
+    """d_gates[t, j] = <expanded[t, j], grad_out[t]>: bmm(expanded[T,k,H], grad_out[T,H,1])  (ops.py:204)."""
+    return (expanded.to(compute_dtype) * grad_out.to(compute_dtype).unsqueeze(1)).sum(dim=-1).to(expanded.dtype)
 
 
 # =====================================================================================================

@@ -106,6 +106,28 @@ def test_group(gpu, dtype, K, with_coeff):
         assert torch.equal(out.cpu(), expected)
 
 
+# ---- mixing with the routing weights ------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape", [(1, 1, 8), (77, 2, 4096), (33, 6, 2048), (50, 3, 30)])
+def test_moe_combine(gpu, dtype, shape):
+    from cute_kernels.kernels.scattermoe.ops import moe_combine_backward_gates, moe_combine_forward
+
+    announce("moe_combine", dtype, shape)
+    T, k, H = shape
+    expanded, gates, dy = randn((T, k, H), dtype, 54), randn((T, k), dtype, 55, 0.5), randn((T, H), dtype, 56)
+    out = torch.empty(T, H, dtype=dtype, device=gpu)
+    moe_combine_forward(expanded.to(gpu), gates.to(gpu), out)
+    assert_close(out, O.moe_combine_forward(expanded, gates, acc_dtype(dtype)), dtype, "out")
+    d_gates = torch.empty(T, k, dtype=dtype, device=gpu)
+    moe_combine_backward_gates(expanded.to(gpu), dy.to(gpu), d_gates)
+    # a dot product over H terms of O(1): compared norm-wise for fp32 (fp32 accumulation), element-wise for 16 bit
+    expected = O.moe_combine_backward_gates(expanded, dy, acc_dtype(dtype))
+    if dtype == torch.float32:
+        assert_norm_close(d_gates, expected, 1e-5, "d_gates")
+    else:
+        assert_close(d_gates, expected, dtype, "d_gates")
+
+
 # ---- the whole layer ----------------------------------------------------------------------------------
 def build_moe(cls, gpu, dtype, E, k, H, I, w_gate, w_fc, w_proj):
     from cute_kernels import swiglu_unchunked_cute

@@ -216,6 +216,15 @@ def test_group_bwd_w_and_group():
     assert torch.equal(O.group(A, s_idx, None, k), A[s_idx // k])
 
 
+def test_moe_combine_against_bmm():
+    T, k, H = 9, 3, 7
+    expanded = torch.randn(T, k, H, dtype=F64)
+    gates = torch.randn(T, k, dtype=F64)
+    dy = torch.randn(T, H, dtype=F64)
+    assert torch.allclose(O.moe_combine_forward(expanded, gates, F64), torch.bmm(gates.unsqueeze(1), expanded).squeeze(1), atol=1e-13)
+    assert torch.allclose(O.moe_combine_backward_gates(expanded, dy, F64), torch.bmm(expanded, dy.unsqueeze(2)).squeeze(-1), atol=1e-13)
+
+
 # ---- the MoE layer ------------------------------------------------------------------------------------
 @pytest.mark.parametrize("top_k", [1, 2, 3])
 def test_moe_restatement_against_dense_per_token(top_k):
