@@ -354,6 +354,303 @@ __global__ void __launch_bounds__(TL::THREADS) grouped_gemm_kernel(GemmParams p)
     }
 }
 
+// =====================================================================================================
+// Direct-to-LDS version of the MFMA kernel (BK = 64, two LDS stages)
+// =====================================================================================================
+// Operand tiles go from global memory straight into LDS with global_load_lds_dwordx4: no staging
+// registers, no ds_write burst at the end of a step, and the copy overlaps the MFMAs of the current step.
+// One wave instruction fills 64 consecutive 16-byte slots, so rows cannot be padded; bank conflicts are
+// avoided by an XOR swizzle applied on the global side (which 16-byte chunk a lane fetches) and undone
+// when fragments are read:
+//   k-contiguous operand, row = 128 B = 8 slots:   slot = chunk ^ ((row >> 1) & 7)
+//   other layout, contraction row = ROWS * 2 B:    slot = chunk ^ ((k & 3) << 2)
+// LDS positions whose contraction index lies beyond the end of the contraction range are cleared with a
+// plain store in the (single) partial step; positions of rows / columns outside the problem keep whatever
+// they held, which only reaches outputs that are never stored.
+template <typename S, int ROWS, bool KC, int NWAVES>
+struct DtlOperand {
+    static constexpr int BK = 64;
+    static constexpr int STAGE_BYTES = ROWS * BK * 2;
+    static constexpr int SLOTS = STAGE_BYTES / 16;
+    static constexpr int IPW = SLOTS / (CK_WAVE * NWAVES);  // load instructions per wave per stage
+    static constexpr int SLOTS_PER_LINE = KC ? 8 : ROWS / 8;
+    static_assert(SLOTS % (CK_WAVE * NWAVES) == 0, "operand tile / waves");
+
+    // slot p of the stage -> (line, chunk) it has to hold; line = row (KC) or contraction index (other)
+    static __device__ __forceinline__ void slot_source(int p, int& line, int& chunk) {
+        line = p / SLOTS_PER_LINE;
+        const int slot = p % SLOTS_PER_LINE;
+        chunk = KC ? (slot ^ ((line >> 1) & 7)) : (slot ^ ((line & 3) << 2));
+    }
+};
+
+template <typename T, typename TL, bool B_KC, bool GROUP_K>
+__global__ void __launch_bounds__(TL::THREADS) grouped_gemm_dtl_kernel(GemmParams p) {
+    typedef typename T::storage_t S;
+    typedef typename Mma<T>::frag_t frag_t;
+    constexpr int BM = TL::BM, BN = TL::BN, BK = 64, WM = TL::WM, WN = TL::WN;
+    constexpr int THREADS = TL::THREADS, TM = TL::TM, TN = TL::TN, NWAVES = WM * WN;
+    static_assert(TL::BK == 64, "the direct-to-LDS kernel is written for BK = 64");
+    static_assert(WM == 2, "the epilogue stages one half of the rows per stage buffer");
+    constexpr bool A_KC = !GROUP_K;
+    constexpr bool B_KCC = GROUP_K ? false : B_KC;
+    typedef DtlOperand<S, BM, A_KC, NWAVES> AOp;
+    typedef DtlOperand<S, BN, B_KCC, NWAVES> BOp;
+    constexpr int STAGE_BYTES = AOp::STAGE_BYTES + BOp::STAGE_BYTES;
+    constexpr int C_LD = BN + 8;
+    constexpr int HALF_C_BYTES = (BM / 2) * C_LD * 2;  // staged output rows of one wave row-group
+    constexpr int BUF_BYTES = STAGE_BYTES > HALF_C_BYTES ? STAGE_BYTES : HALF_C_BYTES;
+    // Two separate LDS objects, one per stage: a read of one stage then provably does not touch the other, so
+    // the compiler does not make fragment reads wait for the copies that are filling the other stage.
+    __shared__ __attribute__((aligned(1024))) char lds0[BUF_BYTES];
+    __shared__ __attribute__((aligned(1024))) char lds1[BUF_BYTES];
+    __shared__ int sh_info[4];
+
+    int mt, nt;
+    if (!logical_tile(p.m_tiles, p.n_tiles, mt, nt)) return;
+
+    const int tid = threadIdx.x;
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane(tid / CK_WAVE);
+    const int wm = wave / WN, wn = wave % WN;
+
+    int expert, row_start, rows_valid, k_begin, k_end, i_base;
+    if (!GROUP_K) {
+        find_tile<BM>(p.offsets, p.E, mt, sh_info);
+        expert = sh_info[0];
+        row_start = sh_info[1];
+        rows_valid = sh_info[2];
+        if (expert < 0) return;
+        k_begin = 0;
+        k_end = p.K;
+        i_base = 0;
+    } else {
+        const int i_tiles = p.m_tiles / p.E;
+        expert = mt / i_tiles;
+        i_base = (mt % i_tiles) * BM;
+        k_begin = expert == 0 ? 0 : (int)p.offsets[expert - 1];
+        k_end = (int)p.offsets[expert];
+        row_start = 0;
+        rows_valid = min(BM, p.K - i_base);
+    }
+    const int n_base = nt * BN;
+    const int cols_valid = min(BN, p.N - n_base);  // > 0 and a multiple of 8
+
+    // ---- per-lane sources of the LDS slots this lane fills ----------------------------------------
+    // Lines / chunks outside the problem are redirected to a valid one (their LDS content is never used for a
+    // stored output), so full steps need no predicate at all.
+    const S* Abase = reinterpret_cast<const S*>(p.A);
+    const S* Bbase = reinterpret_cast<const S*>(p.B) + (GROUP_K ? 0 : (int64_t)expert * p.b_stride_e);
+    const S* a_ptr[AOp::IPW];
+    int a_k[AOp::IPW];  // contraction offset of the slot inside a step
+    const S* b_ptr[BOp::IPW];
+    int b_k[BOp::IPW];
+#pragma unroll
+    for (int j = 0; j < AOp::IPW; ++j) {
+        int line, chunk;
+        AOp::slot_source((wave * AOp::IPW + j) * CK_WAVE + lane, line, chunk);
+        if (A_KC) {
+            const int r = min(line, rows_valid - 1);
+            const int64_t slot = row_start + r;
+            const int64_t src_row = p.x_grouped ? slot : (int64_t)((uint32_t)p.row_idx[slot] / (uint32_t)p.fan_out);
+            a_k[j] = chunk * 8;
+            a_ptr[j] = Abase + src_row * p.lda + k_begin + a_k[j];
+        } else {
+            const int cc = (chunk * 8 < rows_valid) ? chunk * 8 : 0;
+            a_k[j] = line;
+            a_ptr[j] = Abase + (int64_t)(k_begin + line) * p.lda + i_base + cc;
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < BOp::IPW; ++j) {
+        int line, chunk;
+        BOp::slot_source((wave * BOp::IPW + j) * CK_WAVE + lane, line, chunk);
+        if (B_KCC) {
+            const int r = min(line, cols_valid - 1);
+            b_k[j] = chunk * 8;
+            b_ptr[j] = Bbase + (int64_t)(n_base + r) * p.ldb + k_begin + b_k[j];
+        } else {
+            const int cc = (chunk * 8 < cols_valid) ? chunk * 8 : 0;
+            b_k[j] = line;
+            b_ptr[j] = Bbase + (int64_t)(k_begin + line) * p.ldb + n_base + cc;
+        }
+    }
+    const int64_t a_step = A_KC ? BK : (int64_t)BK * p.lda;
+    const int64_t b_step = B_KCC ? BK : (int64_t)BK * p.ldb;
+
+    typedef __attribute__((address_space(1))) const void* gptr_t;
+    typedef __attribute__((address_space(3))) void* lptr_t;
+    // request tile `kt` into stage buffer `st`; slots past the end of the contraction are cleared instead
+    auto issue = [&](int kt, char* st) {
+        const int k0 = k_begin + kt * BK;
+        if (k0 + BK <= k_end) {
+#pragma unroll
+            for (int j = 0; j < AOp::IPW; ++j) {
+                __builtin_amdgcn_global_load_lds((gptr_t)a_ptr[j], (lptr_t)(st + (wave * AOp::IPW + j) * 1024), 16, 0, 0);
+                a_ptr[j] += a_step;
+            }
+#pragma unroll
+            for (int j = 0; j < BOp::IPW; ++j) {
+                __builtin_amdgcn_global_load_lds(
+                    (gptr_t)b_ptr[j], (lptr_t)(st + AOp::STAGE_BYTES + (wave * BOp::IPW + j) * 1024), 16, 0, 0);
+                b_ptr[j] += b_step;
+            }
+        } else {
+            const u32x4_t zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int j = 0; j < AOp::IPW; ++j) {
+                char* dst = st + (wave * AOp::IPW + j) * 1024;
+                if (k0 + a_k[j] < k_end)
+                    __builtin_amdgcn_global_load_lds((gptr_t)a_ptr[j], (lptr_t)dst, 16, 0, 0);
+                else
+                    *reinterpret_cast<u32x4_t*>(dst + lane * 16) = zero;
+            }
+#pragma unroll
+            for (int j = 0; j < BOp::IPW; ++j) {
+                char* dst = st + AOp::STAGE_BYTES + (wave * BOp::IPW + j) * 1024;
+                if (k0 + b_k[j] < k_end)
+                    __builtin_amdgcn_global_load_lds((gptr_t)b_ptr[j], (lptr_t)dst, 16, 0, 0);
+                else
+                    *reinterpret_cast<u32x4_t*>(dst + lane * 16) = zero;
+            }
+        }
+    };
+
+    // ---- per-lane fragment addresses (bytes inside an operand stage) ---------------------------------
+    int a_off[TM], a_xor[TM], b_off[TN], b_xor[TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        const int r0 = wm * (BM / WM) + i * 32;
+        if (A_KC) {
+            const int r = r0 + lane % 32;
+            a_off[i] = r * 128;
+            a_xor[i] = ((lane / 32) ^ ((r >> 1) & 7)) << 4;  // chunk (kk / 8 + lane / 32) ^ swizzle, kk / 8 even
+        } else {
+            const int g = lane / 16, q = lane % 16;
+            const int col = r0 + (g % 2) * 16 + (q % 4) * 4;
+            a_off[i] = ((g / 2) * 8 + q / 4) * (BM * 2) + ((((col / 8) ^ ((q / 4) << 2))) << 4) + (col % 8) * 2;
+            a_xor[i] = 0;
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int c0 = wn * (BN / WN) + j * 32;
+        if (B_KCC) {
+            const int r = c0 + lane % 32;
+            b_off[j] = AOp::STAGE_BYTES + r * 128;
+            b_xor[j] = ((lane / 32) ^ ((r >> 1) & 7)) << 4;
+        } else {
+            const int g = lane / 16, q = lane % 16;
+            const int col = c0 + (g % 2) * 16 + (q % 4) * 4;
+            b_off[j] = AOp::STAGE_BYTES + ((g / 2) * 8 + q / 4) * (BN * 2) + ((((col / 8) ^ ((q / 4) << 2))) << 4) +
+                       (col % 8) * 2;
+            b_xor[j] = 0;
+        }
+    }
+    auto a_frag = [&](const char* st, int i, int kk) -> frag_t {
+        if (A_KC) {
+            return *reinterpret_cast<const frag_t*>(st + a_off[i] + (a_xor[i] ^ ((kk / 8) << 4)));
+        } else {
+            const char* q = st + a_off[i] + kk * (BM * 2);
+            union {
+                v4i16_t h[2];
+                frag_t f;
+            } u;
+            u.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(q));
+            u.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(q + 4 * (BM * 2)));
+            return u.f;
+        }
+    };
+    auto b_frag = [&](const char* st, int j, int kk) -> frag_t {
+        if (B_KCC) {
+            return *reinterpret_cast<const frag_t*>(st + b_off[j] + (b_xor[j] ^ ((kk / 8) << 4)));
+        } else {
+            const char* q = st + b_off[j] + kk * (BN * 2);
+            union {
+                v4i16_t h[2];
+                frag_t f;
+            } u;
+            u.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(q));
+            u.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(q + 4 * (BN * 2)));
+            return u.f;
+        }
+    };
+
+    f32x16_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    // one step: request tile kt + 1 into `fill` (last read in step kt - 1, which every wave has left), multiply
+    // tile kt out of `cur`, then wait for the requested tile and meet the other waves
+    auto step = [&](int kt, int k_tiles, const char* cur, char* fill) {
+        if (kt + 1 < k_tiles && !(p.debug & 1)) issue(kt + 1, fill);
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 16) {
+            frag_t af[TM], bf[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) af[i] = a_frag(cur, i, kk);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) bf[j] = b_frag(cur, j, kk);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) acc[i][j] = Mma<T>::mma(af[i], bf[j], acc[i][j]);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+    };
+
+    const int k_tiles = (k_end - k_begin + BK - 1) / BK;
+    if (k_tiles > 0) issue(0, lds0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    for (int kt = 0; kt < k_tiles; kt += 2) {
+        step(kt, k_tiles, lds0, lds1);
+        if (kt + 1 < k_tiles) step(kt + 1, k_tiles, lds1, lds0);
+    }
+
+    // ---- epilogue -----------------------------------------------------------------------------------
+    // Accumulators (lane: column lane % 32, rows 8 * (r / 4) + 4 * (lane / 32) + r % 4 of each 32x32 tile) are
+    // rounded and staged in LDS - the upper half of the rows in one stage buffer, the lower half in the other -
+    // then written out as 16-byte packets along rows, rows going to their mapped position.
+    S* Ch = reinterpret_cast<S*>(wm == 0 ? lds0 : lds1);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);  // inside this half
+                const int col = wn * (BN / WN) + j * 32 + lane % 32;
+                Ch[row * C_LD + col] = T::down(acc[i][j][r]);
+            }
+    __syncthreads();
+    S* Cbase = reinterpret_cast<S*>(p.C) + (GROUP_K ? (int64_t)expert * p.c_stride_e : 0);
+    constexpr int C_CHUNKS_PER_ROW = BN / 8;
+    constexpr int C_CH = BM * C_CHUNKS_PER_ROW / THREADS;
+#pragma unroll
+    for (int i = 0; i < C_CH; ++i) {
+        const int c = tid + i * THREADS;
+        const int row = c / C_CHUNKS_PER_ROW;
+        const int col = (c % C_CHUNKS_PER_ROW) * 8;
+        if (row < rows_valid && col < cols_valid) {
+            int64_t out_row;
+            if (GROUP_K) {
+                out_row = i_base + row;
+            } else {
+                const int64_t slot = row_start + row;
+                out_row = p.y_grouped ? slot : p.row_idx[slot];
+            }
+            const S* src = reinterpret_cast<const S*>(row < BM / 2 ? lds0 : lds1) + (row % (BM / 2)) * C_LD + col;
+            *reinterpret_cast<u32x4_t*>(Cbase + out_row * p.ldc + n_base + col) = *reinterpret_cast<const u32x4_t*>(src);
+        }
+    }
+}
+
 // ---- plain kernels (fp32 and irregular shapes) ---------------------------------------------------
 // One lane per output element, fp64 accumulation: the fp32 path promises 1e-5, which an fp32 sum of a few
 // hundred O(1) terms does not keep in any order, so the sum is made exact and rounded once.
@@ -434,15 +731,22 @@ __global__ void __launch_bounds__(256)
 // ---- host side ------------------------------------------------------------------------------
 namespace {
 
-typedef ck::Tile<256, 256, 64, 2, 4> MainTile;
+#ifndef CK_TILE_CONFIG
+#define CK_TILE_CONFIG 256, 256, 64, 2, 4
+#endif
+typedef ck::Tile<CK_TILE_CONFIG> MainTile;
 constexpr int kBM = MainTile::BM, kBN = MainTile::BN;
 
 template <typename T, bool B_KC, bool GROUP_K>
 void launch_mfma(const ck::GemmParams& p, hipStream_t s) {
     const int total = p.m_tiles * p.n_tiles;
     const int grid = (total + 7) / 8 * 8;
-    hipLaunchKernelGGL((ck::grouped_gemm_kernel<T, MainTile, B_KC, GROUP_K>), dim3((unsigned)grid),
-                       dim3(MainTile::THREADS), 0, s, p);
+    if (p.debug & 16)
+        hipLaunchKernelGGL((ck::grouped_gemm_kernel<T, MainTile, B_KC, GROUP_K>), dim3((unsigned)grid),
+                           dim3(MainTile::THREADS), 0, s, p);
+    else
+        hipLaunchKernelGGL((ck::grouped_gemm_dtl_kernel<T, MainTile, B_KC, GROUP_K>), dim3((unsigned)grid),
+                           dim3(MainTile::THREADS), 0, s, p);
 }
 
 bool mult8(int64_t v) { return (v & 7) == 0; }

@@ -15,7 +15,10 @@ import threading
 import torch
 
 
-_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libcute_hip.so")
+# CUTE_HIP_LIBRARY points at another build of the same library (kernel experiments)
+_LIB_PATH = os.environ.get("CUTE_HIP_LIBRARY") or os.path.join(
+    os.path.dirname(os.path.abspath(__file__)), "lib", "libcute_hip.so"
+)
 _ABI_VERSION = 1
 
 _lib = None
