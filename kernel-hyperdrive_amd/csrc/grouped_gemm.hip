@@ -475,8 +475,8 @@ __global__ void __launch_bounds__(TL::THREADS) grouped_gemm_dtl_kernel(GemmParam
             b_ptr[j] = Bbase + (int64_t)(k_begin + line) * p.ldb + n_base + cc;
         }
     }
-    const int64_t a_step = A_KC ? BK : (int64_t)BK * p.lda;
-    const int64_t b_step = B_KCC ? BK : (int64_t)BK * p.ldb;
+    const int64_t a_step = (p.debug & 2) ? 0 : (A_KC ? BK : (int64_t)BK * p.lda);
+    const int64_t b_step = (p.debug & 2) ? 0 : (B_KCC ? BK : (int64_t)BK * p.ldb);
 
     typedef __attribute__((address_space(1))) const void* gptr_t;
     typedef __attribute__((address_space(3))) void* lptr_t;
@@ -584,10 +584,35 @@ __global__ void __launch_bounds__(TL::THREADS) grouped_gemm_dtl_kernel(GemmParam
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
+    // copies of a full tile, one quarter at a time (quarter q of 4), so that they can be spread over a step
+    auto issue_quarter = [&](char* st, int q) {
+#pragma unroll
+        for (int j = 0; j < AOp::IPW; ++j)
+            if (j % 4 == q || AOp::IPW < 4) {
+                if (AOp::IPW >= 4 || q == 0) {
+                    __builtin_amdgcn_global_load_lds((gptr_t)a_ptr[j], (lptr_t)(st + (wave * AOp::IPW + j) * 1024), 16, 0, 0);
+                    a_ptr[j] += a_step;
+                }
+            }
+#pragma unroll
+        for (int j = 0; j < BOp::IPW; ++j)
+            if (j % 4 == q || BOp::IPW < 4) {
+                if (BOp::IPW >= 4 || q == 0) {
+                    __builtin_amdgcn_global_load_lds(
+                        (gptr_t)b_ptr[j], (lptr_t)(st + AOp::STAGE_BYTES + (wave * BOp::IPW + j) * 1024), 16, 0, 0);
+                    b_ptr[j] += b_step;
+                }
+            }
+    };
+
     // one step: request tile kt + 1 into `fill` (last read in step kt - 1, which every wave has left), multiply
-    // tile kt out of `cur`, then wait for the requested tile and meet the other waves
+    // tile kt out of `cur`, then wait for the requested tile and meet the other waves.  The copies of a full
+    // tile are issued in four parts between the four MFMA groups, which keeps the memory pipeline and the LDS
+    // evenly loaded instead of hitting them with the whole tile at once.
     auto step = [&](int kt, int k_tiles, const char* cur, char* fill) {
-        if (kt + 1 < k_tiles && !(p.debug & 1)) issue(kt + 1, fill);
+        const bool more = kt + 1 < k_tiles && !(p.debug & 1);
+        const bool spread = more && k_begin + (kt + 2) * BK <= k_end;
+        if (more && !spread) issue(kt + 1, fill);
 #pragma unroll
         for (int kk = 0; kk < BK; kk += 16) {
             frag_t af[TM], bf[TN];
@@ -595,13 +620,14 @@ __global__ void __launch_bounds__(TL::THREADS) grouped_gemm_dtl_kernel(GemmParam
             for (int i = 0; i < TM; ++i) af[i] = a_frag(cur, i, kk);
 #pragma unroll
             for (int j = 0; j < TN; ++j) bf[j] = b_frag(cur, j, kk);
+            if (spread) issue_quarter(fill, kk / 16);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j) acc[i][j] = Mma<T>::mma(af[i], bf[j], acc[i][j]);
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
+        if (!(p.debug & 32)) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (!(p.debug & 64)) __syncthreads();
     };
 
     const int k_tiles = (k_end - k_begin + BK - 1) / BK;
