@@ -38,6 +38,7 @@ def parse_args():
     p.add_argument("--warmup", type=int, default=3)
     p.add_argument("--no-extras", action="store_true", help="skip the SwiGLU / RMSNorm / embedding bandwidth figures")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    p.add_argument("--only-extras", action="store_true", help="only the HBM-bound ops (for profiling them)")
     p.add_argument("--tokens", type=int, default=8192, help="T of the MoE workload (default: the BASELINE shape)")
     return p.parse_args()
 
@@ -242,6 +243,9 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     device = torch.device("cuda", 0)
+    if args.only_extras:
+        print(json.dumps({"extras": bench_extras(device)}))
+        return
     result, roofline, config = bench_moe(device, args)
     line = {
         "metric": "scattermoe_fwd_bwd_tflops",

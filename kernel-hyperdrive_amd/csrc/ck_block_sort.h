@@ -17,6 +17,7 @@ constexpr int kSortThreads = 1024;
 constexpr int kSortWaves = kSortThreads / CK_WAVE;
 constexpr int kSortMaxBits = 8;
 constexpr int kSortBins = 1 << kSortMaxBits;
+constexpr int kSortAhead = 16;  // batches of 64 keys requested together
 
 struct SortShared {
     int hist[kSortWaves][kSortBins];  // per-wave digit counts, then per-wave exclusive offsets
@@ -51,14 +52,25 @@ __device__ __forceinline__ void block_radix_pass(SortShared& sh, int n, int shif
     for (int d = lane; d < nbins; d += CK_WAVE) sh.hist[wave][d] = 0;
     // (each wave touches only its own histogram row: program order inside the wave is enough)
 
-    for (int i0 = begin; i0 < end; i0 += CK_WAVE) {
-        const int i = i0 + lane;
-        const bool valid = i < end;
-        uint32_t key = 0, val = 0;
-        if (valid) load(i, key, val);
-        const uint32_t digit = (key >> shift) & mask;
-        const uint64_t m = wave_match(digit, bits, valid);
-        if (valid && (m & lanemask_lt()) == 0) sh.hist[wave][digit] += __popcll(m);
+    // keys are fetched kSortAhead batches at a time so that their memory latency is paid once per group, not
+    // once per batch; the batches of a group are then ranked one after the other, in order
+    for (int g0 = begin; g0 < end; g0 += CK_WAVE * kSortAhead) {
+        uint32_t keys[kSortAhead], vals[kSortAhead];
+#pragma unroll
+        for (int u = 0; u < kSortAhead; ++u) {
+            const int i = g0 + u * CK_WAVE + lane;
+            keys[u] = 0;
+            vals[u] = 0;
+            if (i < end) load(i, keys[u], vals[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < kSortAhead; ++u) {
+            const int i = g0 + u * CK_WAVE + lane;
+            const bool valid = i < end;
+            const uint32_t digit = (keys[u] >> shift) & mask;
+            const uint64_t m = wave_match(digit, bits, valid);
+            if (valid && (m & lanemask_lt()) == 0) sh.hist[wave][digit] += __popcll(m);
+        }
     }
     __syncthreads();
 
@@ -94,19 +106,28 @@ __device__ __forceinline__ void block_radix_pass(SortShared& sh, int n, int shif
     }
     __syncthreads();
 
-    for (int i0 = begin; i0 < end; i0 += CK_WAVE) {
-        const int i = i0 + lane;
-        const bool valid = i < end;
-        uint32_t key = 0, val = 0;
-        if (valid) load(i, key, val);
-        const uint32_t digit = (key >> shift) & mask;
-        const uint64_t m = wave_match(digit, bits, valid);
-        const uint64_t lower = m & lanemask_lt();
-        int pos = 0;
-        if (valid) pos = sh.digit_base[digit] + sh.hist[wave][digit] + __popcll(lower);
-        // all lanes have read the running offset before the group's first lane advances it
-        if (valid && lower == 0) sh.hist[wave][digit] += __popcll(m);
-        if (valid) store(pos, key, val);
+    for (int g0 = begin; g0 < end; g0 += CK_WAVE * kSortAhead) {
+        uint32_t keys[kSortAhead], vals[kSortAhead];
+#pragma unroll
+        for (int u = 0; u < kSortAhead; ++u) {
+            const int i = g0 + u * CK_WAVE + lane;
+            keys[u] = 0;
+            vals[u] = 0;
+            if (i < end) load(i, keys[u], vals[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < kSortAhead; ++u) {
+            const int i = g0 + u * CK_WAVE + lane;
+            const bool valid = i < end;
+            const uint32_t digit = (keys[u] >> shift) & mask;
+            const uint64_t m = wave_match(digit, bits, valid);
+            const uint64_t lower = m & lanemask_lt();
+            int pos = 0;
+            if (valid) pos = sh.digit_base[digit] + sh.hist[wave][digit] + __popcll(lower);
+            // all lanes have read the running offset before the group's first lane advances it
+            if (valid && lower == 0) sh.hist[wave][digit] += __popcll(m);
+            if (valid) store(pos, keys[u], vals[u]);
+        }
     }
     __threadfence_block();
     __syncthreads();

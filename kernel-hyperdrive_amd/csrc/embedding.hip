@@ -5,17 +5,18 @@
 //             (math: cute_kernels/kernels/embedding/README.md:7-15).  The reference adds rows with
 //             floating-point atomics into a zeroed table (kernels_backward.py:13-45); here the token
 //             ids are sorted first so that every table row has exactly one writer:
-//               1. sort kernel (one workgroup): stable radix sort of (id, position); marks which
-//                  table rows are selected at all; for every sorted slot the index of the first slot
-//                  of its run of equal ids.
-//               2. fill kernel: rows no id selects are written as zeros (the bulk of the traffic).
-//               3. chunk kernel: a run of equal ids is cut into chunks of kChunk slots; one wave sums
-//                  the dy rows of a chunk in fp32 registers, in ascending token position.  A run that
-//                  fits one chunk is rounded and stored straight into dW; longer runs leave one fp32
-//                  partial row per chunk in the workspace.
-//               4. combine kernel: sums the partial rows of each long run and stores the dW row.
+//               1. stable radix sort of (id, position) spread over the GPU (histogram / scan / scatter
+//                  per 9-bit digit), then one workgroup marks which table rows are selected at all
+//                  and records, for every sorted slot, the first slot of its run of equal ids.
+//               2. rows kernel, one launch for two jobs: rows no id selects are written as zeros (the
+//                  bulk of the traffic); a run of equal ids is cut into chunks of kChunk slots and one
+//                  wave sums the dy rows of a chunk in fp32 registers, in ascending token position.  A
+//                  run that fits one chunk is rounded and stored straight into dW; longer runs leave
+//                  one fp32 partial row per chunk in the workspace.
+//               3. combine kernel: sums the partial rows of each long run and stores the dW row.
 //             No floating-point atomics, no zero-fill of rows that are written anyway, deterministic.
 #include "ck_block_sort.h"
+#include "ck_grid_sort.h"
 
 namespace ck {
 
@@ -74,6 +75,7 @@ __global__ void __launch_bounds__(256)
 struct EmbWorkspace {
     uint32_t* keys[2];
     uint32_t* vals[2];
+    uint32_t* hist;      // [bins][waves] of the grid sort
     uint32_t* run_head;  // [n] first sorted slot of the run of equal ids that slot i belongs to
     uint8_t* touched;    // [V] 1 when some id selects the row
     float* partial;      // [2 * ceil(n / kChunk)][H]
@@ -91,6 +93,8 @@ static inline int64_t emb_carve(void* base, int64_t n, int64_t V, int64_t H, Emb
         if (ws) ws->vals[i] = (uint32_t*)(b + off);
         off += arr;
     }
+    if (ws) ws->hist = (uint32_t*)(b + off);
+    off += align_up((int64_t)(1 << kGridSortMaxBits) * grid_sort_waves(n) * 4, 256);
     if (ws) ws->run_head = (uint32_t*)(b + off);
     off += arr;
     if (ws) ws->touched = (uint8_t*)(b + off);
@@ -100,115 +104,147 @@ static inline int64_t emb_carve(void* base, int64_t n, int64_t V, int64_t H, Emb
     return off;
 }
 
+// Sort of the token ids, spread over the GPU (ck_grid_sort.h).  Ids outside [0, V) get the key V: they sort
+// last and are skipped by the later kernels.
 template <bool I32>
-__global__ void __launch_bounds__(kSortThreads)
-    embedding_sort_kernel(const void* __restrict__ ids, EmbWorkspace ws, int n, int64_t V, int key_bits) {
-    __shared__ SortShared sh;
-    __shared__ int wave_last[kSortWaves];
+struct IdLoader {
+    const void* ids;
+    int64_t V;
+    __device__ __forceinline__ void operator()(int i, uint32_t& k, uint32_t& v) const {
+        const int64_t id = load_tok<I32>(ids, i);
+        k = (id < 0 || id >= V) ? (uint32_t)V : (uint32_t)id;
+        v = (uint32_t)i;
+    }
+};
+struct PairLoader {
+    const uint32_t* keys;
+    const uint32_t* vals;
+    __device__ __forceinline__ void operator()(int i, uint32_t& k, uint32_t& v) const {
+        k = keys[i];
+        v = vals[i];
+    }
+};
+struct PairStorer {
+    uint32_t* keys;
+    uint32_t* vals;
+    __device__ __forceinline__ void operator()(int pos, uint32_t k, uint32_t v) const {
+        keys[pos] = k;
+        vals[pos] = v;
+    }
+};
 
-    // clear the row marks (V bytes, padded to a multiple of 256 by the workspace layout)
-    uint32_t* tw = reinterpret_cast<uint32_t*>(ws.touched);
-    for (int64_t i = threadIdx.x; i < (V + 3) / 4; i += kSortThreads) tw[i] = 0u;
+template <typename Loader>
+__global__ void __launch_bounds__(256)
+    embedding_sort_hist_kernel(Loader load, int n, int shift, int bits, uint32_t* __restrict__ hist, int num_waves,
+                               uint32_t* __restrict__ clear, int64_t clear_words) {
+    __shared__ GridSortShared sh;
+    // side job of the first pass: clear the row marks
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < clear_words; i += (int64_t)gridDim.x * blockDim.x)
+        clear[i] = 0u;
+    grid_sort_histogram(sh, n, shift, bits, hist, num_waves, load);
+}
 
-    const int passes = ck_sort_passes(key_bits);
-    const int bits_per_pass = (key_bits + passes - 1) / passes;
-    for (int p = 0; p < passes; ++p) {
-        const int shift = p * bits_per_pass;
-        const int bits = min(bits_per_pass, key_bits - shift);
-        const bool first = p == 0;
-        const uint32_t* kin = ws.keys[(p + 1) & 1];
-        const uint32_t* vin = ws.vals[(p + 1) & 1];
-        uint32_t* kout = ws.keys[p & 1];
-        uint32_t* vout = ws.vals[p & 1];
-        auto load = [&](int i, uint32_t& k, uint32_t& v) {
-            if (first) {
-                const int64_t id = load_tok<I32>(ids, i);
-                k = (id < 0 || id >= V) ? (uint32_t)V : (uint32_t)id;  // invalid ids sort last and are skipped
-                v = (uint32_t)i;
-            } else {
-                k = kin[i];
-                v = vin[i];
+__global__ void __launch_bounds__(1024) embedding_sort_scan_kernel(uint32_t* __restrict__ hist, int total) {
+    grid_sort_scan(hist, total);
+}
+
+template <typename Loader>
+__global__ void __launch_bounds__(256)
+    embedding_sort_scatter_kernel(Loader load, PairStorer store, int n, int shift, int bits,
+                                  const uint32_t* __restrict__ offsets, int num_waves) {
+    __shared__ GridSortShared sh;
+    grid_sort_scatter(sh, n, shift, bits, offsets, num_waves, load, store);
+}
+
+// Runs of equal ids in the sorted order: marks the table rows that are selected at all and records, for every
+// sorted slot, the first slot of its run.  Every wave owns kRunsWaveSlots consecutive slots: it first looks
+// backwards from its first slot, 64 slots at a time, for the head of the run it starts in, then walks its
+// slots 64 at a time carrying the latest head forward with a wave max-scan.
+constexpr int kRunsWaveSlots = 4 * CK_WAVE;
+__global__ void __launch_bounds__(256)
+    embedding_runs_kernel(const uint32_t* __restrict__ skeys, uint32_t* __restrict__ run_head, uint8_t* __restrict__ touched,
+                          int n, int64_t V) {
+    const int lane = lane_id();
+    const int gw = (blockIdx.x * blockDim.x + threadIdx.x) / CK_WAVE;
+    const int begin = gw * kRunsWaveSlots;
+    if (begin >= n) return;
+    const int end = min(begin + kRunsWaveSlots, n);
+    // head of the run that contains slot `begin`: the last slot j <= begin with skeys[j - 1] != skeys[j]
+    int carry = -1;
+    const uint32_t first_key = skeys[begin];
+    for (int hi = begin; carry < 0; hi -= CK_WAVE) {
+        const int j = hi - lane;  // lane 0 looks at hi, lane 63 at hi - 63
+        const bool is_head = j >= 0 && (j == 0 || skeys[j - 1] != first_key);
+        const uint64_t found = __ballot(is_head);
+        if (found != 0) carry = hi - (__ffsll((unsigned long long)found) - 1);
+    }
+    for (int i0 = begin; i0 < end; i0 += CK_WAVE) {
+        const int i = i0 + lane;
+        int head = -1;
+        if (i < end) {
+            const uint32_t k = skeys[i];
+            if (i == 0 || skeys[i - 1] != k) {
+                head = i;
+                if ((int64_t)k < V) touched[k] = 1;
             }
-        };
-        auto store = [&](int pos, uint32_t k, uint32_t v) {
-            kout[pos] = k;
-            vout[pos] = v;
-        };
-        block_radix_pass(sh, n, shift, bits, load, store);
-    }
-    const uint32_t* skeys = ws.keys[(passes - 1) & 1];
-
-    // run heads: each lane owns a contiguous range of sorted slots; the index of the last head at or
-    // before a slot is a running maximum, carried across lanes with a wave scan and across waves in LDS
-    const int per = (n + kSortThreads - 1) / kSortThreads;
-    const int b0 = min((int)threadIdx.x * per, n);
-    const int b1 = min(b0 + per, n);
-    int last = -1;
-    for (int i = b0; i < b1; ++i) {
-        const uint32_t k = skeys[i];
-        if (i == 0 || skeys[i - 1] != k) {
-            last = i;
-            if ((int64_t)k < V) ws.touched[k] = 1;
         }
-    }
-    const int wave = threadIdx.x / CK_WAVE;
-    const int incl = wave_inclusive_max_i(last);
-    if (lane_id() == CK_WAVE - 1) wave_last[wave] = incl;
-    __syncthreads();
-    int carry = __shfl_up(incl, 1, CK_WAVE);
-    if (lane_id() == 0) carry = -1;
-    for (int w = 0; w < wave; ++w) carry = max(carry, wave_last[w]);
-    for (int i = b0; i < b1; ++i) {
-        if (i == 0 || skeys[i - 1] != skeys[i]) carry = i;
-        ws.run_head[i] = (uint32_t)carry;
+        const int incl = max(wave_inclusive_max_i(head), carry);
+        if (i < end) run_head[i] = (uint32_t)incl;
+        carry = __shfl(incl, CK_WAVE - 1, CK_WAVE);
     }
 }
 
-// ---- backward 2: zero rows nobody selects ---------------------------------------------------------
+// ---- backward 2: one launch for the two row-wise jobs ---------------------------------------------
+// Workgroups [0, chunk_groups) sum chunks of runs (two dependent memory round trips per wave: latency-bound);
+// the remaining workgroups write zeros into the rows nobody selects (pure streaming writes, the bulk of the
+// bytes).  Running both in one grid lets the streaming part hide the latency of the other.
+//   chunk job: a run of equal ids is cut into chunks of kChunk slots; one wave sums the dy rows of a chunk in
+//   fp32 (fp64 for fp32 tables) in ascending token position.  A run that fits one chunk is rounded and stored
+//   straight into dW; longer runs leave one fp32 partial row per chunk in the workspace.
 template <typename T, int VEC>
 __global__ void __launch_bounds__(256)
-    embedding_bwd_fill_kernel(const uint8_t* __restrict__ touched, typename T::storage_t* __restrict__ dw, int64_t V,
-                              int64_t H) {
+    embedding_bwd_rows_kernel(const uint32_t* __restrict__ skeys, const uint32_t* __restrict__ spos,
+                              const uint32_t* __restrict__ run_head, const uint8_t* __restrict__ touched,
+                              const typename T::storage_t* __restrict__ dy, typename T::storage_t* __restrict__ dw,
+                              float* __restrict__ partial, int n, int chunk_groups, int64_t V, int64_t H) {
     typedef VPack<T, VEC> P;
-    const int64_t row = (int64_t)blockIdx.x * 4 + threadIdx.x / CK_WAVE;
-    if (row >= V) return;
-    if (touched[row]) return;
-    P z;
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) z.v[j] = T::down(0.f);
-    P* dst = reinterpret_cast<P*>(dw + row * H);
+    const int lane = lane_id();
     const int64_t packs = H / VEC;
-    for (int64_t p = lane_id(); p < packs; p += CK_WAVE) nt_store(z, dst + p);
-}
 
-// ---- backward 3: sum the dy rows of one chunk of a run ----------------------------------------------
-template <typename T, int VEC>
-__global__ void __launch_bounds__(256)
-    embedding_bwd_chunk_kernel(const uint32_t* __restrict__ skeys, const uint32_t* __restrict__ spos,
-                               const uint32_t* __restrict__ run_head, const typename T::storage_t* __restrict__ dy,
-                               typename T::storage_t* __restrict__ dw, float* __restrict__ partial, int n, int64_t V,
-                               int64_t H) {
-    typedef VPack<T, VEC> P;
+    if ((int)blockIdx.x >= chunk_groups) {
+        // ---- zero fill ----
+        const int64_t row = (int64_t)(blockIdx.x - chunk_groups) * 4 + threadIdx.x / CK_WAVE;
+        if (row >= V) return;
+        if (touched[row]) return;
+        P z;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) z.v[j] = T::down(0.f);
+        P* dst = reinterpret_cast<P*>(dw + row * H);
+        for (int64_t p = lane; p < packs; p += CK_WAVE) nt_store(z, dst + p);
+        return;
+    }
+
+    // ---- chunk sums ----
     const int i = blockIdx.x * 4 + threadIdx.x / CK_WAVE;
     if (i >= n) return;
+    // every index load is issued before any of them is used: one round trip
     const uint32_t id = skeys[i];
-    if ((int64_t)id >= V) return;
     const int head = (int)run_head[i];
+    const bool in_range = lane <= kChunk && i + lane < n;
+    const uint32_t key_l = in_range ? skeys[i + lane] : 0xffffffffu;
+    const uint32_t pos_l = (in_range && lane < kChunk) ? spos[i + lane] : 0u;
+    if ((int64_t)id >= V) return;
     if ((i - head) % kChunk != 0) return;
-    const int lane = lane_id();
 
     // slots of this chunk: leading slots i, i+1, ... with the same id, at most kChunk
-    const bool same = lane < kChunk && i + lane < n && skeys[i + lane] == id;
-    const uint64_t bal = __ballot(same);
+    const uint64_t bal = __ballot(lane < kChunk && key_l == id);
     const int cnt = __ffsll((unsigned long long)~bal) - 1;  // lane 0 always matches, so cnt >= 1
-    const bool continues = cnt == kChunk && i + kChunk < n && skeys[i + kChunk] == id;
+    const bool continues = cnt == kChunk && __shfl(key_l, kChunk, CK_WAVE) == id;
     const bool multi = (i != head) || continues;
-    const uint32_t my_pos = lane < cnt ? spos[i + lane] : 0u;
 
-    const int64_t packs = H / VEC;
-    const int64_t tile = (int64_t)CK_WAVE * kRowPacks;
     // fp32 tables sum in fp64 so that the result is the correctly rounded sum whatever the order
     typedef typename AccOf<T>::type acc_t;
+    const int64_t tile = (int64_t)CK_WAVE * kRowPacks;
     for (int64_t p0 = 0; p0 < packs; p0 += tile) {
         acc_t acc[kRowPacks][VEC];
 #pragma unroll
@@ -216,7 +252,7 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
             for (int j = 0; j < VEC; ++j) acc[q][j] = 0;
         for (int r = 0; r < cnt; ++r) {
-            const uint32_t pos = __shfl(my_pos, r, CK_WAVE);
+            const uint32_t pos = __shfl(pos_l, r, CK_WAVE);
             const P* src = reinterpret_cast<const P*>(dy + (int64_t)pos * H);
             P v[kRowPacks];
 #pragma unroll
@@ -269,26 +305,63 @@ __global__ void __launch_bounds__(256)
     }
 }
 
-// ---- backward 4: add up the partial rows of long runs --------------------------------------------
-// One workgroup per sorted slot; only heads of runs longer than kChunk do work.  Lane per column.
+// ---- backward 3: add up the partial rows of long runs ------------------------------------------------
+// Workgroup (g, part) looks at the 64 sorted slots [64 g, 64 g + 64): the slots that head a run longer than kChunk
+// are found with one coalesced look, then the whole workgroup sums, for each of them in turn, the partial rows
+// of the run over its quarter (`part`) of the columns.
+constexpr int kCombineParts = 4;
+
 template <typename T>
 __global__ void __launch_bounds__(256)
     embedding_bwd_combine_kernel(const uint32_t* __restrict__ skeys, const uint32_t* __restrict__ run_head,
                                  const float* __restrict__ partial, typename T::storage_t* __restrict__ dw, int n,
                                  int64_t V, int64_t H) {
-    const int i = blockIdx.x;
-    const uint32_t id = skeys[i];
-    if ((int64_t)id >= V) return;
-    if ((int)run_head[i] != i) return;
-    if (!(i + kChunk < n && skeys[i + kChunk] == id)) return;
-    typedef typename AccOf<T>::type acc_t;
-    for (int64_t c = threadIdx.x; c < H; c += blockDim.x) {
-        acc_t acc = 0;
-        for (int s = i; s < n && skeys[s] == id; s += kChunk) {
-            const int64_t slot = 2 * (int64_t)(s / kChunk) + (s == i ? 1 : 0);
-            acc += (acc_t)partial[slot * H + c];
+    __shared__ unsigned long long sh_hits;
+    if (threadIdx.x < CK_WAVE) {
+        const int i = blockIdx.x * CK_WAVE + threadIdx.x;
+        bool hit = false;
+        if (i < n) {
+            const uint32_t id = skeys[i];
+            hit = (int64_t)id < V && (int)run_head[i] == i && i + kChunk < n && skeys[i + kChunk] == id;
         }
-        dw[(int64_t)id * H + c] = T::down((float)acc);
+        const uint64_t hits = __ballot(hit);
+        if (threadIdx.x == 0) sh_hits = hits;
+    }
+    __syncthreads();
+    uint64_t hits = sh_hits;
+    typedef typename AccOf<T>::type acc_t;
+    const int64_t cols = (H + kCombineParts - 1) / kCombineParts;
+    const int64_t c0 = (int64_t)blockIdx.y * cols;
+    const int64_t c1 = c0 + cols < H ? c0 + cols : H;
+    while (hits != 0) {
+        const int i = blockIdx.x * CK_WAVE + (__ffsll((unsigned long long)hits) - 1);
+        hits &= hits - 1;
+        const uint32_t id = skeys[i];
+        // number of chunks of the run: chunk starts i, i + kChunk, ... that still hold this id
+        int chunks = 0;
+        for (int base = 0;; base += 256) {
+            const int64_t s = (int64_t)i + (int64_t)(base + threadIdx.x) * kChunk;
+            const int c = __syncthreads_count(s < n && skeys[s] == id);
+            chunks += c;
+            if (c < 256) break;
+        }
+        const int64_t first_slot = 2 * (int64_t)(i / kChunk) + 1;
+        for (int64_t c = c0 + threadIdx.x; c < c1; c += 256) {
+            acc_t acc = (acc_t)partial[first_slot * H + c];
+            int k = 1;
+            for (; k + 3 < chunks; k += 4) {
+                const float v0 = partial[2 * (int64_t)((i + k * kChunk) / kChunk) * H + c];
+                const float v1 = partial[2 * (int64_t)((i + (k + 1) * kChunk) / kChunk) * H + c];
+                const float v2 = partial[2 * (int64_t)((i + (k + 2) * kChunk) / kChunk) * H + c];
+                const float v3 = partial[2 * (int64_t)((i + (k + 3) * kChunk) / kChunk) * H + c];
+                acc += (acc_t)v0;
+                acc += (acc_t)v1;
+                acc += (acc_t)v2;
+                acc += (acc_t)v3;
+            }
+            for (; k < chunks; ++k) acc += (acc_t)partial[2 * (int64_t)((i + k * kChunk) / kChunk) * H + c];
+            dw[(int64_t)id * H + c] = T::down((float)acc);
+        }
     }
 }
 
@@ -335,14 +408,13 @@ static void launch_bwd(hipStream_t s, const ck::EmbWorkspace& ws, int passes, co
     typedef typename T::storage_t S;
     const uint32_t* skeys = ws.keys[(passes - 1) & 1];
     const uint32_t* spos = ws.vals[(passes - 1) & 1];
-    hipLaunchKernelGGL((ck::embedding_bwd_fill_kernel<T, VEC>), dim3((unsigned)ck_ceil_div(V, 4)), dim3(256), 0, s,
-                       ws.touched, (S*)dw, V, H);
-    if (n > 0) {
-        hipLaunchKernelGGL((ck::embedding_bwd_chunk_kernel<T, VEC>), dim3((unsigned)ck_ceil_div(n, 4)), dim3(256), 0, s,
-                           skeys, spos, ws.run_head, (const S*)dy, (S*)dw, ws.partial, n, V, H);
-        hipLaunchKernelGGL((ck::embedding_bwd_combine_kernel<T>), dim3((unsigned)n), dim3(256), 0, s, skeys,
-                           ws.run_head, ws.partial, (S*)dw, n, V, H);
-    }
+    const int chunk_groups = (int)ck_ceil_div(n, 4);
+    const int64_t fill_groups = ck_ceil_div(V, 4);
+    hipLaunchKernelGGL((ck::embedding_bwd_rows_kernel<T, VEC>), dim3((unsigned)(chunk_groups + fill_groups)), dim3(256), 0,
+                       s, skeys, spos, ws.run_head, ws.touched, (const S*)dy, (S*)dw, ws.partial, n, chunk_groups, V, H);
+    if (n > 0)
+        hipLaunchKernelGGL((ck::embedding_bwd_combine_kernel<T>), dim3((unsigned)ck_ceil_div(n, CK_WAVE), ck::kCombineParts),
+                           dim3(256), 0, s, skeys, ws.run_head, ws.partial, (S*)dw, n, V, H);
 }
 
 extern "C" int ck_embedding_backward(const void* ids, int ids_are_i32, const void* output_grad, void* weight_grad,
@@ -354,20 +426,53 @@ extern "C" int ck_embedding_backward(const void* ids, int ids_are_i32, const voi
     if (!weight_grad || (num_ids > 0 && (!ids || !output_grad))) return CK_ERR_NULL;
     if (!ck_aligned_elem(weight_grad, dtype) || (output_grad && !ck_aligned_elem(output_grad, dtype)))
         return CK_ERR_ALIGN;
-    if (ck_ceil_div(V, 4) > 0x7fffffff) return CK_ERR_SHAPE;
+    if (ck_ceil_div(V, 4) + ck_ceil_div(num_ids, 4) > 0x7fffffff) return CK_ERR_SHAPE;
     if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return CK_ERR_WORKSPACE;
     if (workspace_bytes < ck_embedding_backward_workspace_size(num_ids, V, H)) return CK_ERR_WORKSPACE;
     hipStream_t s = (hipStream_t)stream;
     ck::EmbWorkspace ws;
     ck::emb_carve(workspace, num_ids, V, H, &ws);
     const int key_bits = ck::ck_key_bits(V + 1);  // one extra key value marks ids outside [0, V)
-    const int passes = ck::ck_sort_passes(key_bits);
-    if (ids_are_i32)
-        hipLaunchKernelGGL(ck::embedding_sort_kernel<true>, dim3(1), dim3(ck::kSortThreads), 0, s, ids, ws,
-                           (int)num_ids, V, key_bits);
-    else
-        hipLaunchKernelGGL(ck::embedding_sort_kernel<false>, dim3(1), dim3(ck::kSortThreads), 0, s, ids, ws,
-                           (int)num_ids, V, key_bits);
+    const int passes = (key_bits + ck::kGridSortMaxBits - 1) / ck::kGridSortMaxBits;
+    const int bits_per_pass = (key_bits + passes - 1) / passes;
+    const int n = (int)num_ids;
+    const int num_waves = ck::grid_sort_waves(n);
+    const unsigned sort_grid = (unsigned)(num_waves > 0 ? ck_ceil_div(num_waves, ck::kGridSortBlockWaves) : 1);
+    const int64_t clear_words = (V + 3) / 4;
+    for (int p = 0; p < passes; ++p) {
+        const int shift = p * bits_per_pass;
+        const int bits = key_bits - shift < bits_per_pass ? key_bits - shift : bits_per_pass;
+        const int total = (1 << bits) * num_waves;
+        ck::PairStorer store = {ws.keys[p & 1], ws.vals[p & 1]};
+        if (p == 0) {
+            // the clear of the row marks rides on the first histogram launch (needs at least one workgroup)
+            if (ids_are_i32) {
+                ck::IdLoader<true> load = {ids, V};
+                hipLaunchKernelGGL((ck::embedding_sort_hist_kernel<ck::IdLoader<true>>), dim3(sort_grid), dim3(256), 0, s,
+                                   load, n, shift, bits, ws.hist, num_waves, (uint32_t*)ws.touched, clear_words);
+                hipLaunchKernelGGL(ck::embedding_sort_scan_kernel, dim3(1), dim3(1024), 0, s, ws.hist, total);
+                hipLaunchKernelGGL((ck::embedding_sort_scatter_kernel<ck::IdLoader<true>>), dim3(sort_grid), dim3(256), 0,
+                                   s, load, store, n, shift, bits, ws.hist, num_waves);
+            } else {
+                ck::IdLoader<false> load = {ids, V};
+                hipLaunchKernelGGL((ck::embedding_sort_hist_kernel<ck::IdLoader<false>>), dim3(sort_grid), dim3(256), 0, s,
+                                   load, n, shift, bits, ws.hist, num_waves, (uint32_t*)ws.touched, clear_words);
+                hipLaunchKernelGGL(ck::embedding_sort_scan_kernel, dim3(1), dim3(1024), 0, s, ws.hist, total);
+                hipLaunchKernelGGL((ck::embedding_sort_scatter_kernel<ck::IdLoader<false>>), dim3(sort_grid), dim3(256), 0,
+                                   s, load, store, n, shift, bits, ws.hist, num_waves);
+            }
+        } else {
+            ck::PairLoader load = {ws.keys[(p + 1) & 1], ws.vals[(p + 1) & 1]};
+            hipLaunchKernelGGL((ck::embedding_sort_hist_kernel<ck::PairLoader>), dim3(sort_grid), dim3(256), 0, s, load, n,
+                               shift, bits, ws.hist, num_waves, (uint32_t*)nullptr, (int64_t)0);
+            hipLaunchKernelGGL(ck::embedding_sort_scan_kernel, dim3(1), dim3(1024), 0, s, ws.hist, total);
+            hipLaunchKernelGGL((ck::embedding_sort_scatter_kernel<ck::PairLoader>), dim3(sort_grid), dim3(256), 0, s, load,
+                               store, n, shift, bits, ws.hist, num_waves);
+        }
+    }
+    if (n > 0)
+        hipLaunchKernelGGL(ck::embedding_runs_kernel, dim3((unsigned)ck_ceil_div(n, 4 * ck::kRunsWaveSlots)), dim3(256), 0,
+                           s, ws.keys[(passes - 1) & 1], ws.run_head, ws.touched, n, V);
     CK_DISPATCH_DTYPE(dtype, {
         const bool vec = ck_aligned16(weight_grad) && (!output_grad || ck_aligned16(output_grad)) && (H % T::kVec == 0);
         if (vec) launch_bwd<T, T::kVec>(s, ws, passes, output_grad, weight_grad, (int)num_ids, V, H);

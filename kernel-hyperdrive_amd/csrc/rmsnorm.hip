@@ -33,59 +33,97 @@ __device__ __forceinline__ float team_sum(float v, float* red) {
     return v;
 }
 
+// Registers: the row stays packed in its storage type (8 packets = 32 VGPRs for a 16-bit row of 4096) and is
+// widened to fp32 element by element where it is used; the bound of two waves per SIMD keeps the compiler from
+// hoisting the widened copies (which would leave one wave per SIMD and nothing to hide latency with).
+// Makes the compiler forget what it knows about a packed register set: values widened from it before this
+// point cannot be kept alive in place of the packed form.
+template <typename P>
+__device__ __forceinline__ void forget(P& p) {
+    static_assert(sizeof(P) % 4 == 0, "whole registers");
+    uint32_t* w = reinterpret_cast<uint32_t*>(&p);
+#pragma unroll
+    for (int i = 0; i < (int)(sizeof(P) / 4); ++i) asm volatile("" : "+v"(w[i]));
+}
+
+#define CK_RMS_BOUNDS(TPR) __launch_bounds__((TPR) > 256 ? (TPR) : 256, (TPR) > 256 ? 1 : 2)
+
 template <typename T, int TPR>
-__global__ void __launch_bounds__(TPR > 256 ? TPR : 256)
+__global__ void CK_RMS_BOUNDS(TPR)
     rmsnorm_fwd_kernel(const typename T::storage_t* __restrict__ x, const typename T::storage_t* __restrict__ w,
                        typename T::storage_t* __restrict__ y, float* __restrict__ rstd_out, int64_t B, int H,
                        float eps) {
     typedef VPack<T, T::kVec> P;
     __shared__ float red[16];
     const int teams_per_block = blockDim.x / TPR;
-    const int team = threadIdx.x / TPR;
+    const int team = blockIdx.x * teams_per_block + threadIdx.x / TPR;
+    const int num_teams = gridDim.x * teams_per_block;
     const int t = threadIdx.x % TPR;
-    const int64_t row = (int64_t)blockIdx.x * teams_per_block + team;
     const int packs = H / T::kVec;
-    // with TPR > 64 the whole block is one team, so `row < B` is uniform across the barriers below
-    if (row >= B) return;
+    const float inv_h = 1.0f / (float)H;
 
-    const P* xr = reinterpret_cast<const P*>(x + row * H);
-    P xv[kMaxPacks];
-    float ss = 0.f;
+    // rows are dealt round-robin; the next row is requested before the current one is reduced.
+    // With TPR > 64 the block is one team, so the trip count is uniform across the barriers in team_sum.
+    P cur[kMaxPacks], nxt[kMaxPacks];
+    int64_t row = team;
+    if (row < B) {
+        const P* xr = reinterpret_cast<const P*>(x + row * H);
 #pragma unroll
-    for (int i = 0; i < kMaxPacks; ++i) {
-        const int p = t + i * TPR;
-        if (p < packs) {
-            xv[i] = nt_load(xr + p);
-#pragma unroll
-            for (int j = 0; j < T::kVec; ++j) {
-                const float f = T::up(xv[i].v[j]);
-                ss += f * f;
-            }
+        for (int i = 0; i < kMaxPacks; ++i) {
+            const int p = t + i * TPR;
+            if (p < packs) cur[i] = nt_load(xr + p);
         }
     }
-    ss = team_sum<TPR>(ss, red);
-    const float rstd = rsqrtf(ss / (float)H + eps);
-    if (rstd_out != nullptr && t == 0) rstd_out[row] = rstd;
-
-    P* yr = reinterpret_cast<P*>(y + row * H);
+    for (; row < B; row += num_teams) {
+        const int64_t next_row = row + num_teams;
+        if (next_row < B) {
+            const P* xr = reinterpret_cast<const P*>(x + next_row * H);
 #pragma unroll
-    for (int i = 0; i < kMaxPacks; ++i) {
-        const int p = t + i * TPR;
-        if (p < packs) {
-            P o;
-            if (w != nullptr) {
-                const P wv = reinterpret_cast<const P*>(w)[p];
-#pragma unroll
-                for (int j = 0; j < T::kVec; ++j) o.v[j] = T::down(T::up(xv[i].v[j]) * rstd * T::up(wv.v[j]));
-            } else {
-#pragma unroll
-                for (int j = 0; j < T::kVec; ++j) o.v[j] = T::down(T::up(xv[i].v[j]) * rstd);
+            for (int i = 0; i < kMaxPacks; ++i) {
+                const int p = t + i * TPR;
+                if (p < packs) nxt[i] = nt_load(xr + p);
             }
-            nt_store(o, yr + p);
         }
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < kMaxPacks; ++i) {
+            const int p = t + i * TPR;
+            if (p < packs) {
+#pragma unroll
+                for (int j = 0; j < T::kVec; ++j) {
+                    const float f = T::up(cur[i].v[j]);
+                    ss += f * f;
+                }
+            }
+        }
+        ss = team_sum<TPR>(ss, red);
+        const float rstd = rsqrtf(ss * inv_h + eps);
+        if (rstd_out != nullptr && t == 0) rstd_out[row] = rstd;
+
+        P* yr = reinterpret_cast<P*>(y + row * H);
+#pragma unroll
+        for (int i = 0; i < kMaxPacks; ++i) {
+            const int p = t + i * TPR;
+            if (p < packs) {
+                P o;
+                if (w != nullptr) {
+                    const P wv = reinterpret_cast<const P*>(w)[p];
+#pragma unroll
+                    for (int j = 0; j < T::kVec; ++j) o.v[j] = T::down(T::up(cur[i].v[j]) * rstd * T::up(wv.v[j]));
+                } else {
+#pragma unroll
+                    for (int j = 0; j < T::kVec; ++j) o.v[j] = T::down(T::up(cur[i].v[j]) * rstd);
+                }
+                nt_store(o, yr + p);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kMaxPacks; ++i) cur[i] = nxt[i];
     }
 }
 
+// Backward: one wave per SIMD with the whole register file (packed current row and next row of x and dy, packed
+// weight, 64 fp32 dweight accumulators); the next row's loads are in flight while the current row is reduced.
 template <typename T, int TPR, bool HAS_W>
 __global__ void __launch_bounds__(TPR > 256 ? TPR : 256)
     rmsnorm_bwd_kernel(const typename T::storage_t* __restrict__ x, const typename T::storage_t* __restrict__ w,
@@ -114,16 +152,45 @@ __global__ void __launch_bounds__(TPR > 256 ? TPR : 256)
     }
 
     // rows are dealt round-robin; with TPR > 64 the block is one team so the trip count is block-uniform
-    for (int64_t row = team; row < B; row += num_teams) {
-        const P* xr = reinterpret_cast<const P*>(x + row * H);
-        const P* gr = reinterpret_cast<const P*>(dy + row * H);
-        P xv[kMaxPacks], gv[kMaxPacks];
+    constexpr bool PREFETCH = TPR <= 256;  // the 1024-lane variant has 128 registers per lane: no room
+    P xv[kMaxPacks], gv[kMaxPacks], xn[kMaxPacks], gn[kMaxPacks];
+    if (PREFETCH && team < B) {
+        const P* xr = reinterpret_cast<const P*>(x + (int64_t)team * H);
+        const P* gr = reinterpret_cast<const P*>(dy + (int64_t)team * H);
 #pragma unroll
         for (int i = 0; i < kMaxPacks; ++i) {
             const int p = t + i * TPR;
             if (p < packs) {
                 xv[i] = nt_load(xr + p);
                 gv[i] = nt_load(gr + p);
+            }
+        }
+    }
+    for (int64_t row = team; row < B; row += num_teams) {
+        if (PREFETCH) {
+            const int64_t next_row = row + num_teams;
+            if (next_row < B) {
+                const P* xr = reinterpret_cast<const P*>(x + next_row * H);
+                const P* gr = reinterpret_cast<const P*>(dy + next_row * H);
+#pragma unroll
+                for (int i = 0; i < kMaxPacks; ++i) {
+                    const int p = t + i * TPR;
+                    if (p < packs) {
+                        xn[i] = nt_load(xr + p);
+                        gn[i] = nt_load(gr + p);
+                    }
+                }
+            }
+        } else {
+            const P* xr = reinterpret_cast<const P*>(x + row * H);
+            const P* gr = reinterpret_cast<const P*>(dy + row * H);
+#pragma unroll
+            for (int i = 0; i < kMaxPacks; ++i) {
+                const int p = t + i * TPR;
+                if (p < packs) {
+                    xv[i] = nt_load(xr + p);
+                    gv[i] = nt_load(gr + p);
+                }
             }
         }
         float ss = 0.f, dot = 0.f;
@@ -139,6 +206,16 @@ __global__ void __launch_bounds__(TPR > 256 ? TPR : 256)
                     ss += xf * xf;
                     dot += g * xf;
                 }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (sizeof(typename T::storage_t) == 2) {
+            // 16-bit rows: keep only the packed form across the reductions
+#pragma unroll
+            for (int i = 0; i < kMaxPacks; ++i) {
+                forget(xv[i]);
+                forget(gv[i]);
+                if (HAS_W) forget(wv[i]);
             }
         }
         float rstd;
@@ -170,6 +247,15 @@ __global__ void __launch_bounds__(TPR > 256 ? TPR : 256)
                 }
                 nt_store(o, dr + p);
             }
+            // one packet at a time: keeps the widened values of later packets from piling up in registers
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (PREFETCH) {
+#pragma unroll
+            for (int i = 0; i < kMaxPacks; ++i) {
+                xv[i] = xn[i];
+                gv[i] = gn[i];
+            }
         }
     }
 
@@ -192,17 +278,22 @@ __global__ void __launch_bounds__(TPR > 256 ? TPR : 256)
 // dweight[j] = sum over `parts` partial rows of partial[r][j].  One wave per block owns 16 columns:
 // lane = 16 row-groups x 4 column-quads; each lane strides over the partial rows with float4 loads,
 // then the 16 row-groups are folded with shuffles.  Requires H % 4 == 0.
+// With gridDim.y > 1 the partial rows are split over blockIdx.y and the result goes, still in fp32, to
+// `out32` ([gridDim.y][H]); a second launch with gridDim.y == 1 then folds those rows into `dw`.
 template <typename T>
 __global__ void __launch_bounds__(64)
-    rmsnorm_dw_reduce_kernel(const float* __restrict__ partial, typename T::storage_t* __restrict__ dw, int parts,
-                             int H) {
+    rmsnorm_dw_reduce_kernel(const float* __restrict__ partial, typename T::storage_t* __restrict__ dw,
+                             float* __restrict__ out32, int parts, int H) {
     const int lane = threadIdx.x;
     const int quad = lane & 3;
     const int group = lane >> 2;
     const int col = blockIdx.x * 16 + quad * 4;
+    const int per_split = (parts + gridDim.y - 1) / gridDim.y;
+    const int r0 = blockIdx.y * per_split;
+    const int r1 = min(r0 + per_split, parts);
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
     if (col < H) {
-        for (int r = group; r < parts; r += 16) {
+        for (int r = r0 + group; r < r1; r += 16) {
             const float4 v = *reinterpret_cast<const float4*>(partial + (int64_t)r * H + col);
             acc.x += v.x;
             acc.y += v.y;
@@ -218,10 +309,14 @@ __global__ void __launch_bounds__(64)
         acc.w += __shfl_xor(acc.w, off, CK_WAVE);
     }
     if (group == 0 && col < H) {
-        dw[col + 0] = T::down(acc.x);
-        dw[col + 1] = T::down(acc.y);
-        dw[col + 2] = T::down(acc.z);
-        dw[col + 3] = T::down(acc.w);
+        if (out32 != nullptr) {
+            *reinterpret_cast<float4*>(out32 + (int64_t)blockIdx.y * H + col) = acc;
+        } else {
+            dw[col + 0] = T::down(acc.x);
+            dw[col + 1] = T::down(acc.y);
+            dw[col + 2] = T::down(acc.z);
+            dw[col + 3] = T::down(acc.w);
+        }
     }
 }
 
@@ -329,6 +424,8 @@ __global__ void __launch_bounds__(256)
 }  // namespace ck
 
 // ---- host side ------------------------------------------------------------------------------
+constexpr int kReduceSplits = 16;  // row splits of the first dweight reduction pass
+
 static int cu_count() {
     static int cached[64] = {0};
     int dev = 0;
@@ -356,7 +453,7 @@ static int fast_tpr(int64_t H, int dtype) {
 static int bwd_teams(int64_t B, int tpr) {
     const int block = tpr > 256 ? tpr : 256;
     const int teams_per_block = block / tpr;
-    int64_t blocks = (int64_t)cu_count() * (tpr == 1024 ? 1 : 2);
+    int64_t blocks = (int64_t)cu_count();  // one workgroup per CU: the kernel uses the whole register file
     const int64_t need = ck_ceil_div(B, teams_per_block);
     if (blocks > need) blocks = need;
     if (blocks < 1) blocks = 1;
@@ -376,13 +473,20 @@ extern "C" int ck_rmsnorm_forward(const void* x, const void* weight, void* outpu
     CK_DISPATCH_DTYPE(dtype, {
         typedef typename T::storage_t S;
         if (tpr == 64) {
-            hipLaunchKernelGGL((ck::rmsnorm_fwd_kernel<T, 64>), dim3((unsigned)ck_ceil_div(B, 4)), dim3(256), 0, s,
-                               (const S*)x, (const S*)weight, (S*)output, rstd, B, (int)H, eps);
+            // persistent: a few workgroups per CU, each wave walking rows with the next row in flight
+            int64_t grid = (int64_t)cu_count() * 4;
+            if (grid > ck_ceil_div(B, 4)) grid = ck_ceil_div(B, 4);
+            hipLaunchKernelGGL((ck::rmsnorm_fwd_kernel<T, 64>), dim3((unsigned)grid), dim3(256), 0, s, (const S*)x,
+                               (const S*)weight, (S*)output, rstd, B, (int)H, eps);
         } else if (tpr == 256) {
-            hipLaunchKernelGGL((ck::rmsnorm_fwd_kernel<T, 256>), dim3((unsigned)B), dim3(256), 0, s, (const S*)x,
+            int64_t grid = (int64_t)cu_count() * 4;
+            if (grid > B) grid = B;
+            hipLaunchKernelGGL((ck::rmsnorm_fwd_kernel<T, 256>), dim3((unsigned)grid), dim3(256), 0, s, (const S*)x,
                                (const S*)weight, (S*)output, rstd, B, (int)H, eps);
         } else if (tpr == 1024) {
-            hipLaunchKernelGGL((ck::rmsnorm_fwd_kernel<T, 1024>), dim3((unsigned)B), dim3(1024), 0, s, (const S*)x,
+            int64_t grid = (int64_t)cu_count() * 2;
+            if (grid > B) grid = B;
+            hipLaunchKernelGGL((ck::rmsnorm_fwd_kernel<T, 1024>), dim3((unsigned)grid), dim3(1024), 0, s, (const S*)x,
                                (const S*)weight, (S*)output, rstd, B, (int)H, eps);
         } else {
             const int64_t grid = B < 65536 ? B : 65536;
@@ -404,7 +508,7 @@ extern "C" int64_t ck_rmsnorm_backward_workspace_size(int64_t B, int64_t H) {
         const int64_t t = bwd_teams(B, tpr);
         if (t > teams) teams = t;
     }
-    const int64_t fast = teams * H * 4;
+    const int64_t fast = (teams + kReduceSplits) * H * 4;
     const int64_t generic = (B + 3) / 4 * 16 + (int64_t)ck::kColSegments * padded_h(H) * 4;
     return fast > generic ? fast : generic;
 }
@@ -458,9 +562,20 @@ extern "C" int ck_rmsnorm_backward(const void* x, const void* weight, const void
             if (tpr == 64) launch_bwd<T, 64>(grid, block, s, x, weight, output_grad, rstd, x_grad, ws, B, (int)H, eps);
             else if (tpr == 256) launch_bwd<T, 256>(grid, block, s, x, weight, output_grad, rstd, x_grad, ws, B, (int)H, eps);
             else launch_bwd<T, 1024>(grid, block, s, x, weight, output_grad, rstd, x_grad, ws, B, (int)H, eps);
-            if (weight)
-                hipLaunchKernelGGL((ck::rmsnorm_dw_reduce_kernel<T>), dim3((unsigned)ck_ceil_div(H, 16)), dim3(64), 0, s,
-                                   ws, (S*)weight_grad, teams, (int)H);
+            if (weight) {
+                // teams partial rows -> kReduceSplits rows (fp32, behind the partial rows) -> dweight
+                const int splits = teams >= 4 * kReduceSplits ? kReduceSplits : 1;
+                float* second = ws + (int64_t)teams * H;
+                if (splits > 1) {
+                    hipLaunchKernelGGL((ck::rmsnorm_dw_reduce_kernel<T>), dim3((unsigned)ck_ceil_div(H, 16), splits),
+                                       dim3(64), 0, s, ws, (S*)nullptr, second, teams, (int)H);
+                    hipLaunchKernelGGL((ck::rmsnorm_dw_reduce_kernel<T>), dim3((unsigned)ck_ceil_div(H, 16), 1), dim3(64),
+                                       0, s, second, (S*)weight_grad, (float*)nullptr, splits, (int)H);
+                } else {
+                    hipLaunchKernelGGL((ck::rmsnorm_dw_reduce_kernel<T>), dim3((unsigned)ck_ceil_div(H, 16), 1), dim3(64),
+                                       0, s, ws, (S*)weight_grad, (float*)nullptr, teams, (int)H);
+                }
+            }
         } else {
             const int64_t grid = B < 65536 ? B : 65536;
             float* rstd_ws = weight ? ws : nullptr;
