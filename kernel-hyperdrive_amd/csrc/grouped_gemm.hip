@@ -11,8 +11,6 @@
 // never mixes rows of two experts (the reference lets a 128-row block straddle experts and repeats the
 // product once per expert present in it).  fp32, and shapes whose contiguous dimensions are not
 // multiples of 8 elements, go through a plain kernel with exact (fp64) accumulation.
-#include <cstdlib>
-
 #include "ck_device.h"
 
 namespace ck {
@@ -46,7 +44,7 @@ struct GemmParams {
     int M, N, K, E;          // S2S: slots, N, K.  XTY: rows, J (= N), I (= K)
     int fan_out, x_grouped, y_grouped;
     int m_tiles, n_tiles;    // S2S: upper bound of row tiles; XTY: tiles along I
-    int debug;
+    int wide;                // operands too large for 32-bit byte offsets inside a tile's source
 };
 
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -295,7 +293,7 @@ __global__ void __launch_bounds__(TL::THREADS) grouped_gemm_kernel(GemmParams p)
     __syncthreads();
     for (int kt = 0; kt < k_tiles; ++kt) {
         const int buf = kt & 1;
-        if (kt + 1 < k_tiles && !(p.debug & 1)) load_tiles(k_begin + (kt + 1) * BK);
+        if (kt + 1 < k_tiles) load_tiles(k_begin + (kt + 1) * BK);
         const S* At = lds + buf * STAGE_ELEMS;
         const S* Bt = At + ATile::ELEMS;
 #pragma unroll
@@ -310,9 +308,9 @@ __global__ void __launch_bounds__(TL::THREADS) grouped_gemm_kernel(GemmParams p)
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int j = 0; j < TN; ++j) if (!(p.debug & 2)) acc[i][j] = Mma<T>::mma(af[i], bf[j], acc[i][j]);
+                for (int j = 0; j < TN; ++j) acc[i][j] = Mma<T>::mma(af[i], bf[j], acc[i][j]);
         }
-        if (kt + 1 < k_tiles && !(p.debug & 4)) store_tiles(buf ^ 1);
+        if (kt + 1 < k_tiles) store_tiles(buf ^ 1);
         __syncthreads();
     }
 
@@ -367,6 +365,12 @@ __global__ void __launch_bounds__(TL::THREADS) grouped_gemm_kernel(GemmParams p)
 // LDS positions whose contraction index lies beyond the end of the contraction range are cleared with a
 // plain store in the (single) partial step; positions of rows / columns outside the problem keep whatever
 // they held, which only reaches outputs that are never stored.
+#ifndef CK_DTL_PART_A
+#define CK_DTL_PART_A 4
+#endif
+#ifndef CK_DTL_PART_B
+#define CK_DTL_PART_B 8
+#endif
 template <typename S, int ROWS, bool KC, int NWAVES>
 struct DtlOperand {
     static constexpr int BK = 64;
@@ -383,6 +387,13 @@ struct DtlOperand {
         chunk = KC ? (slot ^ ((line >> 1) & 7)) : (slot ^ ((line & 3) << 2));
     }
 };
+
+// Hides how a value was computed from the optimiser, which then cannot move the arithmetic that follows out
+// of the loop and keep every variant of it alive in a register of its own.
+__device__ __forceinline__ int opaque(int v) {
+    asm volatile("" : "+v"(v));
+    return v;
+}
 
 template <typename T, typename TL, bool B_KC, bool GROUP_K>
 __global__ void __launch_bounds__(TL::THREADS) grouped_gemm_dtl_kernel(GemmParams p) {
@@ -410,16 +421,15 @@ __global__ void __launch_bounds__(TL::THREADS) grouped_gemm_dtl_kernel(GemmParam
     if (!logical_tile(p.m_tiles, p.n_tiles, mt, nt)) return;
 
     const int tid = threadIdx.x;
-    const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane(tid / CK_WAVE);
     const int wm = wave / WN, wn = wave % WN;
 
     int expert, row_start, rows_valid, k_begin, k_end, i_base;
     if (!GROUP_K) {
         find_tile<BM>(p.offsets, p.E, mt, sh_info);
-        expert = sh_info[0];
-        row_start = sh_info[1];
-        rows_valid = sh_info[2];
+        expert = __builtin_amdgcn_readfirstlane(sh_info[0]);
+        row_start = __builtin_amdgcn_readfirstlane(sh_info[1]);
+        rows_valid = __builtin_amdgcn_readfirstlane(sh_info[2]);
         if (expert < 0) return;
         k_begin = 0;
         k_end = p.K;
@@ -436,143 +446,166 @@ __global__ void __launch_bounds__(TL::THREADS) grouped_gemm_dtl_kernel(GemmParam
     const int n_base = nt * BN;
     const int cols_valid = min(BN, p.N - n_base);  // > 0 and a multiple of 8
 
-    // ---- per-lane sources of the LDS slots this lane fills ----------------------------------------
-    // Lines / chunks outside the problem are redirected to a valid one (their LDS content is never used for a
-    // stored output), so full steps need no predicate at all.
-    const S* Abase = reinterpret_cast<const S*>(p.A);
-    const S* Bbase = reinterpret_cast<const S*>(p.B) + (GROUP_K ? 0 : (int64_t)expert * p.b_stride_e);
-    const S* a_ptr[AOp::IPW];
-    int a_k[AOp::IPW];  // contraction offset of the slot inside a step
-    const S* b_ptr[BOp::IPW];
-    int b_k[BOp::IPW];
-#pragma unroll
-    for (int j = 0; j < AOp::IPW; ++j) {
-        int line, chunk;
-        AOp::slot_source((wave * AOp::IPW + j) * CK_WAVE + lane, line, chunk);
-        if (A_KC) {
-            const int r = min(line, rows_valid - 1);
-            const int64_t slot = row_start + r;
-            const int64_t src_row = p.x_grouped ? slot : (int64_t)((uint32_t)p.row_idx[slot] / (uint32_t)p.fan_out);
-            a_k[j] = chunk * 8;
-            a_ptr[j] = Abase + src_row * p.lda + k_begin + a_k[j];
-        } else {
-            const int cc = (chunk * 8 < rows_valid) ? chunk * 8 : 0;
-            a_k[j] = line;
-            a_ptr[j] = Abase + (int64_t)(k_begin + line) * p.lda + i_base + cc;
-        }
-    }
-#pragma unroll
-    for (int j = 0; j < BOp::IPW; ++j) {
-        int line, chunk;
-        BOp::slot_source((wave * BOp::IPW + j) * CK_WAVE + lane, line, chunk);
-        if (B_KCC) {
-            const int r = min(line, cols_valid - 1);
-            b_k[j] = chunk * 8;
-            b_ptr[j] = Bbase + (int64_t)(n_base + r) * p.ldb + k_begin + b_k[j];
-        } else {
-            const int cc = (chunk * 8 < cols_valid) ? chunk * 8 : 0;
-            b_k[j] = line;
-            b_ptr[j] = Bbase + (int64_t)(k_begin + line) * p.ldb + n_base + cc;
-        }
-    }
-    const int64_t a_step = (p.debug & 2) ? 0 : (A_KC ? BK : (int64_t)BK * p.lda);
-    const int64_t b_step = (p.debug & 2) ? 0 : (B_KCC ? BK : (int64_t)BK * p.ldb);
-
+    // ---- global sources of the LDS slots this lane fills ---------------------------------------------
+    // address = wave-uniform base of the tile (scalar registers, advanced by a fixed step per tile) + a 32-bit
+    // byte offset per lane and copy instruction.  Lines / chunks outside the problem are redirected to a valid
+    // one (their LDS content never reaches a stored output), so tiles inside the contraction range need no
+    // predicate at all.
+    typedef __attribute__((address_space(1))) const char* gchar_t;
     typedef __attribute__((address_space(1))) const void* gptr_t;
     typedef __attribute__((address_space(3))) void* lptr_t;
-    // request tile `kt` into stage buffer `st`; slots past the end of the contraction are cleared instead
-    auto issue = [&](int kt, char* st) {
-        const int k0 = k_begin + kt * BK;
+    const gchar_t a_base = (gchar_t)p.A + (A_KC ? (int64_t)k_begin : (int64_t)k_begin * p.lda + i_base) * 2;
+    const gchar_t b_base = (gchar_t)p.B + ((GROUP_K ? 0 : (int64_t)expert * p.b_stride_e) +
+                                          (B_KCC ? (int64_t)k_begin : (int64_t)k_begin * p.ldb + n_base)) * 2;
+    const int64_t a_step = (A_KC ? (int64_t)BK : (int64_t)BK * p.lda) * 2;
+    const int64_t b_step = (B_KCC ? (int64_t)BK : (int64_t)BK * p.ldb) * 2;
+    uint32_t a_voff[AOp::IPW], b_voff[BOp::IPW];
+    {
+        const int lane = lane_id();
+#pragma unroll
+        for (int j = 0; j < AOp::IPW; ++j) {
+            int line, chunk;
+            AOp::slot_source((wave * AOp::IPW + j) * CK_WAVE + lane, line, chunk);
+            if (A_KC) {
+                const int64_t slot = row_start + min(line, rows_valid - 1);
+                const int64_t src_row = p.x_grouped ? slot : (int64_t)((uint32_t)p.row_idx[slot] / (uint32_t)p.fan_out);
+                a_voff[j] = (uint32_t)((src_row * p.lda + chunk * 8) * 2);
+            } else {
+                const int cc = (chunk * 8 < rows_valid) ? chunk * 8 : 0;
+                a_voff[j] = (uint32_t)(((int64_t)line * p.lda + cc) * 2);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < BOp::IPW; ++j) {
+            int line, chunk;
+            BOp::slot_source((wave * BOp::IPW + j) * CK_WAVE + lane, line, chunk);
+            if (B_KCC) {
+                const int r = min(line, cols_valid - 1);
+                b_voff[j] = (uint32_t)(((int64_t)(n_base + r) * p.ldb + chunk * 8) * 2);
+            } else {
+                const int cc = (chunk * 8 < cols_valid) ? chunk * 8 : 0;
+                b_voff[j] = (uint32_t)(((int64_t)line * p.ldb + cc) * 2);
+            }
+        }
+    }
+
+    constexpr int LOADS = AOp::IPW + BOp::IPW;  // copy instructions per wave per tile, A first
+    // copy instructions [j0, j1) of tile t, which lies completely inside the contraction range
+    auto issue_range = [&](char* st, int j0, int j1, int t) {
+        const gchar_t at = a_base + (int64_t)t * a_step;
+        const gchar_t bt = b_base + (int64_t)t * b_step;
+#pragma unroll
+        for (int j = 0; j < LOADS; ++j) {
+            if (j < j0 || j >= j1) continue;
+            if (j < AOp::IPW) {
+                __builtin_amdgcn_global_load_lds((gptr_t)(at + a_voff[j]), (lptr_t)(st + (wave * AOp::IPW + j) * 1024), 16, 0, 0);
+            } else {
+                const int jb = j - AOp::IPW;
+                __builtin_amdgcn_global_load_lds((gptr_t)(bt + b_voff[jb]),
+                                                 (lptr_t)(st + AOp::STAGE_BYTES + (wave * BOp::IPW + jb) * 1024), 16, 0, 0);
+            }
+        }
+    };
+    // tile t whatever its position: slots past the end of the contraction range are cleared instead of copied
+    auto issue = [&](int t, char* st) {
+        const int k0 = k_begin + t * BK;
         if (k0 + BK <= k_end) {
+            issue_range(st, 0, LOADS, t);
+            return;
+        }
+        const gchar_t at = a_base + (int64_t)t * a_step;
+        const gchar_t bt = b_base + (int64_t)t * b_step;
+        const int lane = opaque(lane_id());
+        const u32x4_t zero = {0u, 0u, 0u, 0u};
 #pragma unroll
-            for (int j = 0; j < AOp::IPW; ++j) {
-                __builtin_amdgcn_global_load_lds((gptr_t)a_ptr[j], (lptr_t)(st + (wave * AOp::IPW + j) * 1024), 16, 0, 0);
-                a_ptr[j] += a_step;
-            }
+        for (int j = 0; j < AOp::IPW; ++j) {
+            int line, chunk;
+            AOp::slot_source((wave * AOp::IPW + j) * CK_WAVE + lane, line, chunk);
+            char* dst = st + (wave * AOp::IPW + j) * 1024;
+            if (k0 + (A_KC ? chunk * 8 : line) < k_end)
+                __builtin_amdgcn_global_load_lds((gptr_t)(at + a_voff[j]), (lptr_t)dst, 16, 0, 0);
+            else
+                *reinterpret_cast<u32x4_t*>(dst + lane * 16) = zero;
+        }
 #pragma unroll
-            for (int j = 0; j < BOp::IPW; ++j) {
-                __builtin_amdgcn_global_load_lds(
-                    (gptr_t)b_ptr[j], (lptr_t)(st + AOp::STAGE_BYTES + (wave * BOp::IPW + j) * 1024), 16, 0, 0);
-                b_ptr[j] += b_step;
-            }
-        } else {
-            const u32x4_t zero = {0u, 0u, 0u, 0u};
-#pragma unroll
-            for (int j = 0; j < AOp::IPW; ++j) {
-                char* dst = st + (wave * AOp::IPW + j) * 1024;
-                if (k0 + a_k[j] < k_end)
-                    __builtin_amdgcn_global_load_lds((gptr_t)a_ptr[j], (lptr_t)dst, 16, 0, 0);
-                else
-                    *reinterpret_cast<u32x4_t*>(dst + lane * 16) = zero;
-            }
-#pragma unroll
-            for (int j = 0; j < BOp::IPW; ++j) {
-                char* dst = st + AOp::STAGE_BYTES + (wave * BOp::IPW + j) * 1024;
-                if (k0 + b_k[j] < k_end)
-                    __builtin_amdgcn_global_load_lds((gptr_t)b_ptr[j], (lptr_t)dst, 16, 0, 0);
-                else
-                    *reinterpret_cast<u32x4_t*>(dst + lane * 16) = zero;
-            }
+        for (int j = 0; j < BOp::IPW; ++j) {
+            int line, chunk;
+            BOp::slot_source((wave * BOp::IPW + j) * CK_WAVE + lane, line, chunk);
+            char* dst = st + AOp::STAGE_BYTES + (wave * BOp::IPW + j) * 1024;
+            if (k0 + (B_KCC ? chunk * 8 : line) < k_end)
+                __builtin_amdgcn_global_load_lds((gptr_t)(bt + b_voff[j]), (lptr_t)dst, 16, 0, 0);
+            else
+                *reinterpret_cast<u32x4_t*>(dst + lane * 16) = zero;
         }
     };
 
-    // ---- per-lane fragment addresses (bytes inside an operand stage) ---------------------------------
-    int a_off[TM], a_xor[TM], b_off[TN], b_xor[TN];
+    // ---- fragment addresses (bytes inside a stage) -----------------------------------------------------
+    // k-contiguous operand: row r of the tile starts at r * 128; the 16-byte chunk c of that row sits in slot
+    //   c ^ ((r >> 1) & 7).  A lane reads chunk kk / 8 + lane / 32 of row (lane % 32) + 32 * i: the swizzle term
+    //   depends on the lane only, and kk / 8 is even, so the slot is (lane-dependent part) ^ (kk / 8).
+    // other layout: see OperandTile; one address per 32-wide block, the contraction index adds a multiple of the
+    //   line size.
+    int frag_row, frag_swz;
+    int a_off[TM], b_off[TN];
+    {
+        const int lane = lane_id();
+        frag_row = (lane % 32) * 128;
+        frag_swz = ((lane / 32) ^ (((lane % 32) >> 1) & 7)) << 4;
+        const int g = lane / 16, q = lane % 16;
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-        const int r0 = wm * (BM / WM) + i * 32;
-        if (A_KC) {
-            const int r = r0 + lane % 32;
-            a_off[i] = r * 128;
-            a_xor[i] = ((lane / 32) ^ ((r >> 1) & 7)) << 4;  // chunk (kk / 8 + lane / 32) ^ swizzle, kk / 8 even
-        } else {
-            const int g = lane / 16, q = lane % 16;
-            const int col = r0 + (g % 2) * 16 + (q % 4) * 4;
-            a_off[i] = ((g / 2) * 8 + q / 4) * (BM * 2) + ((((col / 8) ^ ((q / 4) << 2))) << 4) + (col % 8) * 2;
-            a_xor[i] = 0;
+        for (int i = 0; i < TM; ++i) {
+            const int r0 = wm * (BM / WM) + i * 32;
+            if (A_KC) {
+                a_off[i] = r0 * 128;
+            } else {
+                const int col = r0 + (g % 2) * 16 + (q % 4) * 4;
+                a_off[i] = ((g / 2) * 8 + q / 4) * (BM * 2) + ((((col / 8) ^ ((q / 4) << 2))) << 4) + (col % 8) * 2;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int c0 = wn * (BN / WN) + j * 32;
+            if (B_KCC) {
+                b_off[j] = AOp::STAGE_BYTES + c0 * 128;
+            } else {
+                const int col = c0 + (g % 2) * 16 + (q % 4) * 4;
+                b_off[j] = AOp::STAGE_BYTES + ((g / 2) * 8 + q / 4) * (BN * 2) + ((((col / 8) ^ ((q / 4) << 2))) << 4) +
+                           (col % 8) * 2;
+            }
         }
     }
+    auto read_frags = [&](const char* st, int kk, frag_t* af, frag_t* bf) {
+        // position of this lane's chunk in a k-contiguous row, recomputed here on purpose
+        const int kc = frag_row + (opaque(frag_swz) ^ ((kk / 8) << 4));
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        const int c0 = wn * (BN / WN) + j * 32;
-        if (B_KCC) {
-            const int r = c0 + lane % 32;
-            b_off[j] = AOp::STAGE_BYTES + r * 128;
-            b_xor[j] = ((lane / 32) ^ ((r >> 1) & 7)) << 4;
-        } else {
-            const int g = lane / 16, q = lane % 16;
-            const int col = c0 + (g % 2) * 16 + (q % 4) * 4;
-            b_off[j] = AOp::STAGE_BYTES + ((g / 2) * 8 + q / 4) * (BN * 2) + ((((col / 8) ^ ((q / 4) << 2))) << 4) +
-                       (col % 8) * 2;
-            b_xor[j] = 0;
+        for (int i = 0; i < TM; ++i) {
+            if (A_KC) {
+                af[i] = *reinterpret_cast<const frag_t*>(st + kc + a_off[i]);
+            } else {
+                const char* q = st + a_off[i] + kk * (BM * 2);
+                union {
+                    v4i16_t h[2];
+                    frag_t f;
+                } u;
+                u.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(q));
+                u.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(q + 4 * (BM * 2)));
+                af[i] = u.f;
+            }
         }
-    }
-    auto a_frag = [&](const char* st, int i, int kk) -> frag_t {
-        if (A_KC) {
-            return *reinterpret_cast<const frag_t*>(st + a_off[i] + (a_xor[i] ^ ((kk / 8) << 4)));
-        } else {
-            const char* q = st + a_off[i] + kk * (BM * 2);
-            union {
-                v4i16_t h[2];
-                frag_t f;
-            } u;
-            u.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(q));
-            u.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(q + 4 * (BM * 2)));
-            return u.f;
-        }
-    };
-    auto b_frag = [&](const char* st, int j, int kk) -> frag_t {
-        if (B_KCC) {
-            return *reinterpret_cast<const frag_t*>(st + b_off[j] + (b_xor[j] ^ ((kk / 8) << 4)));
-        } else {
-            const char* q = st + b_off[j] + kk * (BN * 2);
-            union {
-                v4i16_t h[2];
-                frag_t f;
-            } u;
-            u.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(q));
-            u.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(q + 4 * (BN * 2)));
-            return u.f;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            if (B_KCC) {
+                bf[j] = *reinterpret_cast<const frag_t*>(st + kc + b_off[j]);
+            } else {
+                const char* q = st + b_off[j] + kk * (BN * 2);
+                union {
+                    v4i16_t h[2];
+                    frag_t f;
+                } u;
+                u.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(q));
+                u.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(q + 4 * (BN * 2)));
+                bf[j] = u.f;
+            }
         }
     };
 
@@ -584,65 +617,109 @@ __global__ void __launch_bounds__(TL::THREADS) grouped_gemm_dtl_kernel(GemmParam
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    // copies of a full tile, one quarter at a time (quarter q of 4), so that they can be spread over a step
-    auto issue_quarter = [&](char* st, int q) {
+    auto mma_group = [&](const frag_t* af, const frag_t* bf) {
 #pragma unroll
-        for (int j = 0; j < AOp::IPW; ++j)
-            if (j % 4 == q || AOp::IPW < 4) {
-                if (AOp::IPW >= 4 || q == 0) {
-                    __builtin_amdgcn_global_load_lds((gptr_t)a_ptr[j], (lptr_t)(st + (wave * AOp::IPW + j) * 1024), 16, 0, 0);
-                    a_ptr[j] += a_step;
-                }
-            }
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < BOp::IPW; ++j)
-            if (j % 4 == q || BOp::IPW < 4) {
-                if (BOp::IPW >= 4 || q == 0) {
-                    __builtin_amdgcn_global_load_lds(
-                        (gptr_t)b_ptr[j], (lptr_t)(st + AOp::STAGE_BYTES + (wave * BOp::IPW + j) * 1024), 16, 0, 0);
-                    b_ptr[j] += b_step;
-                }
-            }
+            for (int j = 0; j < TN; ++j) acc[i][j] = Mma<T>::mma(af[i], bf[j], acc[i][j]);
     };
-
-    // one step: request tile kt + 1 into `fill` (last read in step kt - 1, which every wave has left), multiply
-    // tile kt out of `cur`, then wait for the requested tile and meet the other waves.  The copies of a full
-    // tile are issued in four parts between the four MFMA groups, which keeps the memory pipeline and the LDS
-    // evenly loaded instead of hitting them with the whole tile at once.
-    auto step = [&](int kt, int k_tiles, const char* cur, char* fill) {
-        const bool more = kt + 1 < k_tiles && !(p.debug & 1);
-        const bool spread = more && k_begin + (kt + 2) * BK <= k_end;
-        if (more && !spread) issue(kt + 1, fill);
+    // Order inside one group of the pipelined loop: each MFMA is followed by its share of the group's LDS reads
+    // and at most one copy instruction, so the reads for the next group and the copies for the next tile trickle
+    // out under the matrix work instead of bunching up at either end.  Nothing crosses the group boundary.
+    constexpr int DS_READS = TM * (A_KC ? 1 : 2) + TN * (B_KCC ? 1 : 2);
+    constexpr int DS_PER_MMA = (DS_READS + TM * TN - 1) / (TM * TN);
+    auto pin_group = [&](int copies) {
+#pragma unroll
+        for (int m = 0; m < TM * TN; ++m) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, DS_PER_MMA, 0);
+            if (m < copies) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // all four groups of one tile, fragments read as they are needed (used outside the pipelined loop)
+    auto multiply_tile = [&](const char* st) {
 #pragma unroll
         for (int kk = 0; kk < BK; kk += 16) {
             frag_t af[TM], bf[TN];
-#pragma unroll
-            for (int i = 0; i < TM; ++i) af[i] = a_frag(cur, i, kk);
-#pragma unroll
-            for (int j = 0; j < TN; ++j) bf[j] = b_frag(cur, j, kk);
-            if (spread) issue_quarter(fill, kk / 16);
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j) acc[i][j] = Mma<T>::mma(af[i], bf[j], acc[i][j]);
+            read_frags(st, kk, af, bf);
+            mma_group(af, bf);
         }
-        if (!(p.debug & 32)) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        if (!(p.debug & 64)) __syncthreads();
+    };
+    // unpipelined step: request tile kt + 1 (whole, clipped to the contraction range), multiply tile kt
+    auto plain_step = [&](int kt, int k_tiles, const char* cur, char* fill) {
+        if (kt + 1 < k_tiles) issue(kt + 1, fill);
+        multiply_tile(cur);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+    };
+
+    // Pipelined step over tile kt in X while tile kt + 1 arrives in Y.  On entry: tile kt is complete in X, the
+    // fragments of its first group are in set 0, and the first PART_A copies of tile kt + 1 are under way.
+    //   groups 0-2  multiply out of X; the remaining copies of tile kt + 1 go out in groups 0 and 1
+    //   then every wave waits for its copies and meets the others: tile kt + 1 is complete, X is free
+    //   group 3     multiplies the last fragments of X (already in registers) while the first fragments of Y are
+    //               read and the first copies of tile kt + 2 start filling X
+    // Copies therefore have from one and a half to three groups of matrix work to land before anybody waits.
+    constexpr int PART_A = CK_DTL_PART_A < LOADS ? CK_DTL_PART_A : LOADS;
+    constexpr int PART_B = CK_DTL_PART_B < LOADS ? (CK_DTL_PART_B > PART_A ? CK_DTL_PART_B : PART_A) : LOADS;
+    frag_t af0[TM], bf0[TN], af1[TM], bf1[TN];
+    auto pipe_step = [&](int kt, char* X, char* Y) {
+        read_frags(X, 16, af1, bf1);
+        issue_range(Y, PART_A, PART_B, kt + 1);
+        mma_group(af0, bf0);
+        pin_group(PART_B - PART_A);
+        read_frags(X, 32, af0, bf0);
+        issue_range(Y, PART_B, LOADS, kt + 1);
+        mma_group(af1, bf1);
+        pin_group(LOADS - PART_B);
+        read_frags(X, 48, af1, bf1);
+        mma_group(af0, bf0);
+        pin_group(0);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        read_frags(Y, 0, af0, bf0);
+        issue_range(X, 0, PART_A, kt + 2);
+        mma_group(af1, bf1);
+        pin_group(PART_A);
     };
 
     const int k_tiles = (k_end - k_begin + BK - 1) / BK;
-    if (k_tiles > 0) issue(0, lds0);
+    const int n_full = (k_end - k_begin) / BK;  // leading tiles that lie completely inside the range
+    const bool primed = n_full >= 2;
+    int kt = 0;
+    if (primed) {
+        issue_range(lds0, 0, LOADS, 0);
+        issue_range(lds1, 0, PART_A, 1);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        read_frags(lds0, 0, af0, bf0);
+        // two steps per turn so that each names its buffers statically; the loop leaves with tile kt complete in
+        // lds0, the first copies of tile kt + 1 under way and at most three more tiles to go
+        for (; kt + 3 < n_full; kt += 2) {
+            pipe_step(kt, lds0, lds1);
+            pipe_step(kt + 1, lds1, lds0);
+        }
+        issue_range(lds1, PART_A, LOADS, kt + 1);
+    } else {
+        if (k_tiles > 0) issue(0, lds0);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (1 < k_tiles) issue(1, lds1);
+    }
+    if (k_tiles > 0) multiply_tile(lds0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    for (int kt = 0; kt < k_tiles; kt += 2) {
-        step(kt, k_tiles, lds0, lds1);
-        if (kt + 1 < k_tiles) step(kt + 1, k_tiles, lds1, lds0);
+    for (int t = kt + 1; t < k_tiles; t += 2) {
+        plain_step(t, k_tiles, lds1, lds0);
+        if (t + 1 < k_tiles) plain_step(t + 1, k_tiles, lds0, lds1);
     }
 
     // ---- epilogue -----------------------------------------------------------------------------------
     // Accumulators (lane: column lane % 32, rows 8 * (r / 4) + 4 * (lane / 32) + r % 4 of each 32x32 tile) are
     // rounded and staged in LDS - the upper half of the rows in one stage buffer, the lower half in the other -
     // then written out as 16-byte packets along rows, rows going to their mapped position.
+    const int lane = opaque(lane_id());
     S* Ch = reinterpret_cast<S*>(wm == 0 ? lds0 : lds1);
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -767,7 +844,7 @@ template <typename T, bool B_KC, bool GROUP_K>
 void launch_mfma(const ck::GemmParams& p, hipStream_t s) {
     const int total = p.m_tiles * p.n_tiles;
     const int grid = (total + 7) / 8 * 8;
-    if (p.debug & 16)
+    if (p.wide)
         hipLaunchKernelGGL((ck::grouped_gemm_kernel<T, MainTile, B_KC, GROUP_K>), dim3((unsigned)grid),
                            dim3(MainTile::THREADS), 0, s, p);
     else
@@ -815,7 +892,8 @@ extern "C" int ck_scatter2scatter(const void* X, int64_t x_stride, const void* W
         p.fan_out = (int)fan_out;
         p.x_grouped = x_grouped;
         p.y_grouped = y_grouped;
-        { const char* d = getenv("CK_GEMM_DEBUG"); p.debug = d ? atoi(d) : 0; }
+        // the direct-to-LDS kernel addresses a tile's sources with 32-bit byte offsets from a per-tile base
+        p.wide = num_slots * x_stride * 2 >= (int64_t)1 << 32 || (b_kc ? N : K) * p.ldb * 2 >= (int64_t)1 << 32;
         p.m_tiles = (int)(num_slots / kBM + E);
         p.n_tiles = (int)ck_ceil_div(N, kBN);
         if ((int64_t)p.m_tiles * p.n_tiles > 0x7ffffff0) return CK_ERR_SHAPE;
@@ -870,7 +948,7 @@ extern "C" int ck_group_bwd_W(const void* DY, int64_t dy_stride, const void* X, 
         p.K = (int)(swap ? N : K);  // I
         p.N = (int)(swap ? K : N);  // J
         p.E = (int)E;
-        { const char* d = getenv("CK_GEMM_DEBUG"); p.debug = d ? atoi(d) : 0; }
+        p.wide = 64 * p.lda * 2 >= (int64_t)1 << 32 || 64 * p.ldb * 2 >= (int64_t)1 << 32;
         p.m_tiles = (int)(E * ck_ceil_div(p.K, kBM));
         p.n_tiles = (int)ck_ceil_div(p.N, kBN);
         if ((int64_t)p.m_tiles * p.n_tiles > 0x7ffffff0) return CK_ERR_SHAPE;
