@@ -40,6 +40,10 @@ def parse_args():
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     p.add_argument("--only-extras", action="store_true", help="only the HBM-bound ops (for profiling them)")
     p.add_argument("--tokens", type=int, default=8192, help="T of the MoE workload (default: the BASELINE shape)")
+    p.add_argument("--no-ceiling", action="store_true", help="skip the sustained-MFMA-rate probe")
+    p.add_argument("--copy-calibration", action="store_true",
+                   help="also run three 1 GiB device copies before the steps (a kernel of known HBM traffic, to scale "
+                        "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     return p.parse_args()
 
 
@@ -101,7 +105,7 @@ def bench_moe(device, args):
     achieved = gemm_flop / (gemm_ms * 1e-3) / 1e12
     roofline = {
         "bound": "mfma",
-        "kernel": "grouped_gemm_kernel (scatter2scatter + group_bwd_W launches)",
+        "kernel": "grouped_gemm_dtl_kernel (scatter2scatter + group_bwd_W launches)",
         "achieved": round(achieved, 2),
         "peak": BF16_MFMA_PEAK_TFLOPS,
         "unit": "TFLOP/s",
@@ -122,6 +126,43 @@ def bench_moe(device, args):
     del moe, x, dy
     torch.cuda.empty_cache()
     return result, roofline, config
+
+
+def mfma_ceiling(device):
+    """TFLOP/s of back-to-back bf16 MFMAs on register operands: all-zero data, then random data (which draws
+    more power and so runs at a lower clock).  The second figure bounds any bf16 GEMM on real data here."""
+    from cute_kernels import _C
+
+    out = {}
+    sink = torch.zeros(1, device=device, dtype=torch.float32)
+    blocks, iters = 256, 20000
+    flop = blocks * 8 * iters * 32 * 32768.0
+    g = torch.Generator(device=device).manual_seed(0)
+    for label in ("zeros", "random"):
+        if label == "zeros":
+            ops = torch.zeros(24 * 512 * 8, device=device, dtype=torch.bfloat16)
+        else:
+            ops = torch.randn(24 * 512 * 8, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
+        best = None
+        for _ in range(3):
+            start = torch.cuda.Event(enable_timing=True)
+            end = torch.cuda.Event(enable_timing=True)
+            start.record()
+            _C.probe_mfma(ops, iters, blocks, sink)
+            end.record()
+            torch.cuda.synchronize()
+            ms = start.elapsed_time(end)
+            best = ms if best is None else min(best, ms)
+        out[label] = round(flop / (best * 1e-3) / 1e12, 1)
+    return out
+
+
+def copy_calibration(device):
+    src = torch.ones(1 << 29, device=device, dtype=torch.bfloat16)  # 1 GiB
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
 
 
 # ---- HBM-bound ops ----------------------------------------------------------------------------------------
@@ -246,6 +287,8 @@ def main():
     if args.only_extras:
         print(json.dumps({"extras": bench_extras(device)}))
         return
+    if args.copy_calibration:
+        copy_calibration(device)
     result, roofline, config = bench_moe(device, args)
     line = {
         "metric": "scattermoe_fwd_bwd_tflops",
@@ -264,6 +307,8 @@ def main():
         "frac_of_mfma_peak": result["frac_of_mfma_peak"],
         "roofline": roofline,
     }
+    if not args.no_ceiling:
+        line["sustained_mfma_tflops"] = mfma_ceiling(device)
     if not args.no_extras:
         line["extras"] = bench_extras(device)
     if not args.no_cpu:

@@ -170,6 +170,15 @@ int ck_moe_combine_forward(const void* expanded, const void* gates, void* out, i
 int ck_moe_combine_backward_gates(const void* expanded, const void* grad_out, void* d_gates, int64_t tokens,
                                   int64_t k, int64_t H, int dtype, void* stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * Measurement aid with no counterpart in the reference: back-to-back v_mfma_f32_32x32x16_bf16 on operands
+ * held in registers (the register footprint of the grouped GEMM's inner loop, no LDS or memory traffic), to
+ * read off the rate the matrix cores sustain on given data under the part's power limit.
+ *   operands : 24 * 512 * 16 bytes of bf16 values (device), sink: one float (device)
+ *   work     : blocks * 8 waves * iters * 32 MFMAs of 32768 flop; the caller times the launch
+ * ------------------------------------------------------------------------------------------- */
+int ck_probe_mfma(const void* operands, int64_t iters, int blocks, float* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

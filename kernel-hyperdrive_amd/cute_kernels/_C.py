@@ -58,6 +58,7 @@ _SIGNATURES = {
     "ck_group": (_i32, [_p, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _i32, _p]),
     "ck_moe_combine_forward": (_i32, [_p, _p, _p, _i64, _i64, _i64, _i32, _p]),
     "ck_moe_combine_backward_gates": (_i32, [_p, _p, _p, _i64, _i64, _i64, _i32, _p]),
+    "ck_probe_mfma": (_i32, [_p, _i64, _i32, _p, _p]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
@@ -391,3 +392,13 @@ def moe_combine_backward_gates(expanded, grad_out, d_gates) -> None:
                                               dtype_code(expanded.dtype), L.stream),
             "ck_moe_combine_backward_gates",
         )
+
+
+def probe_mfma(operands, iters: int, blocks: int, sink) -> None:
+    """Measurement aid: `blocks` workgroups of 8 waves issue `iters` * 32 MFMAs each on `operands` (uint8/any
+    tensor of at least 24 * 512 * 16 bytes, device); `sink` is a one-element float32 device tensor."""
+    lib = load_library()
+    if operands.numel() * operands.element_size() < 24 * 512 * 16:
+        raise ValueError("operands must hold at least 24 * 512 * 16 bytes")
+    with _Launch(operands, sink) as L:
+        _check(lib.ck_probe_mfma(_ptr(operands), iters, blocks, _ptr(sink), L.stream), "ck_probe_mfma")

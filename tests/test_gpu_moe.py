@@ -5,7 +5,7 @@ import pytest
 import torch
 import torch.nn as nn
 
-from helpers import acc_dtype, announce, assert_close, assert_norm_close, randn
+from helpers import acc_dtype, announce, assert_close, assert_close_long_sums, assert_norm_close, randn
 from oracle import cute_oracle as O
 
 
@@ -160,6 +160,9 @@ MOE_CASES = [
     ("odd_rows", 333, 256, 384, 6, 3, None),
     ("skewed_empty", 2048, 256, 128, 32, 4, 2.0),
     ("top1", 200, 128, 128, 4, 1, None),
+    # the fine-grained skewed configuration (H=2048, I=1408, E=64, top-6, Zipf(1.2) expert popularity) at 1/16 of
+    # its tokens, so that the CPU oracle finishes in seconds; the full size is covered below
+    ("config5_tokens_div16", 1024, 2048, 1408, 64, 6, 1.25),
 ]
 
 
@@ -169,6 +172,8 @@ def test_moe_layer_against_oracle(gpu, dtype, case):
     from cute_kernels import MoE_Triton
 
     name, T, H, I, E, k, skew = case
+    if name == "config5_tokens_div16" and dtype == torch.float16:
+        pytest.skip("the CPU oracle's native fp16 matrix products take minutes at this size; bf16 and fp32 run")
     announce("moe layer", dtype, case)
     x, w_gate, w_fc, w_proj, dy = O.moe_inputs(T, H, I, E, dtype, seed=61)
     if skew is not None:
@@ -183,7 +188,17 @@ def test_moe_layer_against_oracle(gpu, dtype, case):
     compute = dtype if dtype != torch.float32 else torch.float64
     expected = O.moe_forward_backward(x, w_gate, w_fc, w_proj, dy, k, compute_dtype=compute, selected=selected)
     for key in ("router_logits", "y", "dx", "dw_fc", "dw_proj"):
-        assert_close(got[key], expected[key], dtype, f"{name}/{key}")
+        a, e = got[key], expected[key]
+        if key == "dx" and skew is not None:
+            # feature 0 carries the popularity bias (|w_gate[:, 0]| up to 6): its gradient is the router's
+            # contribution alone, made by stock torch ops and amplified by those weights, so it is held to a
+            # norm-wise bound like the router gradient below
+            assert_norm_close(a[:, 0], e[:, 0], 1e-5 if dtype == torch.float32 else 2e-2, f"{name}/dx[:, 0]")
+            a, e = a[:, 1:], e[:, 1:]
+        if key in ("dw_fc", "dw_proj") and E >= 64:
+            assert_close_long_sums(a, e, dtype, f"{name}/{key}")
+        else:
+            assert_close(a, e, dtype, f"{name}/{key}")
     # the router gradient is made by stock torch ops (bmm, softmax and linear backward) from the routing
     # weights' gradient; every element is a sum over all tokens of O(1) products whose 16-bit roundings do
     # not cancel, so it is held to a norm-wise bound
@@ -196,7 +211,7 @@ def test_moe_layer_against_oracle(gpu, dtype, case):
         exact = O.moe_forward_backward(x, w_gate, w_fc, w_proj, dy, k, compute_dtype=torch.float32, selected=selected)
         tol = O.tolerance(dtype)
         for key in ("y", "dx", "dw_fc", "dw_proj"):
-            assert O.fraction_outside(got[key], exact[key], **tol) < 2e-3, key
+            assert O.fraction_outside(got[key], exact[key], **tol) < (2e-3 if k <= 4 else 5e-3), key  # more terms per row at top-6
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
@@ -250,3 +265,71 @@ def test_moe_3d_input_and_weight_grad_layout(gpu):
         g, gr = getattr(moe, name).weight.grad, getattr(ref, name).weight.grad
         assert g.shape == gr.shape and g.is_contiguous()
         assert_close(g, gr, dtype, name)
+
+
+# ---- full BASELINE sizes: HIP layer against the torch implementation of the same layer, both on the GPU -------
+FULL_CASES = [
+    # name, T, H, I, E, k, skew
+    ("mixtral", 8192, 4096, 14336, 8, 2, None),
+    ("fine_grained_skewed", 16384, 2048, 1408, 64, 6, 1.25),
+]
+
+
+@pytest.mark.parametrize("case", FULL_CASES, ids=[c[0] for c in FULL_CASES])
+def test_moe_full_size_against_torch_layer(gpu, case):
+    """At the full shapes the CPU oracle is out of reach, so the HIP layer is compared with MoE_Torch (the
+    reference's per-expert F.linear formulation, stock torch ops) on the same device and weights, plus the
+    size-independent properties of the routing step."""
+    from cute_kernels import MoE_Torch, MoE_Triton
+    from cute_kernels.kernels.scattermoe import moe_sort
+
+    name, T, H, I, E, k, skew = case
+    announce("moe full size", case)
+    dtype = torch.bfloat16
+    g = torch.Generator(device=gpu).manual_seed(81)
+    x = torch.randn(T, H, generator=g, device=gpu)
+    w_gate = torch.randn(E, H, generator=g, device=gpu) * 0.02
+    w_fc = torch.randn(E, 2 * I, H, generator=g, device=gpu) * 0.02
+    w_proj = torch.randn(E, H, I, generator=g, device=gpu) * 0.02
+    dy = torch.randn(T, H, generator=g, device=gpu).to(dtype)
+    if skew is not None:
+        w_gate, x = O.skewed_router(w_gate.cpu(), x.cpu(), 1.2, seed=82, scale=skew)
+        w_gate, x = w_gate.to(gpu), x.to(gpu)
+    x = x.to(dtype)
+    moe = build_moe(MoE_Triton, gpu, dtype, E, k, H, I, w_gate, w_fc, w_proj)
+    ref = build_moe(MoE_Torch, gpu, dtype, E, k, H, I, w_gate, w_fc, w_proj)
+    del w_fc, w_proj
+
+    with torch.no_grad():
+        _, _, selected = moe._compute_routing_weights(x)
+    load = selected.flatten().bincount(minlength=E)
+    if skew is not None:
+        assert (load == 0).any(), "the skewed configuration must leave at least one expert without tokens"
+        assert load.max().item() > 0.10 * T, "one expert must be chosen by more than 10 % of the tokens"
+    s_e, s_idx, off = moe_sort(selected, E)
+    assert off[-1].item() == T * k and torch.equal(off, load.cumsum(0))
+    assert torch.equal(s_e, selected.flatten()[s_idx]) and (s_e[1:] >= s_e[:-1]).all()
+    assert torch.equal(s_idx.sort().values, torch.arange(T * k, device=gpu)), "a permutation"
+    same = s_e[1:] == s_e[:-1]
+    assert (s_idx[1:][same] > s_idx[:-1][same]).all(), "stable: positions ascend inside each expert"
+
+    xg = x.clone().requires_grad_(True)
+    xr = x.clone().requires_grad_(True)
+    y, logits = moe(xg)
+    yr, logits_r = ref(xr)
+    (y * dy).sum().backward()
+    (yr * dy).sum().backward()
+    tol = O.tolerance(dtype)
+    assert torch.equal(logits, logits_r)
+    for what, a, b in (("y", y.detach(), yr.detach()), ("dx", xg.grad, xr.grad),
+                       ("dw_fc", moe.c_fc.weight.grad, ref.c_fc.weight.grad),
+                       ("dw_proj", moe.c_proj.weight.grad, ref.c_proj.weight.grad)):
+        # both sides round 16-bit intermediates, in different places: nearly all elements agree within the
+        # tolerance, and the whole tensor agrees norm-wise at the rounding level of bf16
+        frac = ((a.float() - b.float()).abs() > tol["atol"] + tol["rtol"] * b.float().abs()).float().mean().item()
+        assert frac < 5e-3, f"{name}/{what}: {frac:.2e} of the elements outside rtol 2e-2 / atol 1e-2"
+        err = (a.float() - b.float()).norm().item() / max(b.float().norm().item(), 1e-30)
+        assert err < 1e-2, f"{name}/{what}: relative Frobenius error {err:.3e}"
+    empty = (load == 0).nonzero().flatten().tolist()
+    for e in empty:
+        assert not moe.c_fc.weight.grad[e].any() and not moe.c_proj.weight.grad[e].any(), "experts without tokens get zero grads"
