@@ -29,6 +29,11 @@ import torch  # noqa: E402
 
 BF16_MFMA_PEAK_TFLOPS = 2500.0
 HBM_PEAK_GBS = 8000.0
+# HBM-side bytes per grouped-GEMM launch at the Mixtral shape, from two rocprofv3 --pmc runs of this file
+# (FETCH_SIZE, then WRITE_SIZE, each scaled by what the same counter reads for the 1 GiB copies of
+# --copy-calibration): 33.5 GB read + 4.5 GB written per step over 6 launches.  Summary:
+# profiles/grouped_gemm_hbm_traffic_moe_mixtral_bf16.txt
+GEMM_HBM_BYTES_PER_LAUNCH = 6.34e9
 
 
 def parse_args():
@@ -110,7 +115,7 @@ def bench_moe(device, args):
         "peak": BF16_MFMA_PEAK_TFLOPS,
         "unit": "TFLOP/s",
         "frac": round(achieved / BF16_MFMA_PEAK_TFLOPS, 4),
-        "traffic": None,
+        "traffic": GEMM_HBM_BYTES_PER_LAUNCH if (T, H, I, E, k) == (8192, 4096, 14336, 8, 2) else None,
         "launches_per_step": launches // args.steps,
         "avg_launch_ms": round(gemm_ms / max(launches, 1), 4),
         "gemm_ms_per_step": round(gemm_ms / args.steps, 3),
