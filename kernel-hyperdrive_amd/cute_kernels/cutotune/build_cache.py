@@ -1,0 +1,59 @@
+"""Fills the tuning cache on the GPU at hand and writes it next to this module (or to ``--output``).
+
+    python -m cute_kernels.cutotune.build_cache [--output FILE]
+
+Counterpart of the reference's tools/build_cutotune_cache.py:1-62: one forward + backward of every tuned operator
+per dtype, at the reference's tuning shapes plus the shapes of this repository's benchmark, so that first calls
+do not pay for the search.  The add_scalar / add_tensor operators of the reference script are not part of this
+package.
+"""
+
+import argparse
+from typing import Callable
+
+import torch
+
+from .. import embedding_cute, get_powers_of_2, rmsnorm_cute, swiglu_cute, swiglu_unchunked_cute
+from .cache import get_cutotune_cache
+
+
+def forward_backward(kernel: Callable, *args, **kwargs) -> None:
+    output = kernel(*args, **kwargs)
+    output.sum().backward()
+
+
+def main() -> None:
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--output", default=None, help="file to write (default: the package's cutotune_cache.yml)")
+    args = parser.parse_args()
+    if not torch.cuda.is_available():
+        raise SystemExit("build_cache needs the GPU the cache is meant for")
+
+    torch.manual_seed(42)
+    device = torch.device("cuda", torch.cuda.current_device())
+    for dtype in (torch.float32, torch.float16, torch.bfloat16):
+        for size in (104857600, 16384 * 14336):
+            x = torch.randn(size, dtype=dtype, device=device, requires_grad=True)
+            forward_backward(swiglu_cute, x, x)
+            del x
+        for size in ((81920, 8192), (16384, 28672)):
+            forward_backward(swiglu_unchunked_cute, torch.randn(size, dtype=dtype, device=device, requires_grad=True))
+        for power_of_2 in get_powers_of_2(1, 65536):
+            x = torch.randn(2048, power_of_2, dtype=dtype, device=device, requires_grad=True)
+            forward_backward(rmsnorm_cute, x, weight=None, eps=1e-5)
+            weight = torch.randn(power_of_2, dtype=dtype, device=device, requires_grad=True)
+            forward_backward(rmsnorm_cute, x, weight=weight, eps=1e-5)
+        for ids_size, table_size in (((32, 4096), (131072, 4096)), ((8, 4096), (128256, 4096))):
+            ids = torch.randint(0, table_size[0] - 1, ids_size, device=device, dtype=torch.long)
+            table = torch.randn(table_size, device=device, dtype=dtype, requires_grad=True)
+            forward_backward(embedding_cute, input_ids=ids, weight=table)
+            del table
+        print(dtype, "done", flush=True)
+
+    cache = get_cutotune_cache()
+    cache.save(args.output)
+    print("wrote", args.output or cache.filename)
+
+
+if __name__ == "__main__":
+    main()

@@ -325,3 +325,20 @@ def test_replace_swiglu_unchunked_matches_only_the_pattern():
         assert (swiglu_unchunked_cute in _targets(gm)) is expect, fn.__name__
         if expect:
             assert "chunk" not in _targets(gm) and F.silu not in _targets(gm)
+
+
+def test_shipped_tuning_cache_loads_and_covers_the_tuned_launchers():
+    """The cache next to cutotune/cache.py was written by cutotune/build_cache.py on an MI355X; it must parse with the
+    reference's schema and hold a best config per dtype for every launcher that has a search space."""
+    from cute_kernels.cutotune.cache import _CutoTuneCache, _CUTOTUNE_CACHE_FILENAME
+
+    cache = _CutoTuneCache(_CUTOTUNE_CACHE_FILENAME, load=True)
+    for fn in ("kernels/swiglu.py->_forward", "kernels/swiglu.py->_backward", "kernels/swiglu_unchunked.py->_forward",
+               "kernels/swiglu_unchunked.py->_backward", "kernels/rmsnorm.py->_forward", "kernels/embedding.py->_backward"):
+        best = cache.get_best_configs(fn)
+        assert len(best) == 3, (fn, list(best))
+        for key, (config, time) in best.items():
+            assert "dtype = torch." in key
+            assert config.get_key_values()["kernel_backend"].value == "hip"
+    sw = cache.full_cache["kernels/swiglu.py->_forward"]
+    assert all(len(entries) >= 2 for entries in sw.values()), "every candidate's timing is kept"
