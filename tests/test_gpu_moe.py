@@ -333,3 +333,34 @@ def test_moe_full_size_against_torch_layer(gpu, case):
     empty = (load == 0).nonzero().flatten().tolist()
     for e in empty:
         assert not moe.c_fc.weight.grad[e].any() and not moe.c_proj.weight.grad[e].any(), "experts without tokens get zero grads"
+
+
+# ---- operands beyond 32-bit byte offsets: the grouped GEMM switches to 64-bit addressing ------------------------
+def test_grouped_gemm_with_rows_four_gib_apart(gpu):
+    """X rows (scatter2scatter) and the rows of X / DY (group_bwd_W) taken from a buffer with a row stride of 2^26
+    elements: the last row starts 8 GiB after the first, beyond what 32-bit byte offsets reach."""
+    from cute_kernels.kernels.scattermoe import group_bwd_W, scatter2scatter
+
+    announce("grouped GEMM wide strides")
+    dtype = torch.bfloat16
+    T, k, E, K, N = 72, 1, 3, 64, 128
+    stride = 1 << 26
+    s_e, s_idx, off = routing(T, k, E, 91)
+    big = torch.empty(T * stride + K, dtype=dtype, device=gpu)
+    Xw = big.as_strided((T, K), (stride, 1))
+    X = randn((T, K), dtype, 92)
+    Xw.copy_(X.to(gpu))
+    W = randn((E, K, N), dtype, 93, 0.05)
+    out = torch.full((T, N), float("nan"), dtype=dtype, device=gpu)
+    scatter2scatter(Xw, W.to(gpu), s_e.to(gpu), s_idx.to(gpu), out, 1, False, True, off.to(gpu))
+    assert_close(out, O.scatter2scatter(X, W, s_idx, off, 1, False, True, acc_dtype(dtype)), dtype, "s2s wide")
+
+    # group_bwd_W: X rows expert-grouped in the wide buffer, DY dense
+    Xg = X[s_idx]
+    Xw.copy_(Xg.to(gpu))
+    DY = randn((T, N), dtype, 94)
+    DW = torch.full((E, K, N), float("nan"), dtype=dtype, device=gpu)
+    group_bwd_W(DY.to(gpu), Xw, off.to(gpu), DW, E)
+    assert_close(DW, O.group_bwd_W(DY, Xg, off, E, acc_dtype(dtype)), dtype, "dW wide")
+    del big
+    torch.cuda.empty_cache()
