@@ -110,7 +110,7 @@ def bench_moe(device, args):
     achieved = gemm_flop / (gemm_ms * 1e-3) / 1e12
     roofline = {
         "bound": "mfma",
-        "kernel": "grouped_gemm_dtl_kernel (scatter2scatter + group_bwd_W launches)",
+        "kernel": "grouped_gemm_m16_kernel (scatter2scatter + group_bwd_W launches)",
         "achieved": round(achieved, 2),
         "peak": BF16_MFMA_PEAK_TFLOPS,
         "unit": "TFLOP/s",

@@ -6,8 +6,9 @@
 //   ck_group           : out[i] = A[idx[i] / fan_out] * coeff[idx[i]]    (row gather)
 //       cute_kernels/kernels/scattermoe/triton_implementation/kernels.py:243-298
 //
-// 16-bit types run on the matrix cores: v_mfma_f32_32x32x16_{bf16,f16}, fp32 accumulators, operand tiles
-// staged through double-buffered LDS.  Tiles are scheduled per expert from expert_offsets, so a tile
+// 16-bit types run on the matrix cores: v_mfma_f32_16x16x32_{bf16,f16} (which sustains a higher rate on real data
+// under the power limit than the 32x32x16 shape), fp32 accumulators, operand tiles copied straight into
+// double-buffered LDS.  Tiles are scheduled per expert from expert_offsets, so a tile
 // never mixes rows of two experts (the reference lets a 128-row block straddle experts and repeats the
 // product once per expert present in it).  fp32, and shapes whose contiguous dimensions are not
 // multiples of 8 elements, go through a plain kernel with exact (fp64) accumulation.
@@ -30,6 +31,23 @@ struct Mma<F16> {
     typedef f16x8_t frag_t;
     static __device__ __forceinline__ f32x16_t mma(frag_t a, frag_t b, f32x16_t c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
+
+template <typename T>
+struct Mma16;
+template <>
+struct Mma16<BF16> {
+    typedef bf16x8_t frag_t;
+    static __device__ __forceinline__ f32x4_t mma(frag_t a, frag_t b, f32x4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    }
+};
+template <>
+struct Mma16<F16> {
+    typedef f16x8_t frag_t;
+    static __device__ __forceinline__ f32x4_t mma(frag_t a, frag_t b, f32x4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
     }
 };
 
@@ -365,12 +383,6 @@ __global__ void __launch_bounds__(TL::THREADS) grouped_gemm_kernel(GemmParams p)
 // LDS positions whose contraction index lies beyond the end of the contraction range are cleared with a
 // plain store in the (single) partial step; positions of rows / columns outside the problem keep whatever
 // they held, which only reaches outputs that are never stored.
-#ifndef CK_DTL_PART_A
-#define CK_DTL_PART_A 4
-#endif
-#ifndef CK_DTL_PART_B
-#define CK_DTL_PART_B 8
-#endif
 template <typename S, int ROWS, bool KC, int NWAVES>
 struct DtlOperand {
     static constexpr int BK = 64;
@@ -395,12 +407,22 @@ __device__ __forceinline__ int opaque(int v) {
     return v;
 }
 
+__device__ __forceinline__ uint64_t opaque_s64(uint64_t v) {  // same for a wave-uniform 64-bit value
+    asm volatile("" : "+s"(v));
+    return v;
+}
+
 template <typename T, typename TL, bool B_KC, bool GROUP_K>
-__global__ void __launch_bounds__(TL::THREADS) grouped_gemm_dtl_kernel(GemmParams p) {
+// Two waves per SIMD is all the LDS footprint allows; telling the compiler keeps it from spilling to reach a
+// higher occupancy that cannot happen.
+__global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
+    grouped_gemm_m16_kernel(GemmParams p) {
     typedef typename T::storage_t S;
-    typedef typename Mma<T>::frag_t frag_t;
+    typedef typename Mma16<T>::frag_t frag_t;
     constexpr int BM = TL::BM, BN = TL::BN, BK = 64, WM = TL::WM, WN = TL::WN;
-    constexpr int THREADS = TL::THREADS, TM = TL::TM, TN = TL::TN, NWAVES = WM * WN;
+    constexpr int THREADS = TL::THREADS, NWAVES = WM * WN;
+    constexpr int TM = BM / WM / 16, TN = BN / WN / 16, TH = TM / 2;  // 16 x 16 tiles per wave; TH: half of the rows
+    static_assert(TM % 2 == 0, "the loop works on one half of a wave's rows at a time");
     static_assert(TL::BK == 64, "the direct-to-LDS kernel is written for BK = 64");
     static_assert(WM == 2, "the epilogue stages one half of the rows per stage buffer");
     constexpr bool A_KC = !GROUP_K;
@@ -491,9 +513,11 @@ __global__ void __launch_bounds__(TL::THREADS) grouped_gemm_dtl_kernel(GemmParam
 
     constexpr int LOADS = AOp::IPW + BOp::IPW;  // copy instructions per wave per tile, A first
     // copy instructions [j0, j1) of tile t, which lies completely inside the contraction range
-    auto issue_range = [&](char* st, int j0, int j1, int t) {
-        const gchar_t at = a_base + (int64_t)t * a_step;
-        const gchar_t bt = b_base + (int64_t)t * b_step;
+    auto issue_range = [&](char* st, int j0, int j1, int t) __attribute__((always_inline)) {
+        // the tile bases are made opaque so that they stay in scalar registers and each copy is addressed as
+        // scalar base + 32-bit lane offset, instead of being folded into 64-bit per-lane pointers
+        const gchar_t at = (gchar_t)opaque_s64((uint64_t)(a_base + (int64_t)t * a_step));
+        const gchar_t bt = (gchar_t)opaque_s64((uint64_t)(b_base + (int64_t)t * b_step));
 #pragma unroll
         for (int j = 0; j < LOADS; ++j) {
             if (j < j0 || j >= j1) continue;
@@ -507,7 +531,7 @@ __global__ void __launch_bounds__(TL::THREADS) grouped_gemm_dtl_kernel(GemmParam
         }
     };
     // tile t whatever its position: slots past the end of the contraction range are cleared instead of copied
-    auto issue = [&](int t, char* st) {
+    auto issue = [&](int t, char* st) __attribute__((always_inline)) {
         const int k0 = k_begin + t * BK;
         if (k0 + BK <= k_end) {
             issue_range(st, 0, LOADS, t);
@@ -540,49 +564,52 @@ __global__ void __launch_bounds__(TL::THREADS) grouped_gemm_dtl_kernel(GemmParam
     };
 
     // ---- fragment addresses (bytes inside a stage) -----------------------------------------------------
-    // k-contiguous operand: row r of the tile starts at r * 128; the 16-byte chunk c of that row sits in slot
-    //   c ^ ((r >> 1) & 7).  A lane reads chunk kk / 8 + lane / 32 of row (lane % 32) + 32 * i: the swizzle term
-    //   depends on the lane only, and kk / 8 is even, so the slot is (lane-dependent part) ^ (kk / 8).
-    // other layout: see OperandTile; one address per 32-wide block, the contraction index adds a multiple of the
-    //   line size.
+    // v_mfma_f32_16x16x32: lane l holds row (or column) l % 16 and the 8 contraction indices 8 * (l / 16) .. + 7.
+    // k-contiguous operand: row r starts at r * 128, chunk c sits in slot c ^ ((r >> 1) & 7).  A lane reads chunk
+    //   kk / 8 + l / 16 of row l % 16 + 16 * i; kk / 8 is 0 or 4 and l / 16 < 4, so the slot is
+    //   (lane-dependent part) ^ (kk / 8) and i adds a compile-time multiple of 2048 bytes.
+    // other layout (contraction row = ROWS * 2 bytes, chunk c of row k in slot c ^ ((k & 3) << 2)): two transposing
+    //   reads; in each group of 16 lanes, lane q fetches elements 4 (q % 4) .. + 3 of contraction row q / 4 (then
+    //   + 4) of the 16-wide block, and receives element q of each of the four rows.
     int frag_row, frag_swz;
     int a_off[TM], b_off[TN];
     {
         const int lane = lane_id();
-        frag_row = (lane % 32) * 128;
-        frag_swz = ((lane / 32) ^ (((lane % 32) >> 1) & 7)) << 4;
+        frag_row = (lane % 16) * 128;
+        frag_swz = ((lane / 16) ^ ((lane % 16) >> 1)) << 4;
         const int g = lane / 16, q = lane % 16;
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
-            const int r0 = wm * (BM / WM) + i * 32;
+            const int r0 = wm * (BM / WM) + i * 16;
             if (A_KC) {
                 a_off[i] = r0 * 128;
             } else {
-                const int col = r0 + (g % 2) * 16 + (q % 4) * 4;
-                a_off[i] = ((g / 2) * 8 + q / 4) * (BM * 2) + ((((col / 8) ^ ((q / 4) << 2))) << 4) + (col % 8) * 2;
+                const int col = r0 + (q % 4) * 4;
+                a_off[i] = (g * 8 + q / 4) * (BM * 2) + ((((col / 8) ^ ((q / 4) << 2))) << 4) + (col % 8) * 2;
             }
         }
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-            const int c0 = wn * (BN / WN) + j * 32;
+            const int c0 = wn * (BN / WN) + j * 16;
             if (B_KCC) {
                 b_off[j] = AOp::STAGE_BYTES + c0 * 128;
             } else {
-                const int col = c0 + (g % 2) * 16 + (q % 4) * 4;
-                b_off[j] = AOp::STAGE_BYTES + ((g / 2) * 8 + q / 4) * (BN * 2) + ((((col / 8) ^ ((q / 4) << 2))) << 4) +
-                           (col % 8) * 2;
+                const int col = c0 + (q % 4) * 4;
+                b_off[j] = AOp::STAGE_BYTES + (g * 8 + q / 4) * (BN * 2) + ((((col / 8) ^ ((q / 4) << 2))) << 4) + (col % 8) * 2;
             }
         }
     }
-    auto read_frags = [&](const char* st, int kk, frag_t* af, frag_t* bf) {
-        // position of this lane's chunk in a k-contiguous row, recomputed here on purpose
+    // fragments of rows [16 * TH * half, + 16 * TH) of the wave's block, contraction indices kk .. kk + 31
+    auto read_a = [&](const char* st, int kk, int half, frag_t* af) __attribute__((always_inline)) {
         const int kc = frag_row + (opaque(frag_swz) ^ ((kk / 8) << 4));
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
+        for (int i = 0; i < TH; ++i) {
             if (A_KC) {
-                af[i] = *reinterpret_cast<const frag_t*>(st + kc + a_off[i]);
+                af[i] = *reinterpret_cast<const frag_t*>(st + kc + a_off[half * TH + i]);
             } else {
-                const char* q = st + a_off[i] + kk * (BM * 2);
+                // blocks 2m and 2m + 1 differ in bit 1 of the chunk index only, below the swizzled bits: + 32 bytes
+                const int ii = half * TH + i;
+                const char* q = st + a_off[ii & ~1] + (ii & 1) * 32 + kk * (BM * 2);
                 union {
                     v4i16_t h[2];
                     frag_t f;
@@ -592,12 +619,15 @@ __global__ void __launch_bounds__(TL::THREADS) grouped_gemm_dtl_kernel(GemmParam
                 af[i] = u.f;
             }
         }
+    };
+    auto read_b = [&](const char* st, int kk, frag_t* bf) __attribute__((always_inline)) {
+        const int kc = frag_row + (opaque(frag_swz) ^ ((kk / 8) << 4));
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
             if (B_KCC) {
                 bf[j] = *reinterpret_cast<const frag_t*>(st + kc + b_off[j]);
             } else {
-                const char* q = st + b_off[j] + kk * (BN * 2);
+                const char* q = st + b_off[j & ~1] + (j & 1) * 32 + kk * (BN * 2);
                 union {
                     v4i16_t h[2];
                     frag_t f;
@@ -609,79 +639,82 @@ __global__ void __launch_bounds__(TL::THREADS) grouped_gemm_dtl_kernel(GemmParam
         }
     };
 
-    f32x16_t acc[TM][TN];
+    f32x4_t acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+            for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
 
-    auto mma_group = [&](const frag_t* af, const frag_t* bf) {
+    auto mma_half = [&](int half, const frag_t* af, const frag_t* bf) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TH; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; ++j) acc[i][j] = Mma<T>::mma(af[i], bf[j], acc[i][j]);
+            for (int j = 0; j < TN; ++j) acc[half * TH + i][j] = Mma16<T>::mma(af[i], bf[j], acc[half * TH + i][j]);
     };
-    // Order inside one group of the pipelined loop: each MFMA is followed by its share of the group's LDS reads
-    // and at most one copy instruction, so the reads for the next group and the copies for the next tile trickle
-    // out under the matrix work instead of bunching up at either end.  Nothing crosses the group boundary.
-    constexpr int DS_READS = TM * (A_KC ? 1 : 2) + TN * (B_KCC ? 1 : 2);
-    constexpr int DS_PER_MMA = (DS_READS + TM * TN - 1) / (TM * TN);
-    auto pin_group = [&](int copies) {
+    // Order inside one group of TH * TN MFMAs: each MFMA is followed by at most one LDS read of the group and at
+    // most one copy instruction.  Nothing crosses the group boundary.
+    static_assert((TH * (A_KC ? 1 : 2) + TN * (B_KCC ? 1 : 2)) <= TH * TN, "one LDS read per MFMA must be enough");
+    auto pin_group = [&](int copies) __attribute__((always_inline)) {
 #pragma unroll
-        for (int m = 0; m < TM * TN; ++m) {
+        for (int m = 0; m < TH * TN; ++m) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, DS_PER_MMA, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
             if (m < copies) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
     };
-    // all four groups of one tile, fragments read as they are needed (used outside the pipelined loop)
-    auto multiply_tile = [&](const char* st) {
+    // one whole tile, fragments read as they are needed (used outside the pipelined loop)
+    auto multiply_tile = [&](const char* st) __attribute__((always_inline)) {
 #pragma unroll
-        for (int kk = 0; kk < BK; kk += 16) {
-            frag_t af[TM], bf[TN];
-            read_frags(st, kk, af, bf);
-            mma_group(af, bf);
+        for (int kk = 0; kk < BK; kk += 32) {
+            frag_t bf[TN];
+            read_b(st, kk, bf);
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                frag_t af[TH];
+                read_a(st, kk, half, af);
+                mma_half(half, af, bf);
+            }
         }
     };
     // unpipelined step: request tile kt + 1 (whole, clipped to the contraction range), multiply tile kt
-    auto plain_step = [&](int kt, int k_tiles, const char* cur, char* fill) {
+    auto plain_step = [&](int kt, int k_tiles, const char* cur, char* fill) __attribute__((always_inline)) {
         if (kt + 1 < k_tiles) issue(kt + 1, fill);
         multiply_tile(cur);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
     };
 
-    // Pipelined step over tile kt in X while tile kt + 1 arrives in Y.  On entry: tile kt is complete in X, the
-    // fragments of its first group are in set 0, and the first PART_A copies of tile kt + 1 are under way.
-    //   groups 0-2  multiply out of X; the remaining copies of tile kt + 1 go out in groups 0 and 1
-    //   then every wave waits for its copies and meets the others: tile kt + 1 is complete, X is free
-    //   group 3     multiplies the last fragments of X (already in registers) while the first fragments of Y are
-    //               read and the first copies of tile kt + 2 start filling X
-    // Copies therefore have from one and a half to three groups of matrix work to land before anybody waits.
-    constexpr int PART_A = CK_DTL_PART_A < LOADS ? CK_DTL_PART_A : LOADS;
-    constexpr int PART_B = CK_DTL_PART_B < LOADS ? (CK_DTL_PART_B > PART_A ? CK_DTL_PART_B : PART_A) : LOADS;
-    frag_t af0[TM], bf0[TN], af1[TM], bf1[TN];
-    auto pipe_step = [&](int kt, char* X, char* Y) {
-        read_frags(X, 16, af1, bf1);
-        issue_range(Y, PART_A, PART_B, kt + 1);
-        mma_group(af0, bf0);
-        pin_group(PART_B - PART_A);
-        read_frags(X, 32, af0, bf0);
-        issue_range(Y, PART_B, LOADS, kt + 1);
-        mma_group(af1, bf1);
-        pin_group(LOADS - PART_B);
-        read_frags(X, 48, af1, bf1);
-        mma_group(af0, bf0);
+    // Pipelined step over tile kt in X while tile kt + 1 arrives in Y.  A tile is two contraction groups of 32,
+    // each multiplied in two halves of the wave's rows: four groups of TH * TN MFMAs.  On entry the fragments of
+    // the first group (lower rows + columns of contraction group 0) are in registers.
+    //   group 0   reads the upper rows of contraction group 0
+    //   group 1   reads the lower rows and the columns of contraction group 1
+    //   group 2   reads the upper rows of contraction group 1 - the last fragments of X
+    //   then every wave waits for its copies and meets the others: tile kt + 1 is complete in Y, X is free
+    //   group 3   multiplies those last fragments while the first fragments of Y are read and the copies of tile
+    //             kt + 2 start filling X: three groups of matrix work pass before anybody waits for them
+    frag_t a_lo[TH], a_hi[TH], b_0[TN], b_1[TN];
+    auto pipe_step = [&](int kt, char* X, char* Y) __attribute__((always_inline)) {
+        read_a(X, 0, 1, a_hi);
+        mma_half(0, a_lo, b_0);
+        pin_group(0);
+        read_a(X, 32, 0, a_lo);
+        read_b(X, 32, b_1);
+        mma_half(1, a_hi, b_0);
+        pin_group(0);
+        read_a(X, 32, 1, a_hi);
+        mma_half(0, a_lo, b_1);
         pin_group(0);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        read_frags(Y, 0, af0, bf0);
-        issue_range(X, 0, PART_A, kt + 2);
-        mma_group(af1, bf1);
-        pin_group(PART_A);
+        read_a(Y, 0, 0, a_lo);
+        read_b(Y, 0, b_0);
+        issue_range(X, 0, LOADS, kt + 2);
+        mma_half(1, a_hi, b_1);
+        pin_group(LOADS);
     };
 
     const int k_tiles = (k_end - k_begin + BK - 1) / BK;
@@ -690,17 +723,17 @@ __global__ void __launch_bounds__(TL::THREADS) grouped_gemm_dtl_kernel(GemmParam
     int kt = 0;
     if (primed) {
         issue_range(lds0, 0, LOADS, 0);
-        issue_range(lds1, 0, PART_A, 1);
+        issue_range(lds1, 0, LOADS, 1);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        read_frags(lds0, 0, af0, bf0);
+        read_a(lds0, 0, 0, a_lo);
+        read_b(lds0, 0, b_0);
         // two steps per turn so that each names its buffers statically; the loop leaves with tile kt complete in
-        // lds0, the first copies of tile kt + 1 under way and at most three more tiles to go
+        // lds0, the copies of tile kt + 1 under way and at most three more tiles to go
         for (; kt + 3 < n_full; kt += 2) {
             pipe_step(kt, lds0, lds1);
             pipe_step(kt + 1, lds1, lds0);
         }
-        issue_range(lds1, PART_A, LOADS, kt + 1);
     } else {
         if (k_tiles > 0) issue(0, lds0);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -716,7 +749,7 @@ __global__ void __launch_bounds__(TL::THREADS) grouped_gemm_dtl_kernel(GemmParam
     }
 
     // ---- epilogue -----------------------------------------------------------------------------------
-    // Accumulators (lane: column lane % 32, rows 8 * (r / 4) + 4 * (lane / 32) + r % 4 of each 32x32 tile) are
+    // Accumulators (lane: column lane % 16, rows 4 * (lane / 16) + r of each 16x16 tile) are
     // rounded and staged in LDS - the upper half of the rows in one stage buffer, the lower half in the other -
     // then written out as 16-byte packets along rows, rows going to their mapped position.
     const int lane = opaque(lane_id());
@@ -726,9 +759,9 @@ __global__ void __launch_bounds__(TL::THREADS) grouped_gemm_dtl_kernel(GemmParam
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int row = i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);  // inside this half
-                const int col = wn * (BN / WN) + j * 32 + lane % 32;
+            for (int r = 0; r < 4; ++r) {
+                const int row = i * 16 + 4 * (lane / 16) + r;  // inside this half
+                const int col = wn * (BN / WN) + j * 16 + lane % 16;
                 Ch[row * C_LD + col] = T::down(acc[i][j][r]);
             }
     __syncthreads();
@@ -848,7 +881,7 @@ void launch_mfma(const ck::GemmParams& p, hipStream_t s) {
         hipLaunchKernelGGL((ck::grouped_gemm_kernel<T, MainTile, B_KC, GROUP_K>), dim3((unsigned)grid),
                            dim3(MainTile::THREADS), 0, s, p);
     else
-        hipLaunchKernelGGL((ck::grouped_gemm_dtl_kernel<T, MainTile, B_KC, GROUP_K>), dim3((unsigned)grid),
+        hipLaunchKernelGGL((ck::grouped_gemm_m16_kernel<T, MainTile, B_KC, GROUP_K>), dim3((unsigned)grid),
                            dim3(MainTile::THREADS), 0, s, p);
 }
 
