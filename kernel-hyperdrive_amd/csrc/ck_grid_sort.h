@@ -58,9 +58,11 @@ __device__ __forceinline__ void grid_sort_histogram(GridSortShared& sh, int n, i
 }
 
 // in place: hist[k] <- sum of hist[0 .. k-1], k over nbins * num_waves entries; one workgroup of 1024 lanes.
-// Each wave owns a contiguous slice and walks it 64 entries at a time (coalesced), kScanAhead batches being
-// requested together; a first sweep gives the slice totals, the second writes the exclusive sums.
+// Each wave owns a contiguous slice and walks it 64 entries at a time (coalesced).  A slice of up to
+// 64 * kScanHeld entries is read once, all batches requested together, and scanned out of registers; longer
+// slices take two sweeps of kScanAhead batches (totals first, exclusive sums second).
 constexpr int kScanAhead = 8;
+constexpr int kScanHeld = 32;
 __device__ __forceinline__ void grid_sort_scan(uint32_t* __restrict__ hist, int total) {
     __shared__ uint32_t wave_total[16];
     const int lane = lane_id();
@@ -68,6 +70,31 @@ __device__ __forceinline__ void grid_sort_scan(uint32_t* __restrict__ hist, int 
     const int per_wave = ((total + 15) / 16 + CK_WAVE - 1) / CK_WAVE * CK_WAVE;
     const int begin = min(wave * per_wave, total);
     const int end = min(begin + per_wave, total);
+    if (per_wave <= CK_WAVE * kScanHeld) {
+        uint32_t v[kScanHeld];
+        uint32_t sum = 0;
+#pragma unroll
+        for (int u = 0; u < kScanHeld; ++u) {
+            const int i = begin + u * CK_WAVE + lane;
+            v[u] = i < end ? hist[i] : 0u;
+        }
+#pragma unroll
+        for (int u = 0; u < kScanHeld; ++u) sum += v[u];
+        sum = (uint32_t)wave_sum_i((int)sum);
+        if (lane == 0) wave_total[wave] = sum;
+        __syncthreads();
+        uint32_t carry = 0;
+        for (int w = 0; w < wave; ++w) carry += wave_total[w];
+#pragma unroll
+        for (int u = 0; u < kScanHeld; ++u) {
+            const int i = begin + u * CK_WAVE + lane;
+            if (begin + u * CK_WAVE >= end) break;  // wave-uniform
+            const uint32_t incl = (uint32_t)wave_inclusive_scan_i((int)v[u]);
+            if (i < end) hist[i] = carry + incl - v[u];
+            carry += __shfl(incl, CK_WAVE - 1, CK_WAVE);
+        }
+        return;
+    }
     uint32_t sum = 0;
     for (int g0 = begin; g0 < end; g0 += CK_WAVE * kScanAhead) {
 #pragma unroll

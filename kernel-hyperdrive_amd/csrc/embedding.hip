@@ -308,8 +308,8 @@ __global__ void __launch_bounds__(256)
 // ---- backward 3: add up the partial rows of long runs ------------------------------------------------
 // Workgroup (g, part) looks at the 64 sorted slots [64 g, 64 g + 64): the slots that head a run longer than kChunk
 // are found with one coalesced look, then the whole workgroup sums, for each of them in turn, the partial rows
-// of the run over its quarter (`part`) of the columns.
-constexpr int kCombineParts = 4;
+// of the run over its share (`part`) of the columns, eight partial rows in flight per lane.
+constexpr int kCombineParts = 16;
 
 template <typename T>
 __global__ void __launch_bounds__(256)
@@ -349,15 +349,12 @@ __global__ void __launch_bounds__(256)
         for (int64_t c = c0 + threadIdx.x; c < c1; c += 256) {
             acc_t acc = (acc_t)partial[first_slot * H + c];
             int k = 1;
-            for (; k + 3 < chunks; k += 4) {
-                const float v0 = partial[2 * (int64_t)((i + k * kChunk) / kChunk) * H + c];
-                const float v1 = partial[2 * (int64_t)((i + (k + 1) * kChunk) / kChunk) * H + c];
-                const float v2 = partial[2 * (int64_t)((i + (k + 2) * kChunk) / kChunk) * H + c];
-                const float v3 = partial[2 * (int64_t)((i + (k + 3) * kChunk) / kChunk) * H + c];
-                acc += (acc_t)v0;
-                acc += (acc_t)v1;
-                acc += (acc_t)v2;
-                acc += (acc_t)v3;
+            for (; k + 7 < chunks; k += 8) {
+                float v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) v[u] = partial[2 * (int64_t)((i + (k + u) * kChunk) / kChunk) * H + c];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) acc += (acc_t)v[u];
             }
             for (; k < chunks; ++k) acc += (acc_t)partial[2 * (int64_t)((i + k * kChunk) / kChunk) * H + c];
             dw[(int64_t)id * H + c] = T::down((float)acc);
