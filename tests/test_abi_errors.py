@@ -1,0 +1,107 @@
+"""Error behaviour of the C ABI: every entry point validates its arguments before it touches the GPU and reports a
+status code instead of launching.  These calls reach no HIP runtime function, so they run without a GPU.
+
+The reference raises from Python asserts / AT_DISPATCH for the same mistakes (cute_kernels/kernels/swiglu/__init__.py:23-24,
+include/dtypes/common.h:8-14); here the library reports them as ck_status values that the binding turns into
+RuntimeError."""
+
+import ctypes
+
+import pytest
+
+OK, DTYPE, SHAPE, NULL, WORKSPACE, LAUNCH, ALIGN = range(7)
+F32, F16, BF16 = 0, 1, 2
+P = 0x10000  # a well-aligned non-null "device pointer"; no call below gets as far as using it
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from cute_kernels import _C
+
+    return _C.load_library()
+
+
+def test_status_strings(lib):
+    texts = [lib.ck_status_string(i) for i in range(7)]
+    assert texts[0] == b"ok" and len(set(texts)) == 7
+    assert lib.ck_status_string(99)  # unknown codes still give a string
+
+
+def test_swiglu_argument_checks(lib):
+    assert lib.ck_swiglu_forward(P, P, P, -1, BF16, 256, None) == SHAPE
+    assert lib.ck_swiglu_forward(P, P, P, 64, BF16, 100, None) == SHAPE  # workgroup size not a multiple of 64
+    assert lib.ck_swiglu_forward(P, P, P, 64, 7, 256, None) == DTYPE
+    assert lib.ck_swiglu_forward(None, P, P, 64, BF16, 256, None) == NULL
+    assert lib.ck_swiglu_forward(P + 1, P, P, 64, BF16, 256, None) == ALIGN
+    assert lib.ck_swiglu_backward(P, P, P, None, P, 64, BF16, 256, None) == NULL
+    assert lib.ck_swiglu_unchunked_forward(P, P, 4, 7, BF16, 256, None) == SHAPE  # odd last dimension
+    assert lib.ck_swiglu_unchunked_backward(P, None, P, 4, 8, BF16, 256, None) == NULL
+    assert lib.ck_swiglu_forward(None, None, None, 0, BF16, 256, None) == OK  # nothing to do
+
+
+def test_rmsnorm_argument_checks(lib):
+    assert lib.ck_rmsnorm_forward(P, None, P, None, 4, 65537, 1e-5, BF16, None) == SHAPE  # H above the limit
+    assert lib.ck_rmsnorm_forward(None, None, P, None, 4, 64, 1e-5, BF16, None) == NULL
+    assert lib.ck_rmsnorm_forward(P, None, P, None, 4, 64, 1e-5, 9, None) == DTYPE
+    assert lib.ck_rmsnorm_backward(P, P, P, None, P, None, P, 1 << 30, 4, 64, 1e-5, BF16, None) == NULL  # weight, no weight_grad
+    assert lib.ck_rmsnorm_backward(P, P, P, None, P, P, None, 0, 4, 64, 1e-5, BF16, None) == WORKSPACE
+    need = lib.ck_rmsnorm_backward_workspace_size(4, 64)
+    assert need > 0
+    assert lib.ck_rmsnorm_backward(P, P, P, None, P, P, P, need - 1, 4, 64, 1e-5, BF16, None) == WORKSPACE
+    assert lib.ck_rmsnorm_backward(P, P, P + 2, None, P, P, P, need, 4, 64, 1e-5, F32, None) == ALIGN
+
+
+def test_embedding_argument_checks(lib):
+    assert lib.ck_embedding_forward(P, 0, P, P, -1, 10, 8, BF16, None) == SHAPE
+    assert lib.ck_embedding_forward(None, 0, P, P, 4, 10, 8, BF16, None) == NULL
+    assert lib.ck_embedding_forward(P, 0, P, P, 4, 10, 8, 5, None) == DTYPE
+    assert lib.ck_embedding_backward(P, 0, P, None, P, 1 << 30, 4, 10, 8, BF16, None) == NULL
+    need = lib.ck_embedding_backward_workspace_size(4, 10, 8)
+    assert lib.ck_embedding_backward(P, 0, P, P, P, need - 1, 4, 10, 8, BF16, None) == WORKSPACE
+    assert lib.ck_embedding_backward(P, 0, P, P, P + 16, need, 4, 10, 8, BF16, None) == WORKSPACE  # 256-byte alignment
+    assert lib.ck_embedding_backward(P, 0, P, P, P, need, 4, 0, 8, BF16, None) == OK  # empty table
+
+
+def test_routing_argument_checks(lib):
+    assert lib.ck_contiguous_count(P, 0, None, 4, 8, None) == NULL
+    assert lib.ck_contiguous_count(P, 0, P, -1, 8, None) == SHAPE
+    assert lib.ck_moe_sort(P, 0, P, P, P, None, 0, 10, 0, None) == SHAPE  # no experts
+    assert lib.ck_moe_sort(P, 0, P, P, None, None, 0, 10, 8, None) == NULL
+    need = lib.ck_moe_sort_workspace_size(1000, 1000)
+    assert need > 0
+    assert lib.ck_moe_sort(P, 0, P, P, P, P, need - 1, 1000, 1000, None) == WORKSPACE
+    assert lib.ck_offsets_from_sorted(None, P, 4, 8, None) == NULL
+    assert lib.ck_offsets_from_sorted(P, P, 4, 0, None) == SHAPE
+
+
+def test_grouped_gemm_argument_checks(lib):
+    s2s = lib.ck_scatter2scatter
+    #        X  ldx W  se    sk sn idx off out ldo slots K  N  E  fan xg yg dtype stream
+    assert s2s(P, 64, P, 4096, 1, 64, P, P, P, 64, 16, 64, 64, 0, 1, 0, 1, BF16, None) == SHAPE  # E = 0
+    assert s2s(P, 64, P, 4096, 1, 64, P, P, P, 64, 16, 64, 64, 2, 0, 0, 1, BF16, None) == SHAPE  # fan_out = 0
+    assert s2s(P, 64, P, 4096, 1, 64, P, P, P, 64, 16, 64, 64, 2, 1, 0, 1, 3, None) == DTYPE
+    assert s2s(P, 64, P, 4096, 1, 64, P, None, P, 64, 16, 64, 64, 2, 1, 0, 1, BF16, None) == NULL  # no offsets
+    assert s2s(P, 64, P, 4096, 1, 64, None, P, P, 64, 16, 64, 64, 2, 1, 0, 1, BF16, None) == NULL  # gather without index
+    assert s2s(P + 1, 64, P, 4096, 1, 64, P, P, P, 64, 16, 64, 64, 2, 1, 0, 1, BF16, None) == ALIGN
+    assert s2s(P, 64, P, 4096, 1, 64, P, P, P, 64, 0, 64, 64, 2, 1, 0, 1, BF16, None) == OK  # no rows
+    xty = lib.ck_group_bwd_W
+    #        DY ldy X  ldx off DW se    sk  sn M   K   N   E  dtype stream
+    assert xty(P, 64, P, 64, P, P, 4096, 64, 1, 16, 64, 64, 0, BF16, None) == SHAPE
+    assert xty(P, 64, P, 64, P, None, 4096, 64, 1, 16, 64, 64, 2, BF16, None) == NULL
+    assert xty(P, 64, P, 64, None, P, 4096, 64, 1, 16, 64, 64, 2, BF16, None) == NULL
+    assert xty(P, 64, P, 64, P, P, 4096, 64, 1, 16, 64, 64, 2, 4, None) == DTYPE
+    assert lib.ck_group(None, 64, P, None, P, 64, 16, 64, 1, BF16, None) == NULL
+    assert lib.ck_group(P, 64, P, None, P, 64, 16, 64, 0, BF16, None) == SHAPE
+    assert lib.ck_moe_combine_forward(P, P, P, 16, 0, 64, BF16, None) == SHAPE  # k = 0
+    assert lib.ck_moe_combine_forward(P, None, P, 16, 2, 64, BF16, None) == NULL
+    assert lib.ck_moe_combine_backward_gates(P, P, None, 16, 2, 64, BF16, None) == NULL
+    assert lib.ck_probe_mfma(None, 10, 1, P, None) == NULL
+    assert lib.ck_probe_mfma(P, 10, 0, P, None) == SHAPE
+
+
+def test_binding_turns_a_status_into_an_exception():
+    from cute_kernels import _C
+
+    with pytest.raises(RuntimeError, match="ck_swiglu_forward"):
+        _C._check(SHAPE, "ck_swiglu_forward")
+    _C._check(OK, "anything")
