@@ -134,6 +134,36 @@ int ck_scatter2scatter(const void* X, int64_t x_stride, const void* W, int64_t w
                        int64_t K, int64_t N, int64_t E, int64_t fan_out, int x_grouped, int y_grouped,
                        int dtype, void* stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * scatter2scatter with the SwiGLU of the MoE layer in its epilogue.
+ * replaces, in one launch each, the pairs of calls the reference layer makes around its activation
+ * (scattermoe/triton_implementation/__init__.py:83-87: c_fc then self.act; and, in the backward,
+ * ops.py:240-250 of c_proj followed by swiglu_unchunked's backward,
+ * swiglu_unchunked/torch_implementation.py:5-7 being the activation):
+ *
+ *   ck_scatter2scatter_glu:      h[i, :]   = X[in_row(i), :] @ W[e(i)]          W view [E, K, 2I]
+ *                                act[i, c] = h[i, c] * silu(h[i, I + c])        c in [0, I)
+ *   ck_scatter2scatter_glu_bwd:  d_act[i, :] = DY[i, :] @ W[e(i)]               W view [E, K, I]
+ *                                d_h[i, c]     = d_act[i, c] * silu(h[i, I + c])
+ *                                d_h[i, I + c] = d_act[i, c] * h[i, c] * silu'(h[i, I + c])
+ *
+ * Output rows are in sorted-slot order (y_grouped); in the backward so are the rows of DY.  h and d_act are
+ * rounded to the storage type before the activation sees them, so the results equal those of the separate
+ * calls bit for bit.  Shapes the fused kernels do not take (fp32, I not a multiple of 128 / of 8, odd
+ * strides) run as ck_scatter2scatter followed by an element-wise pass, with the same results; d_act then
+ * passes through the first half of each d_h row, so d_h must not alias h.
+ * Strides are in elements; in_row(i), e(i), expert_offsets as for ck_scatter2scatter.
+ * ------------------------------------------------------------------------------------------- */
+int ck_scatter2scatter_glu(const void* X, int64_t x_stride, const void* W, int64_t w_stride_e,
+                           int64_t w_stride_k, int64_t w_stride_n, const int64_t* sorted_scattered_idxs,
+                           const int64_t* expert_offsets, void* h, int64_t h_stride, void* act,
+                           int64_t act_stride, int64_t num_slots, int64_t K, int64_t I, int64_t E,
+                           int64_t fan_out, int x_grouped, int dtype, void* stream);
+int ck_scatter2scatter_glu_bwd(const void* DY, int64_t dy_stride, const void* W, int64_t w_stride_e,
+                               int64_t w_stride_k, int64_t w_stride_n, const int64_t* expert_offsets,
+                               const void* h, int64_t h_stride, void* d_h, int64_t d_h_stride,
+                               int64_t num_slots, int64_t K, int64_t I, int64_t E, int dtype, void* stream);
+
 /* Inclusive expert offsets from already-sorted expert ids (int64 [M] -> int64 [E]); used when a caller
  * of cute::scatter2scatter has the sorted ids but not the offsets (ops.py:16-24 takes only the ids). */
 int ck_offsets_from_sorted(const int64_t* sorted_expert_idxs, int64_t* expert_offsets, int64_t M, int64_t E,

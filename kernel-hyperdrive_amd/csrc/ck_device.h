@@ -136,13 +136,29 @@ __device__ __forceinline__ float sigmoidf_<F32>(float x) {
     const float s = 1.0f / (1.0f + e);
     return x >= 0.f ? s : 1.0f - s;
 }
+// (v_rcp_f32 is good to 1 ulp of fp32, far below what a 16-bit result keeps; a correctly rounded division
+// costs ten more instructions per element, which shows where the activation runs in a GEMM epilogue)
 template <>
 __device__ __forceinline__ float sigmoidf_<F16>(float x) {
-    return __frcp_rn(1.0f + __expf(-x));
+    return __builtin_amdgcn_rcpf(1.0f + __expf(-x));
 }
 template <>
 __device__ __forceinline__ float sigmoidf_<BF16>(float x) {
-    return __frcp_rn(1.0f + __expf(-x));
+    return __builtin_amdgcn_rcpf(1.0f + __expf(-x));
+}
+
+// SwiGLU of one element, y = up * gate * sigmoid(gate), and its derivatives
+// (cute_kernels/kernels/swiglu/README.md:3-13); shared by the streaming kernels and the GEMM epilogues.
+template <typename T>
+__device__ __forceinline__ float swiglu_fwd_1(float g, float u) {
+    return u * g * sigmoidf_<T>(g);
+}
+template <typename T>
+__device__ __forceinline__ void swiglu_bwd_1(float g, float u, float dy, float& dg, float& du) {
+    const float s = sigmoidf_<T>(g);
+    const float gs = g * s;
+    dg = dy * u * (s + gs * (1.0f - s));
+    du = dy * gs;
 }
 
 }  // namespace ck

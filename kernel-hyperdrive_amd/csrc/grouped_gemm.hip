@@ -63,6 +63,12 @@ struct GemmParams {
     int fan_out, x_grouped, y_grouped;
     int m_tiles, n_tiles;    // S2S: upper bound of row tiles; XTY: tiles along I
     int wide;                // operands too large for 32-bit byte offsets inside a tile's source
+    // SwiGLU fused into the epilogue (kernel template argument GLU):
+    //   1: C = h [slots, 2 * glu_half] (up | gate halves), aux = act [slots, glu_half] written as well
+    //   2: the product is d_act (N = glu_half columns), aux = h read, C = d_h [slots, 2 * glu_half] written
+    void* aux;
+    int64_t ld_aux;
+    int glu_half;
 };
 
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -412,7 +418,7 @@ __device__ __forceinline__ uint64_t opaque_s64(uint64_t v) {  // same for a wave
     return v;
 }
 
-template <typename T, typename TL, bool B_KC, bool GROUP_K>
+template <typename T, typename TL, bool B_KC, bool GROUP_K, int GLU = 0>
 // Two waves per SIMD is all the LDS footprint allows; telling the compiler keeps it from spilling to reach a
 // higher occupancy that cannot happen.
 __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
@@ -465,8 +471,12 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
         row_start = 0;
         rows_valid = min(BM, p.K - i_base);
     }
-    const int n_base = nt * BN;
-    const int cols_valid = min(BN, p.N - n_base);  // > 0 and a multiple of 8
+    static_assert(GLU == 0 || !GROUP_K, "the fused activation belongs to the per-expert products");
+    static_assert(GLU != 1 || B_KC, "the forward fusion reads the weight with the contraction contiguous");
+    // GLU == 1: a tile holds BN / 2 "up" columns n_base .. and the BN / 2 "gate" columns glu_half + n_base ..
+    // that pair with them (glu_half is a multiple of BN / 2, checked by the host)
+    const int n_base = GLU == 1 ? nt * (BN / 2) : nt * BN;
+    const int cols_valid = GLU == 1 ? BN : min(BN, p.N - n_base);  // > 0 and a multiple of 8
 
     // ---- global sources of the LDS slots this lane fills ---------------------------------------------
     // address = wave-uniform base of the tile (scalar registers, advanced by a fixed step per tile) + a 32-bit
@@ -503,7 +513,8 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
             BOp::slot_source((wave * BOp::IPW + j) * CK_WAVE + lane, line, chunk);
             if (B_KCC) {
                 const int r = min(line, cols_valid - 1);
-                b_voff[j] = (uint32_t)(((int64_t)(n_base + r) * p.ldb + chunk * 8) * 2);
+                const int w_row = (GLU == 1 && r >= BN / 2) ? p.glu_half + n_base + r - BN / 2 : n_base + r;
+                b_voff[j] = (uint32_t)(((int64_t)w_row * p.ldb + chunk * 8) * 2);
             } else {
                 const int cc = (chunk * 8 < cols_valid) ? chunk * 8 : 0;
                 b_voff[j] = (uint32_t)(((int64_t)line * p.ldb + cc) * 2);
@@ -766,7 +777,9 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
             }
     __syncthreads();
     S* Cbase = reinterpret_cast<S*>(p.C) + (GROUP_K ? (int64_t)expert * p.c_stride_e : 0);
-    constexpr int C_CHUNKS_PER_ROW = BN / 8;
+    typedef VPack<T, 8> P8;
+    // GLU == 1: a lane takes an "up" packet together with its "gate" packet, so packets are counted over half a row
+    constexpr int C_CHUNKS_PER_ROW = (GLU == 1 ? BN / 2 : BN) / 8;
     constexpr int C_CH = BM * C_CHUNKS_PER_ROW / THREADS;
 #pragma unroll
     for (int i = 0; i < C_CH; ++i) {
@@ -782,7 +795,39 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
                 out_row = p.y_grouped ? slot : p.row_idx[slot];
             }
             const S* src = reinterpret_cast<const S*>(row < BM / 2 ? lds0 : lds1) + (row % (BM / 2)) * C_LD + col;
-            *reinterpret_cast<u32x4_t*>(Cbase + out_row * p.ldc + n_base + col) = *reinterpret_cast<const u32x4_t*>(src);
+            if (GLU == 0) {
+                *reinterpret_cast<u32x4_t*>(Cbase + out_row * p.ldc + n_base + col) = *reinterpret_cast<const u32x4_t*>(src);
+            } else if (GLU == 1) {
+                // columns [0, BN / 2) of the tile are "up", [BN / 2, BN) the matching "gate": both go to h, and the
+                // activation is computed from the rounded values exactly as the separate kernel would from h
+                const P8 u = *reinterpret_cast<const P8*>(src);
+                const P8 g = *reinterpret_cast<const P8*>(src + BN / 2);
+                P8 y;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) y.v[e] = T::down(swiglu_fwd_1<T>(T::up(g.v[e]), T::up(u.v[e])));
+                S* hrow = Cbase + out_row * p.ldc + n_base + col;
+                *reinterpret_cast<P8*>(hrow) = u;
+                *reinterpret_cast<P8*>(hrow + p.glu_half) = g;
+                *reinterpret_cast<P8*>(reinterpret_cast<S*>(p.aux) + out_row * p.ld_aux + n_base + col) = y;
+            } else {
+                // the staged tile is d_act (rounded, as the separate kernels would hand it over); h supplies up
+                // and gate of the same positions, and d_h receives both derivatives
+                const S* hrow = reinterpret_cast<const S*>(p.aux) + out_row * p.ld_aux + n_base + col;
+                const P8 u = nt_load(reinterpret_cast<const P8*>(hrow));
+                const P8 g = nt_load(reinterpret_cast<const P8*>(hrow + p.glu_half));
+                const P8 d = *reinterpret_cast<const P8*>(src);
+                P8 du, dg;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    float fg, fu;
+                    swiglu_bwd_1<T>(T::up(g.v[e]), T::up(u.v[e]), T::up(d.v[e]), fg, fu);
+                    dg.v[e] = T::down(fg);
+                    du.v[e] = T::down(fu);
+                }
+                S* drow = Cbase + out_row * p.ldc + n_base + col;
+                *reinterpret_cast<P8*>(drow) = du;
+                *reinterpret_cast<P8*>(drow + p.glu_half) = dg;
+            }
         }
     }
 }
@@ -862,6 +907,35 @@ __global__ void __launch_bounds__(256)
     }
 }
 
+// ---- SwiGLU passes for the shapes the fused epilogues do not take ------------------------------------------
+// act[r][c] = swiglu(up = h[r][c], gate = h[r][half + c]); one lane per element.
+template <typename T>
+__global__ void __launch_bounds__(256)
+    glu_rows_fwd_kernel(const typename T::storage_t* __restrict__ h, int64_t ldh, typename T::storage_t* __restrict__ act,
+                        int64_t ld_act, int64_t rows, int64_t half) {
+    const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t r = blockIdx.y;
+    if (c >= half) return;
+    for (int64_t row = r; row < rows; row += gridDim.y)
+        act[row * ld_act + c] = T::down(swiglu_fwd_1<T>(T::up(h[row * ldh + half + c]), T::up(h[row * ldh + c])));
+}
+// d_h[r][c] holds d_act[r][c] on entry; on exit d_h[r][c] = d_up and d_h[r][half + c] = d_gate.  Every lane
+// reads its own element before it writes, so the pass works in place.
+template <typename T>
+__global__ void __launch_bounds__(256)
+    glu_rows_bwd_kernel(const typename T::storage_t* __restrict__ h, int64_t ldh, typename T::storage_t* d_h, int64_t ld_dh,
+                        int64_t rows, int64_t half) {
+    const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t r = blockIdx.y;
+    if (c >= half) return;
+    for (int64_t row = r; row < rows; row += gridDim.y) {
+        float dg, du;
+        swiglu_bwd_1<T>(T::up(h[row * ldh + half + c]), T::up(h[row * ldh + c]), T::up(d_h[row * ld_dh + c]), dg, du);
+        d_h[row * ld_dh + c] = T::down(du);
+        d_h[row * ld_dh + half + c] = T::down(dg);
+    }
+}
+
 }  // namespace ck
 
 // ---- host side ------------------------------------------------------------------------------
@@ -883,6 +957,15 @@ void launch_mfma(const ck::GemmParams& p, hipStream_t s) {
     else
         hipLaunchKernelGGL((ck::grouped_gemm_m16_kernel<T, MainTile, B_KC, GROUP_K>), dim3((unsigned)grid),
                            dim3(MainTile::THREADS), 0, s, p);
+}
+
+// per-expert product with the SwiGLU epilogue GLU (1: forward, 2: backward); never the wide kernel
+template <typename T, bool B_KC, int GLU>
+void launch_mfma_glu(const ck::GemmParams& p, hipStream_t s) {
+    const int total = p.m_tiles * p.n_tiles;
+    const int grid = (total + 7) / 8 * 8;
+    hipLaunchKernelGGL((ck::grouped_gemm_m16_kernel<T, MainTile, B_KC, false, GLU>), dim3((unsigned)grid),
+                       dim3(MainTile::THREADS), 0, s, p);
 }
 
 bool mult8(int64_t v) { return (v & 7) == 0; }
@@ -946,6 +1029,125 @@ extern "C" int ck_scatter2scatter(const void* X, int64_t x_stride, const void* W
         hipLaunchKernelGGL((ck::s2s_plain_kernel<T>), grid, dim3(256), 0, s, (const S*)X, x_stride, (const S*)W,
                            w_stride_e, w_stride_k, w_stride_n, sorted_scattered_idxs, expert_offsets, (S*)out,
                            out_stride, num_slots, (int)K, (int)N, (int)E, (int)fan_out, x_grouped, y_grouped);
+    });
+    return ck_launch_status();
+}
+
+extern "C" int ck_scatter2scatter_glu(const void* X, int64_t x_stride, const void* W, int64_t w_stride_e,
+                                      int64_t w_stride_k, int64_t w_stride_n, const int64_t* sorted_scattered_idxs,
+                                      const int64_t* expert_offsets, void* h, int64_t h_stride, void* act,
+                                      int64_t act_stride, int64_t num_slots, int64_t K, int64_t I, int64_t E,
+                                      int64_t fan_out, int x_grouped, int dtype, void* stream) {
+    if (num_slots < 0 || K < 0 || I < 0 || E <= 0 || fan_out <= 0) return CK_ERR_SHAPE;
+    if (num_slots > 0x7fffffff || K > 0x7fffffff || I > 0x3fffffff || E > 0x7fffffff) return CK_ERR_SHAPE;
+    if (dtype != CK_F32 && dtype != CK_F16 && dtype != CK_BF16) return CK_ERR_DTYPE;
+    if (num_slots == 0 || I == 0) return CK_OK;
+    if (!h || !act || !expert_offsets || (K > 0 && (!X || !W))) return CK_ERR_NULL;
+    if (!x_grouped && !sorted_scattered_idxs) return CK_ERR_NULL;
+    if (!ck_aligned_elem(X, dtype) || !ck_aligned_elem(W, dtype) || !ck_aligned_elem(h, dtype) ||
+        !ck_aligned_elem(act, dtype))
+        return CK_ERR_ALIGN;
+    hipStream_t s = (hipStream_t)stream;
+    const int64_t N = 2 * I;
+
+    const bool fused = dtype != CK_F32 && K > 0 && w_stride_k == 1 && ck_aligned16(X) && ck_aligned16(W) && mult8(K) &&
+                       mult8(x_stride) && mult8(w_stride_e) && mult8(w_stride_n) && I % (kBN / 2) == 0 &&
+                       ck_aligned16(h) && mult8(h_stride) && ck_aligned16(act) && mult8(act_stride) &&
+                       num_slots * x_stride * 2 < (int64_t)1 << 32 && N * w_stride_n * 2 < (int64_t)1 << 32;
+    if (fused) {
+        ck::GemmParams p = {};
+        p.A = X;
+        p.B = W;
+        p.C = h;
+        p.lda = x_stride;
+        p.ldb = w_stride_n;
+        p.ldc = h_stride;
+        p.b_stride_e = w_stride_e;
+        p.row_idx = sorted_scattered_idxs;
+        p.offsets = expert_offsets;
+        p.M = (int)num_slots;
+        p.N = (int)N;
+        p.K = (int)K;
+        p.E = (int)E;
+        p.fan_out = (int)fan_out;
+        p.x_grouped = x_grouped;
+        p.y_grouped = 1;
+        p.aux = act;
+        p.ld_aux = act_stride;
+        p.glu_half = (int)I;
+        p.m_tiles = (int)(num_slots / kBM + E);
+        p.n_tiles = (int)(I / (kBN / 2));
+        if ((int64_t)p.m_tiles * p.n_tiles > 0x7ffffff0) return CK_ERR_SHAPE;
+        if (dtype == CK_BF16) launch_mfma_glu<ck::BF16, true, 1>(p, s);
+        else launch_mfma_glu<ck::F16, true, 1>(p, s);
+        return ck_launch_status();
+    }
+    const int st = ck_scatter2scatter(X, x_stride, W, w_stride_e, w_stride_k, w_stride_n, sorted_scattered_idxs,
+                                      expert_offsets, h, h_stride, num_slots, K, N, E, fan_out, x_grouped, 1, dtype, stream);
+    if (st != CK_OK) return st;
+    const dim3 grid((unsigned)ck_ceil_div(I, 256), (unsigned)(num_slots < 65535 ? num_slots : 65535));
+    CK_DISPATCH_DTYPE(dtype, {
+        typedef typename T::storage_t S;
+        hipLaunchKernelGGL((ck::glu_rows_fwd_kernel<T>), grid, dim3(256), 0, s, (const S*)h, h_stride, (S*)act, act_stride,
+                           num_slots, I);
+    });
+    return ck_launch_status();
+}
+
+extern "C" int ck_scatter2scatter_glu_bwd(const void* DY, int64_t dy_stride, const void* W, int64_t w_stride_e,
+                                          int64_t w_stride_k, int64_t w_stride_n, const int64_t* expert_offsets,
+                                          const void* h, int64_t h_stride, void* d_h, int64_t d_h_stride,
+                                          int64_t num_slots, int64_t K, int64_t I, int64_t E, int dtype, void* stream) {
+    if (num_slots < 0 || K < 0 || I < 0 || E <= 0) return CK_ERR_SHAPE;
+    if (num_slots > 0x7fffffff || K > 0x7fffffff || I > 0x3fffffff || E > 0x7fffffff) return CK_ERR_SHAPE;
+    if (dtype != CK_F32 && dtype != CK_F16 && dtype != CK_BF16) return CK_ERR_DTYPE;
+    if (num_slots == 0 || I == 0) return CK_OK;
+    if (!h || !d_h || !expert_offsets || (K > 0 && (!DY || !W))) return CK_ERR_NULL;
+    if (!ck_aligned_elem(DY, dtype) || !ck_aligned_elem(W, dtype) || !ck_aligned_elem(h, dtype) ||
+        !ck_aligned_elem(d_h, dtype))
+        return CK_ERR_ALIGN;
+    hipStream_t s = (hipStream_t)stream;
+
+    const bool fused = dtype != CK_F32 && K > 0 && w_stride_n == 1 && ck_aligned16(DY) && ck_aligned16(W) && mult8(K) &&
+                       mult8(dy_stride) && mult8(w_stride_e) && mult8(w_stride_k) && mult8(I) && ck_aligned16(h) &&
+                       mult8(h_stride) && ck_aligned16(d_h) && mult8(d_h_stride) &&
+                       num_slots * dy_stride * 2 < (int64_t)1 << 32 && K * w_stride_k * 2 < (int64_t)1 << 32;
+    if (fused) {
+        ck::GemmParams p = {};
+        p.A = DY;
+        p.B = W;
+        p.C = d_h;
+        p.lda = dy_stride;
+        p.ldb = w_stride_k;
+        p.ldc = d_h_stride;
+        p.b_stride_e = w_stride_e;
+        p.offsets = expert_offsets;
+        p.M = (int)num_slots;
+        p.N = (int)I;
+        p.K = (int)K;
+        p.E = (int)E;
+        p.fan_out = 1;
+        p.x_grouped = 1;
+        p.y_grouped = 1;
+        p.aux = const_cast<void*>(h);
+        p.ld_aux = h_stride;
+        p.glu_half = (int)I;
+        p.m_tiles = (int)(num_slots / kBM + E);
+        p.n_tiles = (int)ck_ceil_div(I, kBN);
+        if ((int64_t)p.m_tiles * p.n_tiles > 0x7ffffff0) return CK_ERR_SHAPE;
+        if (dtype == CK_BF16) launch_mfma_glu<ck::BF16, false, 2>(p, s);
+        else launch_mfma_glu<ck::F16, false, 2>(p, s);
+        return ck_launch_status();
+    }
+    // d_act goes into the first half of every d_h row, then one pass turns the row into (d_up | d_gate) in place
+    const int st = ck_scatter2scatter(DY, dy_stride, W, w_stride_e, w_stride_k, w_stride_n, nullptr, expert_offsets, d_h,
+                                      d_h_stride, num_slots, K, I, E, 1, 1, 1, dtype, stream);
+    if (st != CK_OK) return st;
+    const dim3 grid((unsigned)ck_ceil_div(I, 256), (unsigned)(num_slots < 65535 ? num_slots : 65535));
+    CK_DISPATCH_DTYPE(dtype, {
+        typedef typename T::storage_t S;
+        hipLaunchKernelGGL((ck::glu_rows_bwd_kernel<T>), grid, dim3(256), 0, s, (const S*)h, h_stride, (S*)d_h, d_h_stride,
+                           num_slots, I);
     });
     return ck_launch_status();
 }

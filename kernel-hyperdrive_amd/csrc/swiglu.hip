@@ -12,18 +12,6 @@ namespace ck {
 
 constexpr int kUnroll = 4;  // packets per lane per tensor
 
-template <typename T>
-__device__ __forceinline__ float swiglu_fwd_1(float g, float u) {
-    return u * g * sigmoidf_<T>(g);
-}
-template <typename T>
-__device__ __forceinline__ void swiglu_bwd_1(float g, float u, float dy, float& dg, float& du) {
-    const float s = sigmoidf_<T>(g);
-    const float gs = g * s;
-    dg = dy * u * (s + gs * (1.0f - s));
-    du = dy * gs;
-}
-
 // ---- two-tensor form ---------------------------------------------------------------------
 template <typename T, int VEC>
 __global__ void swiglu_fwd_kernel(const typename T::storage_t* __restrict__ gate,

@@ -53,6 +53,14 @@ _SIGNATURES = {
         _i32,
         [_p, _i64, _p, _i64, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _p],
     ),
+    "ck_scatter2scatter_glu": (
+        _i32,
+        [_p, _i64, _p, _i64, _i64, _i64, _p, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _p],
+    ),
+    "ck_scatter2scatter_glu_bwd": (
+        _i32,
+        [_p, _i64, _p, _i64, _i64, _i64, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _i64, _i32, _p],
+    ),
     "ck_offsets_from_sorted": (_i32, [_p, _p, _i64, _i64, _p]),
     "ck_group_bwd_W": (_i32, [_p, _i64, _p, _i64, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _p]),
     "ck_group": (_i32, [_p, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _i32, _p]),
@@ -341,6 +349,41 @@ def scatter2scatter(X, W, sorted_scattered_idxs, expert_offsets, out, fan_out: i
                                    out.size(0), X.size(1), out.size(1), W.size(0), fan_out, int(x_grouped),
                                    int(y_grouped), dtype_code(X.dtype), L.stream),
             "ck_scatter2scatter",
+        )
+
+
+def scatter2scatter_glu(X, W, sorted_scattered_idxs, expert_offsets, h, act, fan_out: int, x_grouped: bool) -> None:
+    """h [slots, 2I] = gathered X rows times W [E, K, 2I], act [slots, I] = SwiGLU(h); rows grouped by expert."""
+    lib = load_library()
+    if X.stride(1) != 1 or h.stride(1) != 1 or act.stride(1) != 1:
+        raise ValueError("scatter2scatter_glu needs unit column stride for X, h and act")
+    if h.size(1) != 2 * act.size(1) or h.size(0) != act.size(0):
+        raise ValueError("scatter2scatter_glu: h must be [slots, 2I] and act [slots, I]")
+    flop = 2.0 * h.size(0) * X.size(1) * h.size(1)
+    with _Launch(X, W, sorted_scattered_idxs, expert_offsets, h, act) as L, _Timed("scatter2scatter", flop):
+        _check(
+            lib.ck_scatter2scatter_glu(_ptr(X), X.stride(0), _ptr(W), W.stride(0), W.stride(1), W.stride(2),
+                                       _ptr(sorted_scattered_idxs), _ptr(expert_offsets), _ptr(h), h.stride(0),
+                                       _ptr(act), act.stride(0), h.size(0), X.size(1), act.size(1), W.size(0),
+                                       fan_out, int(x_grouped), dtype_code(X.dtype), L.stream),
+            "ck_scatter2scatter_glu",
+        )
+
+
+def scatter2scatter_glu_bwd(DY, W, expert_offsets, h, d_h) -> None:
+    """d_h [slots, 2I] = SwiGLU'(h) applied to DY [slots, K] times W [E, K, I]; all rows grouped by expert."""
+    lib = load_library()
+    if DY.stride(1) != 1 or h.stride(1) != 1 or d_h.stride(1) != 1:
+        raise ValueError("scatter2scatter_glu_bwd needs unit column stride for DY, h and d_h")
+    if h.shape != d_h.shape or h.size(1) != 2 * W.size(2) or h.size(0) != DY.size(0):
+        raise ValueError("scatter2scatter_glu_bwd: h and d_h must be [slots, 2I] for W [E, K, I]")
+    flop = 2.0 * DY.size(0) * DY.size(1) * W.size(2)
+    with _Launch(DY, W, expert_offsets, h, d_h) as L, _Timed("scatter2scatter", flop):
+        _check(
+            lib.ck_scatter2scatter_glu_bwd(_ptr(DY), DY.stride(0), _ptr(W), W.stride(0), W.stride(1), W.stride(2),
+                                           _ptr(expert_offsets), _ptr(h), h.stride(0), _ptr(d_h), d_h.stride(0),
+                                           DY.size(0), DY.size(1), W.size(2), W.size(0), dtype_code(DY.dtype), L.stream),
+            "ck_scatter2scatter_glu_bwd",
         )
 
 

@@ -11,8 +11,9 @@ import torch
 from ... import _C
 from ...constants import LIBRARY_NAME
 from ...utils import cute_op
+from ..swiglu_unchunked import swiglu_unchunked_cute, swiglu_unchunked_torch
 from .moe_torch import Experts_Torch, MoE_Torch
-from .ops import scattered_experts
+from .ops import scattered_experts, scattered_glu_experts
 
 
 def _moe_sort_fake(expert_ids: torch.Tensor, num_experts: int):
@@ -77,11 +78,33 @@ class Experts_HIP(Experts_Torch):
 
 class MoE_HIP(MoE_Torch):
     experts_class = Experts_HIP
+    # With a SwiGLU between the two expert products, run the activation and its derivative inside the grouped
+    # GEMMs' epilogues (same values, two passes over the intermediate activations fewer).  False keeps the three
+    # separate autograd nodes of the reference layer.
+    fuse_swiglu = True
 
     def _compute_experts(
         self, hidden_states: torch.Tensor, router_weights: torch.Tensor, selected_experts: torch.Tensor
     ) -> torch.Tensor:
         sorted_expert_idxs, sorted_scattered_idxs, expert_offsets = moe_sort(selected_experts, self.num_experts)
+
+        # the fused kernels take 16-bit storage with I a multiple of 128 and H a multiple of 8
+        fusable = (
+            hidden_states.dtype in (torch.float16, torch.bfloat16)
+            and self.intermediate_size % 128 == 0
+            and self.hidden_size % 8 == 0
+        )
+        if self.fuse_swiglu and fusable and self.act in (swiglu_unchunked_cute, swiglu_unchunked_torch):
+            return scattered_glu_experts(
+                hidden_states,
+                self.c_fc.weight.permute(0, 2, 1),
+                self.c_proj.weight.permute(0, 2, 1),
+                self.top_k,
+                sorted_expert_idxs,
+                sorted_scattered_idxs,
+                expert_offsets,
+                router_weights,
+            )
 
         # [T, H] -> rows gathered per expert -> [T * k, I or 2I], grouped by expert
         hidden_states = self.c_fc(

@@ -10,6 +10,11 @@ saved tensors, same nine gradient slots).  Differences that do not change result
     single-pass kernels (``moe_combine_forward`` / ``moe_combine_backward_gates``);
   * the weight gradient is written completely by the kernel (zeros for experts without rows), so it is
     allocated with ``empty_like`` instead of ``zeros_like`` (ops.py:237).
+
+``scattered_glu_experts`` is the whole expert MLP with a SwiGLU in between (c_fc -> swiglu_unchunked -> c_proj,
+triton_implementation/__init__.py:83-98) as one autograd node: the activation and its derivative run in the
+epilogues of the grouped GEMMs that produce their inputs, so neither the activation pass nor d_act exists as a
+separate trip through memory.  Every value is rounded where the separate ops round it.
 """
 
 import torch
@@ -46,6 +51,39 @@ def scatter2scatter(
     if X.stride(1) != 1:
         X = X.contiguous()
     _C.scatter2scatter(X, W, sorted_scattered_idxs, expert_offsets, out, FAN_OUT, x_grouped, y_grouped)
+
+
+@cute_op(f"{LIBRARY_NAME}::scatter2scatter_glu", mutates_args={"h", "act"})
+def scatter2scatter_glu(
+    X: torch.Tensor,
+    W: torch.Tensor,
+    sorted_scattered_idxs: torch.Tensor,
+    expert_offsets: torch.Tensor,
+    h: torch.Tensor,
+    act: torch.Tensor,
+    FAN_OUT: int,
+    x_grouped: bool = False,
+) -> None:
+    """h = scatter2scatter(X, W) with grouped rows, act = swiglu_unchunked(h), in one launch."""
+    assert sorted_scattered_idxs.size(0) == X.size(0) * FAN_OUT
+    assert h.size(0) == sorted_scattered_idxs.size(0) and h.size(1) == W.size(-1)
+    assert act.size(0) == h.size(0) and 2 * act.size(1) == h.size(1)
+    assert X.size(1) == W.size(1)
+    if X.stride(1) != 1:
+        X = X.contiguous()
+    _C.scatter2scatter_glu(X, W, sorted_scattered_idxs, expert_offsets, h, act, FAN_OUT, x_grouped)
+
+
+@cute_op(f"{LIBRARY_NAME}::scatter2scatter_glu_bwd", mutates_args={"d_h"})
+def scatter2scatter_glu_bwd(
+    DY: torch.Tensor, W: torch.Tensor, expert_offsets: torch.Tensor, h: torch.Tensor, d_h: torch.Tensor
+) -> None:
+    """d_h = swiglu_unchunked'(h) applied to d_act = DY @ W per expert (all rows grouped), in one launch."""
+    assert DY.size(0) == h.size(0) and DY.size(1) == W.size(1)
+    assert h.shape == d_h.shape and h.size(1) == 2 * W.size(2)
+    if DY.stride(1) != 1:
+        DY = DY.contiguous()
+    _C.scatter2scatter_glu_bwd(DY, W, expert_offsets, h, d_h)
 
 
 @cute_op(f"{LIBRARY_NAME}::group_bwd_W", mutates_args={"DW"})
@@ -209,6 +247,105 @@ class _ScatteredExperts(torch.autograd.Function):
 
         # x, expert_weights, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, gates, grouped_in, grouped_out
         return d_input, d_weights, None, None, None, None, d_gates, None, None
+
+
+class _ScatteredGLUExperts(torch.autograd.Function):
+    """y = combine(c_proj(swiglu_unchunked(c_fc(x)))) over the routed experts.
+
+    Same values as ``scattered_experts(c_fc) -> swiglu_unchunked -> scattered_experts(c_proj, gates)`` of the
+    reference layer (triton_implementation/__init__.py:83-98 with ops.py:133-263 twice), one node."""
+
+    @staticmethod
+    def forward(ctx, x, w_fc, w_proj, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, gates):
+        # w_fc: view [E, H, 2I] of the [E, 2I, H] parameter; w_proj: view [E, I, H] of the [E, H, I] parameter
+        num_slots = sorted_expert_idxs.size(0)
+        half = w_proj.size(1)
+        h = torch.empty(num_slots, 2 * half, device=x.device, dtype=x.dtype)
+        act = torch.empty(num_slots, half, device=x.device, dtype=x.dtype)
+        scatter2scatter_glu(
+            X=x,
+            W=w_fc,
+            sorted_scattered_idxs=sorted_scattered_idxs,
+            expert_offsets=expert_offsets,
+            h=h,
+            act=act,
+            FAN_OUT=k,
+            x_grouped=False,
+        )
+        expanded = torch.empty(num_slots, w_proj.size(-1), device=x.device, dtype=x.dtype)
+        scatter2scatter(
+            X=act,
+            W=w_proj,
+            sorted_expert_idxs=sorted_expert_idxs,
+            sorted_scattered_idxs=sorted_scattered_idxs,
+            out=expanded,
+            FAN_OUT=1,
+            x_grouped=True,
+            y_grouped=False,
+            expert_offsets=expert_offsets,
+        )
+        expanded = expanded.view(gates.size(0), gates.size(1), expanded.size(-1))
+        output = torch.empty(gates.size(0), expanded.size(-1), device=x.device, dtype=x.dtype)
+        moe_combine_forward(expanded=expanded, gates=gates, out=output)
+        ctx.save_for_backward(
+            x, w_fc, w_proj, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, gates, h, act, expanded
+        )
+        ctx.k = k
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        x, w_fc, w_proj, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, gates, h, act, expanded = (
+            ctx.saved_tensors
+        )
+        k = ctx.k
+        E = w_fc.size(0)
+        grad_out = grad_out.contiguous()
+
+        d_gates = torch.empty_like(gates)
+        moe_combine_backward_gates(expanded=expanded, grad_out=grad_out, d_gates=d_gates)
+        # grad_out rows times their routing weight, in expert-grouped order (over the saved expert outputs)
+        grouped_grad_out = expanded.flatten(0, 1)
+        group(
+            A=grad_out,
+            sorted_expert_idxs=sorted_scattered_idxs,
+            out=grouped_grad_out,
+            coeff=gates.flatten(),
+            fan_out=gates.size(1),
+        )
+
+        d_w_proj = torch.empty_like(w_proj)
+        group_bwd_W(DY=grouped_grad_out, X=act, expert_offsets=expert_offsets, DW=d_w_proj, E=E)
+        # d_act = grouped_grad_out @ w_proj^T never reaches memory: the epilogue turns it into d_h (over act's
+        # companion buffer: h itself is still needed by every tile's epilogue, so d_h is a new buffer)
+        d_h = torch.empty_like(h)
+        scatter2scatter_glu_bwd(DY=grouped_grad_out, W=w_proj.permute(0, 2, 1), expert_offsets=expert_offsets, h=h, d_h=d_h)
+
+        grouped_x = torch.empty(sorted_expert_idxs.size(0), x.size(1), dtype=x.dtype, device=x.device)
+        group(A=x, sorted_expert_idxs=sorted_scattered_idxs, out=grouped_x, fan_out=k)
+        d_w_fc = torch.empty_like(w_fc)
+        group_bwd_W(DY=d_h, X=grouped_x, expert_offsets=expert_offsets, DW=d_w_fc, E=E)
+        d_expanded_input = grouped_x  # reused once the weight gradient has consumed it
+        scatter2scatter(
+            X=d_h,
+            W=w_fc.permute(0, 2, 1),
+            sorted_expert_idxs=sorted_expert_idxs,
+            sorted_scattered_idxs=sorted_scattered_idxs,
+            out=d_expanded_input,
+            FAN_OUT=1,
+            x_grouped=True,
+            y_grouped=False,
+            expert_offsets=expert_offsets,
+        )
+        d_input = d_expanded_input if k == 1 else d_expanded_input.view(x.size(0), k, x.size(1)).sum(-2)
+        # x, w_fc, w_proj, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, gates
+        return d_input, d_w_fc, d_w_proj, None, None, None, None, d_gates
+
+
+def scattered_glu_experts(inputs, w_fc, w_proj, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, gates):
+    return _ScatteredGLUExperts.apply(
+        inputs, w_fc, w_proj, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, gates
+    )
 
 
 def scattered_experts(

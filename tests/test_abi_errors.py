@@ -84,6 +84,21 @@ def test_grouped_gemm_argument_checks(lib):
     assert s2s(P, 64, P, 4096, 1, 64, None, P, P, 64, 16, 64, 64, 2, 1, 0, 1, BF16, None) == NULL  # gather without index
     assert s2s(P + 1, 64, P, 4096, 1, 64, P, P, P, 64, 16, 64, 64, 2, 1, 0, 1, BF16, None) == ALIGN
     assert s2s(P, 64, P, 4096, 1, 64, P, P, P, 64, 0, 64, 64, 2, 1, 0, 1, BF16, None) == OK  # no rows
+    glu = lib.ck_scatter2scatter_glu
+    #        X  ldx W  se    sk sn idx off h  ldh  act lda slots K  I  E  fan xg dtype stream
+    assert glu(P, 64, P, 8192, 1, 64, P, P, P, 128, P, 64, 16, 64, 64, 0, 1, 0, BF16, None) == SHAPE  # E = 0
+    assert glu(P, 64, P, 8192, 1, 64, P, P, P, 128, None, 64, 16, 64, 64, 2, 1, 0, BF16, None) == NULL  # no act
+    assert glu(P, 64, P, 8192, 1, 64, None, P, P, 128, P, 64, 16, 64, 64, 2, 1, 0, BF16, None) == NULL  # gather without index
+    assert glu(P, 64, P, 8192, 1, 64, P, P, P, 128, P, 64, 16, 64, 64, 2, 1, 0, 8, None) == DTYPE
+    assert glu(P, 64, P, 8192, 1, 64, P, P, P, 128, P + 1, 64, 16, 64, 64, 2, 1, 0, BF16, None) == ALIGN
+    assert glu(P, 64, P, 8192, 1, 64, P, P, P, 128, P, 64, 0, 64, 64, 2, 1, 0, BF16, None) == OK  # no rows
+    glu_bwd = lib.ck_scatter2scatter_glu_bwd
+    #            DY ldy W  se    sk  sn off h  ldh  d_h ldd slots K  I  E  dtype stream
+    assert glu_bwd(P, 64, P, 4096, 64, 1, P, P, 128, P, 128, 16, 64, 64, 0, BF16, None) == SHAPE
+    assert glu_bwd(P, 64, P, 4096, 64, 1, P, None, 128, P, 128, 16, 64, 64, 2, BF16, None) == NULL  # no h
+    assert glu_bwd(P, 64, P, 4096, 64, 1, None, P, 128, P, 128, 16, 64, 64, 2, BF16, None) == NULL  # no offsets
+    assert glu_bwd(P, 64, P, 4096, 64, 1, P, P, 128, P, 128, 16, 64, 64, 2, 5, None) == DTYPE
+    assert glu_bwd(P, 64, P, 4096, 64, 1, P, P, 128, P, 128, 16, 64, 0, 2, BF16, None) == OK  # I = 0
     xty = lib.ck_group_bwd_W
     #        DY ldy X  ldx off DW se    sk  sn M   K   N   E  dtype stream
     assert xty(P, 64, P, 64, P, P, 4096, 64, 1, 16, 64, 64, 0, BF16, None) == SHAPE

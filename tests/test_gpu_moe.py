@@ -61,6 +61,76 @@ def test_scatter2scatter(gpu, dtype, w_layout, mode, shape):
     assert torch.equal(out2, out)
 
 
+# ---- grouped products with the SwiGLU in the epilogue ----------------------------------------------------
+GLU_SHAPES = [
+    # T, k, E, K (hidden), I, empty experts
+    (64, 2, 4, 64, 128, ()),       # one column tile, fused both ways
+    (300, 3, 7, 200, 384, (0, 6)),  # several column tiles, partial row tiles, empty experts
+    (700, 2, 3, 256, 1408, ()),    # I = 11 * 128: the backward's last column tile is partial
+    (100, 2, 4, 72, 192, (1,)),    # I not a multiple of 128: forward falls back to two launches
+    (50, 2, 5, 40, 100, ()),       # I not a multiple of 8: both fall back
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape", GLU_SHAPES)
+def test_scatter2scatter_glu(gpu, dtype, shape):
+    """h and act of the fused launch equal, bit for bit, scatter2scatter followed by swiglu_unchunked; the same for
+    d_h of the fused backward against scatter2scatter followed by the activation's backward.  Both are also held
+    to the oracle within the storage type's tolerance."""
+    from cute_kernels import KernelBackend, swiglu_unchunked_cute
+    from cute_kernels.kernels.scattermoe import scatter2scatter, scatter2scatter_glu, scatter2scatter_glu_bwd
+
+    T, k, E, K, I, empty = shape
+    announce("scatter2scatter_glu", dtype, shape)
+    hip = KernelBackend.hip
+    s_e, s_idx, off = routing(T, k, E, 35, empty)
+    M = T * k
+    X = randn((T, K), dtype, 36)
+    W_fc = randn((E, 2 * I, K), dtype, 37, 0.1)   # parameter layout [E, out, in]
+    W_proj = randn((E, K, I), dtype, 38, 0.1)
+    DY = randn((M, K), dtype, 39)
+    Xg, s_eg, s_idxg, offg = X.to(gpu), s_e.to(gpu), s_idx.to(gpu), off.to(gpu)
+    w_fc_view = W_fc.to(gpu).permute(0, 2, 1)      # [E, K, 2I], K contiguous
+    w_projT_view = W_proj.to(gpu)                  # as the backward sees it: [E, K, I], I contiguous
+
+    # forward
+    h = torch.full((M, 2 * I), float("nan"), dtype=dtype, device=gpu)
+    act = torch.full((M, I), float("nan"), dtype=dtype, device=gpu)
+    scatter2scatter_glu(Xg, w_fc_view, s_idxg, offg, h, act, k, False)
+    h_ref = torch.empty_like(h)
+    scatter2scatter(Xg, w_fc_view, s_eg, s_idxg, h_ref, k, False, True, offg)
+    h_leaf = h_ref.clone().requires_grad_(True)
+    act_ref = swiglu_unchunked_cute(h_leaf, hip, hip, 256, 64, 256, 64)
+    # where the fused kernels run the results are those of the separate calls bit for bit; the two-launch
+    # fallbacks (fp32, I not a multiple of 128 resp. 8) may round the last step differently
+    fused_fwd = dtype != torch.float32 and I % 128 == 0 and K % 8 == 0
+    fused_bwd = dtype != torch.float32 and I % 8 == 0 and K % 8 == 0
+    assert torch.equal(h, h_ref), "h"
+    if fused_fwd:
+        assert torch.equal(act, act_ref.detach()), "act"
+    else:
+        assert_close(act, act_ref.detach(), dtype, "act")
+    expected_h = O.scatter2scatter(X, W_fc.permute(0, 2, 1), s_idx, off, k, False, True, acc_dtype(dtype))
+    assert_close(h, expected_h, dtype, "h against the oracle")
+    assert_close(act, O.swiglu_unchunked_forward(h.cpu(), acc_dtype(dtype)).to(dtype), dtype, "act against the oracle")
+
+    # backward
+    d_h = torch.full((M, 2 * I), float("nan"), dtype=dtype, device=gpu)
+    scatter2scatter_glu_bwd(DY.to(gpu), w_projT_view, offg, h, d_h)
+    d_act_ref = torch.empty(M, I, dtype=dtype, device=gpu)
+    scatter2scatter(DY.to(gpu), w_projT_view, s_eg, s_idxg, d_act_ref, 1, True, True, offg)
+    act_ref.backward(d_act_ref)
+    if fused_bwd:
+        assert torch.equal(d_h, h_leaf.grad), "d_h"
+    else:
+        assert_close(d_h, h_leaf.grad, dtype, "d_h")
+    expected_d_act = O.scatter2scatter(DY, W_proj, s_idx, off, 1, True, True, acc_dtype(dtype))
+    assert_close(d_act_ref, expected_d_act, dtype, "d_act against the oracle")
+    expected_d_h = O.swiglu_unchunked_backward(h.cpu(), d_act_ref.cpu(), acc_dtype(dtype)).to(dtype)
+    assert_close(d_h, expected_d_h, dtype, "d_h against the oracle")
+
+
 # ---- group_bwd_W --------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("dw_layout", ["k_contiguous", "n_contiguous"])
@@ -212,6 +282,33 @@ def test_moe_layer_against_oracle(gpu, dtype, case):
         tol = O.tolerance(dtype)
         for key in ("y", "dx", "dw_fc", "dw_proj"):
             assert O.fraction_outside(got[key], exact[key], **tol) < (2e-3 if k <= 4 else 5e-3), key  # more terms per row at top-6
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case", MOE_CASES + [("intermediate_192", 300, 128, 192, 4, 2, None),
+                                              ("intermediate_100", 90, 64, 100, 3, 2, None)],
+                         ids=[c[0] for c in MOE_CASES] + ["intermediate_192", "intermediate_100"])
+def test_moe_layer_fused_swiglu_equals_separate_ops(gpu, dtype, case):
+    """The layer with the activation inside the GEMM epilogues (the default) against the same layer running
+    c_fc, swiglu_unchunked and c_proj as separate autograd nodes, as the reference layer does: every output and
+    gradient bit for bit, since each value is rounded at the same places.  (fp32 and intermediate sizes that are
+    not a multiple of 128 take the separate nodes either way.)"""
+    from cute_kernels import MoE_Triton
+
+    name, T, H, I, E, k, skew = case
+    announce("moe fused / separate", dtype, case)
+    x, w_gate, w_fc, w_proj, dy = O.moe_inputs(T, H, I, E, dtype, seed=63)
+    if skew is not None:
+        w_gate, x = O.skewed_router(w_gate, x, 1.2, seed=64, scale=skew)
+    fused = build_moe(MoE_Triton, gpu, dtype, E, k, H, I, w_gate, w_fc, w_proj)
+    separate = build_moe(MoE_Triton, gpu, dtype, E, k, H, I, w_gate, w_fc, w_proj)
+    separate.fuse_swiglu = False
+    assert fused.fuse_swiglu
+    got, selected = run_moe(fused, x, dy, gpu)
+    ref, selected_ref = run_moe(separate, x, dy, gpu)
+    assert torch.equal(selected, selected_ref)
+    for key in got:
+        assert torch.equal(got[key], ref[key]), f"{name}/{key}"
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
