@@ -4,9 +4,9 @@
 //   a "team" of TPR lanes (64, 256 or 1024) owns one row at a time and keeps it in registers, so x (and
 //   dy) are read from HBM exactly once.  Row sums use wave64 shuffles; teams wider than a wave finish
 //   through a few LDS floats.  Backward is persistent: each team walks rows team, team+teams, ... and
-//   accumulates its share of dweight in fp32 registers, writes one fp32 partial row to the workspace,
-//   and a second kernel sums the partial rows column-wise with shuffles.  No atomics anywhere, so
-//   dweight is deterministic for a given team count.
+//   accumulates its share of dweight in fp32 registers; the teams of a workgroup add their shares up through
+//   LDS and write one fp32 partial row per workgroup to the workspace, and a second kernel sums the partial
+//   rows column-wise with shuffles.  No atomics anywhere, so dweight is deterministic for a given team count.
 // Generic path (any H, any element alignment): one 256-lane team per row re-reading the row from cache,
 //   and a column kernel for the dweight partials.
 #include "ck_device.h"
@@ -260,7 +260,12 @@ __global__ void __launch_bounds__(TPR > 256 ? TPR : 256)
     }
 
     if (HAS_W) {
-        float* out = dw_partial + (int64_t)team * H;
+        // One partial row per workgroup.  With one wave per row a workgroup holds four teams: their rows are added
+        // up through LDS first (in team order), which quarters what the reduce pass has to read.
+        constexpr int kTeams = TPR == 64 ? 4 : 1;
+        constexpr int kCols = TPR == 64 ? 64 * kMaxPacks * T::kVec : 4;
+        __shared__ float comb[kTeams > 1 ? kTeams * kCols : 4];
+        float* out = kTeams > 1 ? comb + (threadIdx.x / TPR) * kCols : dw_partial + (int64_t)team * H;
 #pragma unroll
         for (int i = 0; i < kMaxPacks; ++i) {
             const int p = t + i * TPR;
@@ -270,6 +275,22 @@ __global__ void __launch_bounds__(TPR > 256 ? TPR : 256)
                     float4 v = make_float4(dw[i][j], dw[i][j + 1], dw[i][j + 2], dw[i][j + 3]);
                     *reinterpret_cast<float4*>(out + p * T::kVec + j) = v;
                 }
+            }
+        }
+        if (kTeams > 1) {
+            __syncthreads();
+            float* row = dw_partial + (int64_t)blockIdx.x * H;
+            for (int c = threadIdx.x * 4; c < H; c += blockDim.x * 4) {
+                float4 a = *reinterpret_cast<const float4*>(comb + c);
+#pragma unroll
+                for (int k = 1; k < kTeams; ++k) {
+                    const float4 b = *reinterpret_cast<const float4*>(comb + k * kCols + c);
+                    a.x += b.x;
+                    a.y += b.y;
+                    a.z += b.z;
+                    a.w += b.w;
+                }
+                *reinterpret_cast<float4*>(row + c) = a;
             }
         }
     }
@@ -449,7 +470,7 @@ static int fast_tpr(int64_t H, int dtype) {
     return 0;
 }
 
-// teams of the persistent backward kernel (also the number of fp32 partial rows)
+// teams of the persistent backward kernel (an upper bound of the number of fp32 partial rows)
 static int bwd_teams(int64_t B, int tpr) {
     const int block = tpr > 256 ? tpr : 256;
     const int teams_per_block = block / tpr;
@@ -497,7 +518,7 @@ extern "C" int ck_rmsnorm_forward(const void* x, const void* weight, void* outpu
     return ck_launch_status();
 }
 
-// Workspace layout.  Fast path: teams x H fp32 partial rows.  Generic path: B fp32 rstd values, then
+// Workspace layout.  Fast path: room for teams x H fp32 partial rows (one per workgroup is used, then kReduceSplits).  Generic path: B fp32 rstd values, then
 // kColSegments x H_padded fp32 partial rows.  The query returns the larger of the two.
 static int64_t padded_h(int64_t H) { return (H + 3) / 4 * 4; }
 
@@ -563,17 +584,18 @@ extern "C" int ck_rmsnorm_backward(const void* x, const void* weight, const void
             else if (tpr == 256) launch_bwd<T, 256>(grid, block, s, x, weight, output_grad, rstd, x_grad, ws, B, (int)H, eps);
             else launch_bwd<T, 1024>(grid, block, s, x, weight, output_grad, rstd, x_grad, ws, B, (int)H, eps);
             if (weight) {
-                // teams partial rows -> kReduceSplits rows (fp32, behind the partial rows) -> dweight
-                const int splits = teams >= 4 * kReduceSplits ? kReduceSplits : 1;
+                // one partial row per workgroup -> (kReduceSplits rows, fp32, behind the partial rows ->) dweight
+                const int rows = (int)grid;
+                const int splits = rows >= 32 * kReduceSplits ? kReduceSplits : 1;
                 float* second = ws + (int64_t)teams * H;
                 if (splits > 1) {
                     hipLaunchKernelGGL((ck::rmsnorm_dw_reduce_kernel<T>), dim3((unsigned)ck_ceil_div(H, 16), splits),
-                                       dim3(64), 0, s, ws, (S*)nullptr, second, teams, (int)H);
+                                       dim3(64), 0, s, ws, (S*)nullptr, second, rows, (int)H);
                     hipLaunchKernelGGL((ck::rmsnorm_dw_reduce_kernel<T>), dim3((unsigned)ck_ceil_div(H, 16), 1), dim3(64),
                                        0, s, second, (S*)weight_grad, (float*)nullptr, splits, (int)H);
                 } else {
                     hipLaunchKernelGGL((ck::rmsnorm_dw_reduce_kernel<T>), dim3((unsigned)ck_ceil_div(H, 16), 1), dim3(64),
-                                       0, s, ws, (S*)weight_grad, (float*)nullptr, teams, (int)H);
+                                       0, s, ws, (S*)weight_grad, (float*)nullptr, rows, (int)H);
                 }
             }
         } else {
