@@ -102,6 +102,18 @@ int ck_embedding_backward(const void* ids, int ids_are_i32, const void* output_g
 int ck_contiguous_count(const void* x, int x_is_i32, int32_t* output, int64_t n, int64_t size, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * Element-wise additions: output = x + y and output = x + scalar (sum formed in fp32, one rounding)
+ * replace add_tensor_forward_cuda (kernels/add/add_tensor/cuda_implementation/ops.cpp:3-7) and
+ *         add_scalar_forward_cuda (kernels/add/add_scalar/cuda_implementation/ops.cpp:3-7);
+ * the reference's vector_instruction_width has no counterpart: packets are 16 bytes whenever the
+ * pointers allow it.  Tensors are dense with identical layout; block_size as for the SwiGLU kernels.
+ * ------------------------------------------------------------------------------------------- */
+int ck_add_tensor_forward(const void* x, const void* y, void* output, int64_t num_elements, int dtype,
+                          int block_size, void* stream);
+int ck_add_scalar_forward(const void* x, double y, void* output, int64_t num_elements, int dtype, int block_size,
+                          void* stream);
+
+/* ---------------------------------------------------------------------------------------------
  * Expert sort for the MoE layer: STABLE ascending sort of expert ids with their positions, plus the
  * inclusive prefix sum of the per-expert counts.
  * replaces scattermoe/triton_implementation/__init__.py:80-81

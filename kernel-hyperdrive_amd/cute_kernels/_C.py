@@ -36,6 +36,8 @@ _f32 = ctypes.c_float
 _SIGNATURES = {
     "ck_status_string": (ctypes.c_char_p, [_i32]),
     "ck_abi_version": (_i32, []),
+    "ck_add_tensor_forward": (_i32, [_p, _p, _p, _i64, _i32, _i32, _p]),
+    "ck_add_scalar_forward": (_i32, [_p, ctypes.c_double, _p, _i64, _i32, _i32, _p]),
     "ck_swiglu_forward": (_i32, [_p, _p, _p, _i64, _i32, _i32, _p]),
     "ck_swiglu_backward": (_i32, [_p, _p, _p, _p, _p, _i64, _i32, _i32, _p]),
     "ck_swiglu_unchunked_forward": (_i32, [_p, _p, _i64, _i64, _i32, _i32, _p]),
@@ -196,6 +198,26 @@ def _ids_are_i32(ids: torch.Tensor) -> int:
 
 # ---- one Python function per C entry point ----------------------------------------------------------
 # All tensors must be contiguous unless a stride is passed explicitly.
+
+
+def add_tensor_forward(x, y, output, block_size: int) -> None:
+    lib = load_library()
+    with _Launch(x, y, output) as L:
+        _check(
+            lib.ck_add_tensor_forward(_ptr(x), _ptr(y), _ptr(output), x.numel(), dtype_code(x.dtype), block_size,
+                                      L.stream),
+            "ck_add_tensor_forward",
+        )
+
+
+def add_scalar_forward(x, y: float, output, block_size: int) -> None:
+    lib = load_library()
+    with _Launch(x, output) as L:
+        _check(
+            lib.ck_add_scalar_forward(_ptr(x), float(y), _ptr(output), x.numel(), dtype_code(x.dtype), block_size,
+                                      L.stream),
+            "ck_add_scalar_forward",
+        )
 
 
 def swiglu_forward(gate, up, output, block_size: int) -> None:

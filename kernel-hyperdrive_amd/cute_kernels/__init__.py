@@ -16,6 +16,10 @@ from .kernels import (
     MoE_HIP,
     MoE_Torch,
     MoE_Triton,
+    add_scalar_cute,
+    add_scalar_torch,
+    add_tensor_cute,
+    add_tensor_torch,
     contiguous_count_cute,
     embedding_cute,
     embedding_torch,

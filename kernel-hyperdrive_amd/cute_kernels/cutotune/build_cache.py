@@ -4,8 +4,7 @@
 
 Counterpart of the reference's tools/build_cutotune_cache.py:1-62: one forward + backward of every tuned operator
 per dtype, at the reference's tuning shapes plus the shapes of this repository's benchmark, so that first calls
-do not pay for the search.  The add_scalar / add_tensor operators of the reference script are not part of this
-package.
+do not pay for the search.
 """
 
 import argparse
@@ -13,7 +12,15 @@ from typing import Callable
 
 import torch
 
-from .. import embedding_cute, get_powers_of_2, rmsnorm_cute, swiglu_cute, swiglu_unchunked_cute
+from .. import (
+    add_scalar_cute,
+    add_tensor_cute,
+    embedding_cute,
+    get_powers_of_2,
+    rmsnorm_cute,
+    swiglu_cute,
+    swiglu_unchunked_cute,
+)
 from .cache import get_cutotune_cache
 
 
@@ -34,6 +41,9 @@ def main() -> None:
     for dtype in (torch.float32, torch.float16, torch.bfloat16):
         for size in (104857600, 16384 * 14336):
             x = torch.randn(size, dtype=dtype, device=device, requires_grad=True)
+            if size == 104857600:
+                forward_backward(add_scalar_cute, x, 3)
+                forward_backward(add_tensor_cute, x, x)
             forward_backward(swiglu_cute, x, x)
             del x
         for size in ((81920, 8192), (16384, 28672)):

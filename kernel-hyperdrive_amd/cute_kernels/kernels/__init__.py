@@ -1,3 +1,4 @@
+from .add import add_scalar_cute, add_scalar_torch, add_tensor_cute, add_tensor_torch
 from .contiguous_count import contiguous_count_cute
 from .embedding import embedding_cute, embedding_torch
 from .rmsnorm import rmsnorm_cute, rmsnorm_torch

@@ -6,6 +6,10 @@ that the HIP kernels can be checked against it.  Only tests, ``__graft_entry__.s
 
 How each function is pinned (the reference holds no golden vectors for this path; its tests compare against
 stock torch ops on random inputs):
+  add_tensor, add_scalar
+                      ``x + y`` (cute_kernels/kernels/add/add_*/torch_implementation.py:4-5): the sum formed in fp32
+                      and rounded once; checked against numpy float32 addition with a hand-written
+                      round-to-nearest-even to bf16 / numpy's own to fp16
   swiglu_*            closed form cute_kernels/kernels/swiglu/README.md:3-13; checked against autograd of
                       ``up * F.silu(gate)`` in fp64 and the limits g -> +-inf, g = 0
   rmsnorm_*           closed form cute_kernels/kernels/rmsnorm/README.md:3-25; checked against autograd of
@@ -59,6 +63,19 @@ def fraction_outside(actual: torch.Tensor, expected: torch.Tensor, rtol: float, 
     e = expected.detach().double().cpu()
     bad = (a - e).abs() > atol + rtol * e.abs()
     return bad.double().mean().item() if bad.numel() else 0.0
+
+
+# =====================================================================================================
+# Additions   (cute_kernels/kernels/add/add_tensor/torch_implementation.py:4-5, add_scalar/...:4-5)
+# =====================================================================================================
+def add_tensor(x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+    # stock torch forms the sum of two 16-bit values in fp32 and rounds once
+    return (x.float() + y.float()).to(x.dtype)
+
+
+def add_scalar(x: torch.Tensor, y: float) -> torch.Tensor:
+    # the Python scalar becomes an fp32 value before the addition, for every storage type
+    return (x.float() + torch.tensor(y, dtype=torch.float32)).to(x.dtype)
 
 
 # =====================================================================================================

@@ -39,6 +39,17 @@ def test_swiglu_argument_checks(lib):
     assert lib.ck_swiglu_forward(None, None, None, 0, BF16, 256, None) == OK  # nothing to do
 
 
+def test_add_argument_checks(lib):
+    assert lib.ck_add_tensor_forward(P, P, P, -1, BF16, 256, None) == SHAPE
+    assert lib.ck_add_tensor_forward(P, P, P, 64, BF16, 96, None) == SHAPE  # workgroup size not a multiple of 64
+    assert lib.ck_add_tensor_forward(P, P, P, 64, 7, 256, None) == DTYPE
+    assert lib.ck_add_tensor_forward(P, None, P, 64, BF16, 256, None) == NULL
+    assert lib.ck_add_tensor_forward(P, P + 1, P, 64, BF16, 256, None) == ALIGN
+    assert lib.ck_add_scalar_forward(None, 0.5, P, 64, BF16, 256, None) == NULL
+    assert lib.ck_add_scalar_forward(P, 0.5, P + 2, 64, F32, 256, None) == ALIGN
+    assert lib.ck_add_scalar_forward(P, 0.5, P, 0, F32, 256, None) == OK  # nothing to do
+
+
 def test_rmsnorm_argument_checks(lib):
     assert lib.ck_rmsnorm_forward(P, None, P, None, 4, 65537, 1e-5, BF16, None) == SHAPE  # H above the limit
     assert lib.ck_rmsnorm_forward(None, None, P, None, 4, 64, 1e-5, BF16, None) == NULL

@@ -59,6 +59,24 @@ def test_compiled_elementwise_ops(gpu, dtype):
     assert_close(tg.grad, O.embedding_backward(ids, d_out, 300), dtype, "embedding dw")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_compiled_additions(gpu, dtype):
+    from cute_kernels import add_scalar_cute, add_tensor_cute
+
+    announce("compiled additions", dtype)
+    x, y, dz = randn((33, 517), dtype, 21), randn((33, 517), dtype, 22), randn((33, 517), dtype, 23)
+    xg, yg = x.to(gpu).requires_grad_(True), y.to(gpu).requires_grad_(True)
+    z = torch.compile(add_tensor_cute, fullgraph=True)(xg, yg)
+    z.backward(dz.to(gpu))
+    assert torch.equal(z.detach().cpu(), O.add_tensor(x, y))
+    assert torch.equal(xg.grad.cpu(), dz) and torch.equal(yg.grad.cpu(), dz)
+    xs = x.to(gpu).requires_grad_(True)
+    s = torch.compile(add_scalar_cute, fullgraph=True)(xs, 0.42)
+    s.backward(dz.to(gpu))
+    assert torch.equal(s.detach().cpu(), O.add_scalar(x, 0.42))
+    assert torch.equal(xs.grad.cpu(), dz)
+
+
 def test_compiled_contiguous_count(gpu):
     from cute_kernels import contiguous_count_cute
 

@@ -11,6 +11,63 @@ from oracle import cute_oracle as O
 pytestmark = pytest.mark.gpu
 
 
+# ---- additions ----------------------------------------------------------------------------------------
+ADD_SIZES = [(1,), (7,), (8,), (1000,), (4099,), (37, 513), (4, 128, 256), (1 << 20,), (3, (1 << 19) + 3)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("size", ADD_SIZES)
+def test_add_tensor_and_scalar(gpu, dtype, size):
+    """Exact, as in the reference's tests (tests/kernels/add/add_tensor_test.py, add_scalar_test.py): against the
+    oracle and against stock torch on the GPU; gradients are the incoming gradient itself."""
+    from cute_kernels import KernelBackend, add_scalar_cute, add_tensor_cute
+
+    announce("add", dtype, size)
+    x, y, dz = randn(size, dtype, 11, 3.0), randn(size, dtype, 12, 0.01), randn(size, dtype, 13)
+    xg = x.to(gpu).requires_grad_(True)
+    yg = y.to(gpu).requires_grad_(True)
+    z = add_tensor_cute(xg, yg)
+    z.backward(dz.to(gpu))
+    assert z.dtype == dtype and z.shape == x.shape
+    assert torch.equal(z.detach().cpu(), O.add_tensor(x, y))
+    assert torch.equal(z.detach(), xg.detach() + yg.detach())
+    assert torch.equal(xg.grad.cpu(), dz) and torch.equal(yg.grad.cpu(), dz)
+    # every spelling of the tunables the reference accepts
+    for width in (1, 2, 4, 8, None):
+        z2 = add_tensor_cute(xg, yg, kernel_backend=KernelBackend.cuda, vector_instruction_width=width, BLOCK_SIZE=1024)
+        assert torch.equal(z2, z)
+
+    xs = x.to(gpu).requires_grad_(True)
+    s = add_scalar_cute(xs, 0.42)
+    s.mean().backward()
+    assert torch.equal(s.detach().cpu(), O.add_scalar(x, 0.42))
+    assert torch.equal(s.detach(), xs.detach() + 0.42)
+    assert torch.equal(xs.grad, torch.full_like(xs, 1.0 / x.numel()))
+    same = add_scalar_cute(xs, 0)  # add_scalar/__init__.py:19-20: no launch, the input itself comes back
+    assert same.data_ptr() == xs.data_ptr() and torch.equal(same, xs)
+
+
+def test_add_layouts_and_errors(gpu):
+    from cute_kernels import add_scalar_cute, add_tensor_cute
+
+    announce("add layouts")
+    dtype = torch.bfloat16
+    x, y = randn((64, 48), dtype, 14).to(gpu), randn((64, 48), dtype, 15).to(gpu)
+    # same non-contiguous layout on both sides: walked as it lies in memory
+    assert torch.equal(add_tensor_cute(x.t(), y.t()), x.t() + y.t())
+    # different layouts, a strided view, an unaligned view
+    assert torch.equal(add_tensor_cute(x.t(), y.t().contiguous()), x.t() + y.t())
+    assert torch.equal(add_tensor_cute(x[:, ::2], y[:, ::2]), x[:, ::2] + y[:, ::2])
+    assert torch.equal(add_scalar_cute(x[:, ::2], -1.5), x[:, ::2] - 1.5)
+    flat = randn((4100,), dtype, 16).to(gpu)
+    assert torch.equal(add_tensor_cute(flat[1:], flat[1:]), flat[1:] + flat[1:])
+    assert torch.equal(add_scalar_cute(flat[3:], 2.0), flat[3:] + 2.0)
+    with pytest.raises(AssertionError):
+        add_tensor_cute(x, y[:32])
+    with pytest.raises(AssertionError):
+        add_tensor_cute(x, y.float())
+
+
 # ---- swiglu -------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("size", [(1,), (7,), (8,), (1000,), (4099,), (37, 513), (4, 128, 256), (1 << 20,), (3, 1 << 19)])

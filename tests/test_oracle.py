@@ -17,6 +17,39 @@ F64 = torch.float64
 
 
 # ---- swiglu -------------------------------------------------------------------------------------------
+def _round_to_bf16(values32: np.ndarray) -> np.ndarray:
+    """float32 -> nearest bfloat16 (ties to even), returned as float32: plain integer arithmetic on the bits."""
+    bits = values32.astype(np.float32).view(np.uint32).astype(np.uint64)
+    bits = (bits + 0x7FFF + ((bits >> 16) & 1)) & 0xFFFF0000
+    return bits.astype(np.uint32).view(np.float32)
+
+
+def test_additions_round_once_from_fp32():
+    g = torch.Generator().manual_seed(7)
+    x32 = torch.randn(4099, generator=g) * 3
+    y32 = torch.randn(4099, generator=g) * 0.01  # very different magnitudes: the rounding of the sum matters
+    for dtype in (torch.bfloat16, torch.float16, torch.float32):
+        x, y = x32.to(dtype), y32.to(dtype)
+        exact32 = x.float().numpy() + y.float().numpy()
+        if dtype == torch.bfloat16:
+            expected = _round_to_bf16(exact32)
+        elif dtype == torch.float16:
+            expected = exact32.astype(np.float16).astype(np.float32)
+        else:
+            expected = exact32
+        assert np.array_equal(O.add_tensor(x, y).float().numpy(), expected), dtype
+        assert torch.equal(O.add_tensor(x, y), x + y), dtype  # what stock torch gives
+        s32 = x.float().numpy() + np.float32(0.42)
+        expected = _round_to_bf16(s32) if dtype == torch.bfloat16 else (
+            s32.astype(np.float16).astype(np.float32) if dtype == torch.float16 else s32)
+        assert np.array_equal(O.add_scalar(x, 0.42).float().numpy(), expected), dtype
+        # (stock torch on the CPU rounds the scalar to the 16-bit type first; on the GPU, where the reference's test
+        # makes the comparison, it stays fp32 as in the reference's kernel, add_scalar/.../kernels_forward.cu:11 -
+        # the GPU tests compare with that)
+        if dtype == torch.float32:
+            assert torch.equal(O.add_scalar(x, 0.42), x + 0.42)
+
+
 def test_swiglu_matches_autograd_fp64():
     g = torch.randn(37, 19, dtype=F64, requires_grad=True)
     u = torch.randn(37, 19, dtype=F64, requires_grad=True)
