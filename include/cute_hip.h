@@ -205,7 +205,8 @@ int ck_group(const void* A, int64_t a_stride, const int64_t* idx, const void* co
  * replaces the two torch.bmm calls of scattermoe/triton_implementation/ops.py:160-164 and :204.
  *   forward : out[t, :]     = sum_j gates[t, j] * expanded[t, j, :]      expanded [T, k, H], gates [T, k]
  *   backward: d_gates[t, j] = sum_h expanded[t, j, h] * grad_out[t, h]
- * All tensors dense.
+ * gates == NULL in the forward call gives the plain sum over j: the input gradient's
+ * `.view(T, k, H).sum(-2)` of ops.py:261.  All tensors dense.
  * ------------------------------------------------------------------------------------------- */
 int ck_moe_combine_forward(const void* expanded, const void* gates, void* out, int64_t tokens, int64_t k,
                            int64_t H, int dtype, void* stream);

@@ -2,7 +2,8 @@
 // The reference does both with torch.bmm on [T, 1, k] x [T, k, H] batches
 // (cute_kernels/kernels/scattermoe/triton_implementation/ops.py:160-164 and :204), which turns into
 // thousands of degenerate GEMMs; here each is one HBM-bound pass, one wavefront per token.
-//   forward : out[t, :]      = sum_j gates[t, j] * expanded[t, j, :]
+//   forward : out[t, :]      = sum_j gates[t, j] * expanded[t, j, :]      (gates == NULL: plain sum over j, the
+//                              reference's `.view(T, k, H).sum(-2)` of ops.py:261)
 //   backward: d_gates[t, j]  = sum_h expanded[t, j, h] * grad_out[t, h]
 // fp32 accumulation, one rounding.
 #include "ck_device.h"
@@ -25,7 +26,7 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
         for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
         for (int s = 0; s < k; ++s) {
-            const float g = T::up(gates[t * k + s]);
+            const float g = gates != nullptr ? T::up(gates[t * k + s]) : 1.0f;
             const P v = nt_load(src + (int64_t)s * packs + p);
 #pragma unroll
             for (int j = 0; j < VEC; ++j) acc[j] += g * T::up(v.v[j]);
@@ -68,8 +69,8 @@ extern "C" int ck_moe_combine_forward(const void* expanded, const void* gates, v
                                       int64_t H, int dtype, void* stream) {
     if (tokens < 0 || k <= 0 || H < 0 || k > 0x7fffffff) return CK_ERR_SHAPE;
     if (tokens == 0 || H == 0) return CK_OK;
-    if (!expanded || !gates || !out) return CK_ERR_NULL;
-    if (!ck_aligned_elem(expanded, dtype) || !ck_aligned_elem(gates, dtype) || !ck_aligned_elem(out, dtype))
+    if (!expanded || !out) return CK_ERR_NULL;
+    if (!ck_aligned_elem(expanded, dtype) || (gates && !ck_aligned_elem(gates, dtype)) || !ck_aligned_elem(out, dtype))
         return CK_ERR_ALIGN;
     const int64_t grid = ck_ceil_div(tokens, 4);
     if (grid > 0x7fffffff) return CK_ERR_SHAPE;

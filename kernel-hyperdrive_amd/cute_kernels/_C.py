@@ -436,7 +436,7 @@ def group(A, idx, coeff, out, fan_out: int) -> None:
 
 
 def moe_combine_forward(expanded, gates, out) -> None:
-    """expanded [T, k, H], gates [T, k], out [T, H]; all dense."""
+    """expanded [T, k, H], gates [T, k] (or None: plain sum over the k slots), out [T, H]; all dense."""
     lib = load_library()
     T, k, H = expanded.shape
     with _Launch(expanded, gates, out) as L:

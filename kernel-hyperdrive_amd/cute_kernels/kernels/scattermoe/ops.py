@@ -7,7 +7,8 @@ saved tensors, same nine gradient slots).  Differences that do not change result
   * ``scatter2scatter`` takes the expert offsets as an optional trailing argument (the tile scheduler works
     per expert); without it they are recomputed from the sorted expert ids;
   * the two ``torch.bmm`` calls that mix expert outputs with the routing weights (ops.py:160-164, 204) are
-    single-pass kernels (``moe_combine_forward`` / ``moe_combine_backward_gates``);
+    single-pass kernels (``moe_combine_forward`` / ``moe_combine_backward_gates``), and the sum of the input
+    gradient over a token's k slots (ops.py:261) runs on the first of them without weights;
   * the weight gradient is written completely by the kernel (zeros for experts without rows), so it is
     allocated with ``empty_like`` instead of ``zeros_like`` (ops.py:237).
 
@@ -117,6 +118,20 @@ def group(
 def moe_combine_forward(expanded: torch.Tensor, gates: torch.Tensor, out: torch.Tensor) -> None:
     """out[t] = sum_j gates[t, j] * expanded[t, j]  (the reference's bmm(gates[T,1,k], expanded[T,k,H]))."""
     _C.moe_combine_forward(expanded.contiguous(), gates.contiguous(), out)
+
+
+@cute_op(f"{LIBRARY_NAME}::moe_topk_sum", mutates_args={"out"})
+def moe_topk_sum(expanded: torch.Tensor, out: torch.Tensor) -> None:
+    """out[t] = sum_j expanded[t, j]  (the reference's ``.view(T, k, H).sum(-2)``, ops.py:261): fp32 sum, one rounding."""
+    _C.moe_combine_forward(expanded.contiguous(), None, out)
+
+
+def _sum_over_slots(d_expanded_input: torch.Tensor, tokens: int, k: int) -> torch.Tensor:
+    if k == 1:
+        return d_expanded_input
+    d_input = torch.empty(tokens, d_expanded_input.size(-1), device=d_expanded_input.device, dtype=d_expanded_input.dtype)
+    moe_topk_sum(expanded=d_expanded_input.view(tokens, k, d_expanded_input.size(-1)), out=d_input)
+    return d_input
 
 
 @cute_op(f"{LIBRARY_NAME}::moe_combine_backward_gates", mutates_args={"d_gates"})
@@ -240,10 +255,7 @@ class _ScatteredExperts(torch.autograd.Function):
             expert_offsets=expert_offsets,
         )
 
-        if k == 1:
-            d_input = d_expanded_input
-        else:
-            d_input = d_expanded_input.view(x.size(0), k, d_expanded_input.size(-1)).sum(-2)
+        d_input = _sum_over_slots(d_expanded_input, x.size(0), k)
 
         # x, expert_weights, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, gates, grouped_in, grouped_out
         return d_input, d_weights, None, None, None, None, d_gates, None, None
@@ -337,7 +349,7 @@ class _ScatteredGLUExperts(torch.autograd.Function):
             y_grouped=False,
             expert_offsets=expert_offsets,
         )
-        d_input = d_expanded_input if k == 1 else d_expanded_input.view(x.size(0), k, x.size(1)).sum(-2)
+        d_input = _sum_over_slots(d_expanded_input, x.size(0), k)
         # x, w_fc, w_proj, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, gates
         return d_input, d_w_fc, d_w_proj, None, None, None, None, d_gates
 

@@ -119,7 +119,7 @@ def test_grouped_gemm_argument_checks(lib):
     assert lib.ck_group(None, 64, P, None, P, 64, 16, 64, 1, BF16, None) == NULL
     assert lib.ck_group(P, 64, P, None, P, 64, 16, 64, 0, BF16, None) == SHAPE
     assert lib.ck_moe_combine_forward(P, P, P, 16, 0, 64, BF16, None) == SHAPE  # k = 0
-    assert lib.ck_moe_combine_forward(P, None, P, 16, 2, 64, BF16, None) == NULL
+    assert lib.ck_moe_combine_forward(None, P, P, 16, 2, 64, BF16, None) == NULL  # (gates may be NULL: plain sum)
     assert lib.ck_moe_combine_backward_gates(P, P, None, 16, 2, 64, BF16, None) == NULL
     assert lib.ck_probe_mfma(None, 10, 1, P, None) == NULL
     assert lib.ck_probe_mfma(P, 10, 0, P, None) == SHAPE

@@ -188,6 +188,14 @@ def test_moe_combine(gpu, dtype, shape):
     out = torch.empty(T, H, dtype=dtype, device=gpu)
     moe_combine_forward(expanded.to(gpu), gates.to(gpu), out)
     assert_close(out, O.moe_combine_forward(expanded, gates, acc_dtype(dtype)), dtype, "out")
+    # without weights: the sum over a token's k slots, exactly what torch's sum gives (fp32 sum, one rounding)
+    from cute_kernels.kernels.scattermoe.ops import moe_topk_sum
+
+    plain = torch.empty(T, H, dtype=dtype, device=gpu)
+    moe_topk_sum(expanded.to(gpu), plain)
+    assert_close(plain, expanded.to(acc_dtype(dtype)).sum(-2).to(dtype), dtype, "sum over slots")
+    if k <= 2:
+        assert torch.equal(plain, expanded.to(gpu).sum(-2)), "two addends: no freedom in the order"
     d_gates = torch.empty(T, k, dtype=dtype, device=gpu)
     moe_combine_backward_gates(expanded.to(gpu), dy.to(gpu), d_gates)
     # a dot product over H terms of O(1): compared norm-wise for fp32 (fp32 accumulation), element-wise for 16 bit
