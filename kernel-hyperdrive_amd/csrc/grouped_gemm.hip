@@ -131,6 +131,116 @@ __device__ __forceinline__ bool logical_tile(int m_tiles, int n_tiles, int& mt, 
     return true;
 }
 
+// Tile of workgroup blockIdx.x for the products whose rows are cut per expert (forward and input gradient): the
+// XCD-aware order above, applied to the number of row tiles the experts really have.  The host can only bound
+// that number (rows / BM + E); dealing out the bound would leave the XCD that owns the end of the range with
+// mostly empty tiles while the others carry all the work.  Executed by the first wave; the result (expert, first
+// row, valid rows, column tile; expert < 0: nothing to do) is broadcast through LDS.
+template <int BM>
+__device__ __forceinline__ void find_tile_balanced(const int64_t* __restrict__ offsets, int E, int n_tiles, int* sh_info) {
+    if (threadIdx.x < CK_WAVE) {
+        constexpr int XCDS = 8, GROUP_M = 8;
+        const int lane = lane_id();
+        // row tiles of all experts
+        int m_tiles = 0;
+        for (int e0 = 0; e0 < E; e0 += CK_WAVE) {
+            const int e = e0 + lane;
+            int tiles = 0;
+            if (e < E) tiles = ((int)offsets[e] - (e == 0 ? 0 : (int)offsets[e - 1]) + BM - 1) / BM;
+            m_tiles += wave_sum_i(tiles);
+        }
+        int found_e = -1, found_start = 0, found_rows = 0, nt = 0;
+        const int total = m_tiles * n_tiles;
+        // an even share of the tiles where rows of the tile grid are long; whole rows of it where they are short
+        // (measured at 16 column tiles: 1-2 % better than shares that end in the middle of a row, while at 56 and
+        // 112 column tiles the even share is 2-4 % better)
+        const int per_xcd = n_tiles >= 32 ? (total + XCDS - 1) / XCDS : (m_tiles + XCDS - 1) / XCDS * n_tiles;
+        const int xcd = blockIdx.x % XCDS, pos = blockIdx.x / XCDS;
+        const int L = xcd * per_xcd + pos;
+        if (pos < per_xcd && L < total) {
+            const int group_span = GROUP_M * n_tiles;
+            const int group = L / group_span;
+            const int first_m = group * GROUP_M;
+            const int gm = min(GROUP_M, m_tiles - first_m);
+            const int in_group = L - group * group_span;
+            const int mt = first_m + in_group % gm;
+            nt = in_group / gm;
+            int base_tiles = 0;
+            for (int e0 = 0; e0 < E && found_e < 0; e0 += CK_WAVE) {
+                const int e = e0 + lane;
+                int begin = 0, end = 0;
+                if (e < E) {
+                    end = (int)offsets[e];
+                    begin = e == 0 ? 0 : (int)offsets[e - 1];
+                }
+                const int tiles = (end - begin + BM - 1) / BM;
+                const int incl = wave_inclusive_scan_i(tiles) + base_tiles;
+                const uint64_t hit = __ballot(e < E && incl > mt);
+                if (hit != 0) {
+                    const int src = __ffsll((unsigned long long)hit) - 1;
+                    const int excl = __shfl(incl - tiles, src, CK_WAVE);
+                    const int b = __shfl(begin, src, CK_WAVE);
+                    const int en = __shfl(end, src, CK_WAVE);
+                    found_e = e0 + src;
+                    found_start = b + (mt - excl) * BM;
+                    found_rows = min(BM, en - found_start);
+                }
+                base_tiles = __shfl(incl, CK_WAVE - 1, CK_WAVE);
+            }
+        }
+        if (lane == 0) {
+            sh_info[0] = found_e;
+            sh_info[1] = found_start;
+            sh_info[2] = found_rows;
+            sh_info[3] = nt;
+        }
+    }
+    __syncthreads();
+}
+
+// Tile order of the per-expert weight-gradient products.  A tile's cost grows with its expert's row count, which
+// routing can skew by orders of magnitude, and workgroup w always runs on XCD w % 8.  So every XCD gets an
+// eighth of the tiles of EVERY expert (a contiguous piece of the expert's tile grid in the grouped order used
+// above: 8 row tiles per column tile), and takes the experts in the order of falling row count - the long tiles
+// start first, the short ones fill the gaps at the end.
+//   workgroup w -> XCD x = w % 8, position s = w / 8 in that XCD's list; list = for rank r: piece x of expert(r)
+// Returns false for the workgroups past the end of a list.
+__device__ __forceinline__ bool weight_grad_tile(int E, int i_tiles, int n_tiles, int& rank, int& it, int& nt) {
+    constexpr int XCDS = 8, GROUP_M = 8;
+    const int per_expert = i_tiles * n_tiles;
+    const int x = blockIdx.x % XCDS, s = blockIdx.x / XCDS;
+    const int lo = per_expert / XCDS, rem = per_expert % XCDS;
+    const int mine = lo + (x < rem ? 1 : 0);
+    if (mine == 0 || s >= E * mine) return false;
+    rank = s / mine;
+    const int q = x * lo + min(x, rem) + s % mine;  // position in the expert's grid, grouped order
+    const int group_span = GROUP_M * n_tiles;
+    const int group = q / group_span;
+    const int first = group * GROUP_M;
+    const int gm = min(GROUP_M, i_tiles - first);
+    const int in_group = q - group * group_span;
+    it = first + in_group % gm;
+    nt = in_group / gm;
+    return true;
+}
+
+// Expert with the `rank`-th largest row count (ties: lower index first).  Every wave works it out for itself from
+// the offsets: lane e holds the count of expert e and counts the experts ahead of it.  More than 64 experts keep
+// their index order (the split over the XCDs above is what matters most).
+__device__ __forceinline__ int expert_of_rank(const int64_t* __restrict__ offsets, int E, int rank) {
+    if (E > CK_WAVE) return rank;
+    const int lane = lane_id();
+    int count = -1;
+    if (lane < E) count = (int)offsets[lane] - (lane == 0 ? 0 : (int)offsets[lane - 1]);
+    int ahead = 0;
+    for (int e = 0; e < E; ++e) {
+        const int other = __shfl(count, e, CK_WAVE);
+        ahead += (other > count || (other == count && e < lane)) ? 1 : 0;
+    }
+    const uint64_t hit = __ballot(lane < E && ahead == rank);
+    return __builtin_amdgcn_readfirstlane(__ffsll((unsigned long long)hit) - 1);
+}
+
 // Tile shape of the MFMA kernel.  BM x BN outputs per workgroup, BK of the contraction per step,
 // WM x WN wavefronts each owning a (BM/WM) x (BN/WN) block of 32x32 MFMA tiles.
 template <int BM_, int BN_, int BK_, int WM_, int WN_>
@@ -445,27 +555,27 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
     __shared__ __attribute__((aligned(1024))) char lds1[BUF_BYTES];
     __shared__ int sh_info[4];
 
-    int mt, nt;
-    if (!logical_tile(p.m_tiles, p.n_tiles, mt, nt)) return;
-
+    int nt = 0;
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid / CK_WAVE);
     const int wm = wave / WN, wn = wave % WN;
 
     int expert, row_start, rows_valid, k_begin, k_end, i_base;
     if (!GROUP_K) {
-        find_tile<BM>(p.offsets, p.E, mt, sh_info);
+        find_tile_balanced<BM>(p.offsets, p.E, p.n_tiles, sh_info);
         expert = __builtin_amdgcn_readfirstlane(sh_info[0]);
         row_start = __builtin_amdgcn_readfirstlane(sh_info[1]);
         rows_valid = __builtin_amdgcn_readfirstlane(sh_info[2]);
+        nt = __builtin_amdgcn_readfirstlane(sh_info[3]);
         if (expert < 0) return;
         k_begin = 0;
         k_end = p.K;
         i_base = 0;
     } else {
-        const int i_tiles = p.m_tiles / p.E;
-        expert = mt / i_tiles;
-        i_base = (mt % i_tiles) * BM;
+        int rank, it;
+        if (!weight_grad_tile(p.E, p.m_tiles / p.E, p.n_tiles, rank, it, nt)) return;
+        expert = expert_of_rank(p.offsets, p.E, rank);
+        i_base = it * BM;
         k_begin = expert == 0 ? 0 : (int)p.offsets[expert - 1];
         k_end = (int)p.offsets[expert];
         row_start = 0;
@@ -947,6 +1057,14 @@ namespace {
 typedef ck::Tile<CK_TILE_CONFIG> MainTile;
 constexpr int kBM = MainTile::BM, kBN = MainTile::BN;
 
+// Workgroups for the products cut per expert: 8 XCD lists, each long enough for either way find_tile_balanced
+// deals the tiles (an eighth of the tiles, or whole rows of the tile grid), at the bound of the row tile count.
+int64_t dealt_grid(const ck::GemmParams& p) {
+    const int64_t even = ((int64_t)p.m_tiles * p.n_tiles + 7) / 8;
+    const int64_t rows = (int64_t)((p.m_tiles + 7) / 8) * p.n_tiles;
+    return 8 * (even > rows ? even : rows);
+}
+
 template <typename T, bool B_KC, bool GROUP_K>
 void launch_mfma(const ck::GemmParams& p, hipStream_t s) {
     const int total = p.m_tiles * p.n_tiles;
@@ -954,17 +1072,21 @@ void launch_mfma(const ck::GemmParams& p, hipStream_t s) {
     if (p.wide)
         hipLaunchKernelGGL((ck::grouped_gemm_kernel<T, MainTile, B_KC, GROUP_K>), dim3((unsigned)grid),
                            dim3(MainTile::THREADS), 0, s, p);
-    else
-        hipLaunchKernelGGL((ck::grouped_gemm_m16_kernel<T, MainTile, B_KC, GROUP_K>), dim3((unsigned)grid),
+    else if (GROUP_K) {
+        // 8 lists (one per XCD), each with ceil(tiles per expert / 8) entries per expert: see weight_grad_tile
+        const int64_t per_expert = (int64_t)(p.m_tiles / p.E) * p.n_tiles;
+        const int64_t listed = 8 * (int64_t)p.E * ((per_expert + 7) / 8);  // < 2^31: m_tiles * n_tiles is checked by the caller
+        hipLaunchKernelGGL((ck::grouped_gemm_m16_kernel<T, MainTile, B_KC, GROUP_K>), dim3((unsigned)listed),
+                           dim3(MainTile::THREADS), 0, s, p);
+    } else
+        hipLaunchKernelGGL((ck::grouped_gemm_m16_kernel<T, MainTile, B_KC, GROUP_K>), dim3((unsigned)dealt_grid(p)),
                            dim3(MainTile::THREADS), 0, s, p);
 }
 
 // per-expert product with the SwiGLU epilogue GLU (1: forward, 2: backward); never the wide kernel
 template <typename T, bool B_KC, int GLU>
 void launch_mfma_glu(const ck::GemmParams& p, hipStream_t s) {
-    const int total = p.m_tiles * p.n_tiles;
-    const int grid = (total + 7) / 8 * 8;
-    hipLaunchKernelGGL((ck::grouped_gemm_m16_kernel<T, MainTile, B_KC, false, GLU>), dim3((unsigned)grid),
+    hipLaunchKernelGGL((ck::grouped_gemm_m16_kernel<T, MainTile, B_KC, false, GLU>), dim3((unsigned)dealt_grid(p)),
                        dim3(MainTile::THREADS), 0, s, p);
 }
 
@@ -1012,7 +1134,7 @@ extern "C" int ck_scatter2scatter(const void* X, int64_t x_stride, const void* W
         p.wide = num_slots * x_stride * 2 >= (int64_t)1 << 32 || (b_kc ? N : K) * p.ldb * 2 >= (int64_t)1 << 32;
         p.m_tiles = (int)(num_slots / kBM + E);
         p.n_tiles = (int)ck_ceil_div(N, kBN);
-        if ((int64_t)p.m_tiles * p.n_tiles > 0x7ffffff0) return CK_ERR_SHAPE;
+        if ((int64_t)(p.m_tiles + 8) * p.n_tiles > 0x7ffffff0) return CK_ERR_SHAPE;
         if (dtype == CK_BF16) {
             if (b_kc) launch_mfma<ck::BF16, true, false>(p, s);
             else launch_mfma<ck::BF16, false, false>(p, s);
@@ -1077,7 +1199,7 @@ extern "C" int ck_scatter2scatter_glu(const void* X, int64_t x_stride, const voi
         p.glu_half = (int)I;
         p.m_tiles = (int)(num_slots / kBM + E);
         p.n_tiles = (int)(I / (kBN / 2));
-        if ((int64_t)p.m_tiles * p.n_tiles > 0x7ffffff0) return CK_ERR_SHAPE;
+        if ((int64_t)(p.m_tiles + 8) * p.n_tiles > 0x7ffffff0) return CK_ERR_SHAPE;
         if (dtype == CK_BF16) launch_mfma_glu<ck::BF16, true, 1>(p, s);
         else launch_mfma_glu<ck::F16, true, 1>(p, s);
         return ck_launch_status();
@@ -1134,7 +1256,7 @@ extern "C" int ck_scatter2scatter_glu_bwd(const void* DY, int64_t dy_stride, con
         p.glu_half = (int)I;
         p.m_tiles = (int)(num_slots / kBM + E);
         p.n_tiles = (int)ck_ceil_div(I, kBN);
-        if ((int64_t)p.m_tiles * p.n_tiles > 0x7ffffff0) return CK_ERR_SHAPE;
+        if ((int64_t)(p.m_tiles + 8) * p.n_tiles > 0x7ffffff0) return CK_ERR_SHAPE;
         if (dtype == CK_BF16) launch_mfma_glu<ck::BF16, false, 2>(p, s);
         else launch_mfma_glu<ck::F16, false, 2>(p, s);
         return ck_launch_status();
@@ -1186,7 +1308,7 @@ extern "C" int ck_group_bwd_W(const void* DY, int64_t dy_stride, const void* X, 
         p.wide = 64 * p.lda * 2 >= (int64_t)1 << 32 || 64 * p.ldb * 2 >= (int64_t)1 << 32;
         p.m_tiles = (int)(E * ck_ceil_div(p.K, kBM));
         p.n_tiles = (int)ck_ceil_div(p.N, kBN);
-        if ((int64_t)p.m_tiles * p.n_tiles > 0x7ffffff0) return CK_ERR_SHAPE;
+        if ((int64_t)(p.m_tiles + 8) * p.n_tiles > 0x7ffffff0) return CK_ERR_SHAPE;
         if (dtype == CK_BF16) launch_mfma<ck::BF16, false, true>(p, s);
         else launch_mfma<ck::F16, false, true>(p, s);
         return ck_launch_status();
