@@ -7,6 +7,7 @@
 //       input order (stable), which torch's default sort does not promise
 //   - ck_offsets_from_sorted : cumsum(bincount) recovered from already-sorted ids.
 #include "ck_block_sort.h"
+#include "ck_grid_sort.h"
 
 namespace ck {
 
@@ -117,6 +118,54 @@ __global__ void __launch_bounds__(kSortThreads)
     }
 }
 
+// ---- the same sort spread over the GPU -----------------------------------------------------------
+// One workgroup sorts 16K ids in ~30 us but needs ~200 us for 100K: from kGridSortFrom ids on (and up to
+// 2^kGridSortMaxBits experts, one radix pass) the three kernels of ck_grid_sort.h take over.  Ids become the
+// keys, positions the values; the scatter kernel also derives the expert offsets from the scanned histogram
+// (the exclusive offset of bin e + 1 for the first wave = number of ids <= e).
+constexpr int64_t kGridSortFrom = 32768;
+
+template <bool I32>
+struct ExpertIdLoader {
+    const void* ids;
+    __device__ __forceinline__ void operator()(int i, uint32_t& key, uint32_t& val) const {
+        key = (uint32_t)load_id<I32>(ids, i);
+        val = (uint32_t)i;
+    }
+};
+struct SortedStorer {
+    int64_t* sorted_ids;
+    int64_t* sorted_pos;
+    __device__ __forceinline__ void operator()(int pos, uint32_t key, uint32_t val) const {
+        sorted_ids[pos] = (int64_t)key;
+        sorted_pos[pos] = (int64_t)val;
+    }
+};
+
+template <bool I32>
+__global__ void __launch_bounds__(256)
+    moe_grid_hist_kernel(ExpertIdLoader<I32> load, int M, int bits, uint32_t* __restrict__ hist, int num_waves) {
+    __shared__ GridSortShared sh;
+    grid_sort_histogram(sh, M, 0, bits, hist, num_waves, load);
+}
+
+__global__ void __launch_bounds__(1024) moe_grid_scan_kernel(uint32_t* __restrict__ hist, int total) {
+    grid_sort_scan(hist, total);
+}
+
+template <bool I32>
+__global__ void __launch_bounds__(256)
+    moe_grid_scatter_kernel(ExpertIdLoader<I32> load, SortedStorer store, int M, int bits,
+                            const uint32_t* __restrict__ scanned, int num_waves, int64_t* __restrict__ offsets, int E) {
+    __shared__ GridSortShared sh;
+    if (blockIdx.x == 0) {
+        const int nbins = 1 << bits;
+        for (int e = threadIdx.x; e < E; e += blockDim.x)
+            offsets[e] = e + 1 < nbins ? (int64_t)scanned[(int64_t)(e + 1) * num_waves] : (int64_t)M;
+    }
+    grid_sort_scatter(sh, M, 0, bits, scanned, num_waves, load, store);
+}
+
 __global__ void __launch_bounds__(256)
     offsets_from_sorted_kernel(const int64_t* __restrict__ sorted_ids, int64_t* __restrict__ offsets, int64_t M,
                                int64_t E) {
@@ -169,8 +218,14 @@ extern "C" int ck_contiguous_count(const void* x, int x_is_i32, int32_t* output,
     return ck_launch_status();
 }
 
+static bool use_grid_sort(int64_t M, int64_t E) {
+    return M >= ck::kGridSortFrom && ck::ck_key_bits(E) <= ck::kGridSortMaxBits;
+}
+
 extern "C" int64_t ck_moe_sort_workspace_size(int64_t M, int64_t E) {
     if (M <= 0 || E <= 0) return 0;
+    if (use_grid_sort(M, E))  // histogram [bins][waves]
+        return ((int64_t)1 << ck::ck_key_bits(E)) * ck::grid_sort_waves(M) * (int64_t)sizeof(uint32_t);
     return ck::ck_sort_passes(ck::ck_key_bits(E)) > 1 ? 4 * M * (int64_t)sizeof(uint32_t) : 0;
 }
 
@@ -184,6 +239,30 @@ extern "C" int ck_moe_sort(const void* expert_ids, int ids_are_i32, int64_t* sor
     if (need > 0 && (!workspace || workspace_bytes < need)) return CK_ERR_WORKSPACE;
     hipStream_t s = (hipStream_t)stream;
     const int key_bits = ck::ck_key_bits(E);
+    if (use_grid_sort(M, E)) {
+        if (reinterpret_cast<uintptr_t>(workspace) & 3u) return CK_ERR_WORKSPACE;
+        const int num_waves = ck::grid_sort_waves(M);
+        const unsigned grid = (unsigned)ck_ceil_div(num_waves, ck::kGridSortBlockWaves);
+        uint32_t* hist = (uint32_t*)workspace;
+        const int total = (1 << key_bits) * num_waves;
+        ck::SortedStorer store = {sorted_expert_idxs, sorted_scattered_idxs};
+        if (ids_are_i32) {
+            ck::ExpertIdLoader<true> load = {expert_ids};
+            hipLaunchKernelGGL(ck::moe_grid_hist_kernel<true>, dim3(grid), dim3(256), 0, s, load, (int)M, key_bits, hist,
+                               num_waves);
+            hipLaunchKernelGGL(ck::moe_grid_scan_kernel, dim3(1), dim3(1024), 0, s, hist, total);
+            hipLaunchKernelGGL(ck::moe_grid_scatter_kernel<true>, dim3(grid), dim3(256), 0, s, load, store, (int)M,
+                               key_bits, hist, num_waves, expert_offsets, (int)E);
+        } else {
+            ck::ExpertIdLoader<false> load = {expert_ids};
+            hipLaunchKernelGGL(ck::moe_grid_hist_kernel<false>, dim3(grid), dim3(256), 0, s, load, (int)M, key_bits, hist,
+                               num_waves);
+            hipLaunchKernelGGL(ck::moe_grid_scan_kernel, dim3(1), dim3(1024), 0, s, hist, total);
+            hipLaunchKernelGGL(ck::moe_grid_scatter_kernel<false>, dim3(grid), dim3(256), 0, s, load, store, (int)M,
+                               key_bits, hist, num_waves, expert_offsets, (int)E);
+        }
+        return ck_launch_status();
+    }
     if (ids_are_i32)
         hipLaunchKernelGGL(ck::moe_sort_kernel<true>, dim3(1), dim3(ck::kSortThreads), 0, s, expert_ids,
                            sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, (uint32_t*)workspace, (int)M,
