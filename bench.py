@@ -11,7 +11,8 @@ timed region.  Prints ONE JSON line:
                timed region with GPU events on the launch stream, against the 2.5 PFLOP/s dense bf16 MFMA peak
   cpu_baseline the oracle's torch restatement of the reference layer on the host cores, on a bounded sample
   extras       HBM GB/s of SwiGLU, RMSNorm and embedding at their BASELINE shapes (buffers rotated so that the
-               256 MB last-level cache cannot serve them)
+               256 MB last-level cache cannot serve them), and the step of the fine-grained skewed MoE
+               configuration (configs[4]: T=16384 H=2048 I=1408 E=64 top-6, Zipf(1.2) expert popularity)
 """
 
 import argparse
@@ -186,12 +187,61 @@ def _time_rotating(fn, sets, iters=20, warmup=3):
     return start.elapsed_time(end) / iters
 
 
+def zipf_ids(shape, vocab_size, s, seed):
+    """int64 ids with P(rank r) ~ 1 / r^s, ranks mapped through a fixed random permutation of the vocabulary."""
+    g = torch.Generator().manual_seed(seed)
+    cdf = torch.cumsum(torch.arange(1, vocab_size + 1, dtype=torch.float64).pow(-s), 0)
+    cdf = cdf / cdf[-1]
+    count = 1
+    for d in shape:
+        count *= d
+    rank = torch.searchsorted(cdf, torch.rand(count, generator=g, dtype=torch.float64)).clamp_(max=vocab_size - 1)
+    return torch.randperm(vocab_size, generator=g)[rank].reshape(shape)
+
+
+def bench_moe_skewed(device, steps=10, warmup=3):
+    """The fine-grained skewed configuration (BASELINE configs[4]): T=16384 H=2048 I=1408 E=64 top-6, expert
+    popularity Zipf(1.2) through a per-expert logit bias (feature 0 of every token is 1 and carries the bias in
+    the router weight), so that some experts get nothing and one gets more than a tenth of the rows."""
+    import cute_kernels as ck
+
+    T, H, I, E, k = 16384, 2048, 1408, 64, 6
+    dtype = torch.bfloat16
+    g = torch.Generator(device=device).manual_seed(0)
+    moe = ck.MoE_Triton(num_experts=E, num_experts_per_tok=k, hidden_size=H, intermediate_size=I,
+                        activation_function=ck.swiglu_unchunked_cute, is_glu=True, add_bias=False, std=0.02)
+    moe = moe.to(device=device, dtype=dtype)
+    x = torch.randn(T, H, generator=g, device=device)
+    rank = torch.randperm(E, generator=torch.Generator().manual_seed(62)) + 1
+    with torch.no_grad():
+        for prm in moe.parameters():
+            prm.copy_(torch.randn(prm.shape, generator=g, device=device, dtype=torch.float32).mul_(0.02))
+        moe.gate.weight[:, 0] = (-1.25 * 1.2 * torch.log(rank.double())).to(device=device, dtype=dtype)
+    x[:, 0] = 1.0
+    x = x.to(dtype).requires_grad_(True)
+    dy = torch.randn(T, H, generator=g, device=device).to(dtype)
+    with torch.no_grad():
+        _, _, selected = moe._compute_routing_weights(x)
+    counts = torch.bincount(selected.flatten(), minlength=E)
+    assert (counts == 0).any() and counts.max().item() > 0.1 * counts.sum().item(), "the routing is meant to be skewed"
+    for _ in range(warmup):
+        moe_step(moe, x, dy)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        moe_step(moe, x, dy)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    tflops = 18.0 * T * k * H * I / (ms * 1e-3) / 1e12
+    return {"TFLOP/s": round(tflops, 1), "frac_of_mfma_peak": round(tflops / BF16_MFMA_PEAK_TFLOPS, 4), "ms": round(ms, 3),
+            "empty_experts": int((counts == 0).sum().item()), "largest_expert_share": round(counts.max().item() / counts.sum().item(), 3)}
+
+
 def bench_extras(device):
     from cute_kernels import KernelBackend
     from cute_kernels.kernels import embedding as EM
     from cute_kernels.kernels import rmsnorm as RN
     from cute_kernels.kernels import swiglu as SW
-    from oracle import cute_oracle as O
 
     dtype = torch.bfloat16
     hip = KernelBackend.hip
@@ -234,7 +284,7 @@ def bench_extras(device):
     n = 8 * 4096
     dys = [torch.randn(8, 4096, H, device=device, dtype=dtype) for _ in range(2)]
     for label, ids in (("uniform", torch.randint(0, V, (8, 4096), generator=torch.Generator().manual_seed(0))),
-                       ("zipf", O.zipf_ids((8, 4096), V, 1.1, seed=0))):
+                       ("zipf", zipf_ids((8, 4096), V, 1.1, seed=0))):
         ids = ids.to(device)
         ms = _time_rotating(lambda i: EM._forward(input_ids=ids, weight=table, kernel_backend=hip, BLOCK_SIZE_B=4, BLOCK_SIZE_H=512), 1)
         out[f"embedding_fwd_{label}"] = gbs(2 * n * H * 2 + 8 * n, ms)
@@ -242,6 +292,8 @@ def bench_extras(device):
                                                    BLOCK_SIZE_B=4, BLOCK_SIZE_H=512), 2, iters=10)
         out[f"embedding_bwd_{label}"] = gbs(n * H * 2 + V * H * 2 + 8 * n, ms)
     del table, dys
+    torch.cuda.empty_cache()
+    out["moe_fine_grained_skewed"] = bench_moe_skewed(device)
     torch.cuda.empty_cache()
     return out
 
