@@ -214,6 +214,23 @@ int ck_moe_combine_backward_gates(const void* expanded, const void* grad_out, vo
                                   int64_t k, int64_t H, int dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * Per-expert bias of the grouped linears
+ * replaces the bias term of F.linear(rows_e, W[e], bias[e]) in scattermoe/torch_implementation.py:35-43 (the
+ * reference's Triton experts, triton_implementation/__init__.py:24-34, do not read their bias parameter).
+ *   forward : y[r(i), :] += bias[e(i), :]   for every expert-sorted position i in [0, num_rows), where e(i) is the
+ *             expert whose offset range holds i and r(i) = row_index ? row_index[i] : i (NULL: y is expert-grouped;
+ *             sorted_scattered_idxs: y is in (token, slot) order).  In place, fp32 add, one rounding.
+ *   backward: d_bias[e, :] = sum of the expert-grouped rows dy[offsets[e-1] .. offsets[e]) (fp32 sum in a fixed
+ *             order, one rounding; zeros for an expert without rows).  Every element of d_bias is written.
+ * y / dy / bias / d_bias have unit column stride and the given row strides (in elements); E <= 65535 backward.
+ * ------------------------------------------------------------------------------------------- */
+int ck_expert_bias_forward(void* y, int64_t y_stride, const void* bias, int64_t bias_stride,
+                           const int64_t* row_index, const int64_t* expert_offsets, int64_t num_rows, int64_t N,
+                           int64_t E, int dtype, void* stream);
+int ck_expert_bias_backward(const void* dy, int64_t dy_stride, const int64_t* expert_offsets, void* d_bias,
+                            int64_t d_bias_stride, int64_t num_rows, int64_t N, int64_t E, int dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
  * Measurement aid with no counterpart in the reference: back-to-back v_mfma_f32_32x32x16_bf16 on operands
  * held in registers (the register footprint of the grouped GEMM's inner loop, no LDS or memory traffic), to
  * read off the rate the matrix cores sustain on given data under the part's power limit.

@@ -68,6 +68,8 @@ _SIGNATURES = {
     "ck_group": (_i32, [_p, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _i32, _p]),
     "ck_moe_combine_forward": (_i32, [_p, _p, _p, _i64, _i64, _i64, _i32, _p]),
     "ck_moe_combine_backward_gates": (_i32, [_p, _p, _p, _i64, _i64, _i64, _i32, _p]),
+    "ck_expert_bias_forward": (_i32, [_p, _i64, _p, _i64, _p, _p, _i64, _i64, _i64, _i32, _p]),
+    "ck_expert_bias_backward": (_i32, [_p, _i64, _p, _p, _i64, _i64, _i64, _i64, _i32, _p]),
     "ck_probe_mfma": (_i32, [_p, _i64, _i32, _p, _p]),
 }
 
@@ -456,6 +458,46 @@ def moe_combine_backward_gates(expanded, grad_out, d_gates) -> None:
             lib.ck_moe_combine_backward_gates(_ptr(expanded), _ptr(grad_out), _ptr(d_gates), T, k, H,
                                               dtype_code(expanded.dtype), L.stream),
             "ck_moe_combine_backward_gates",
+        )
+
+
+def expert_bias_forward(y, bias, row_index, expert_offsets) -> None:
+    """y[r(i)] += bias[expert of sorted position i], in place; row_index None for expert-grouped y, else the
+    position -> row map (sorted_scattered_idxs)."""
+    lib = load_library()
+    if y.stride(1) != 1 or bias.stride(1) != 1:
+        raise ValueError("expert_bias_forward needs unit column stride for y and bias")
+    if bias.size(1) != y.size(1) or bias.size(0) != expert_offsets.numel():
+        raise ValueError("expert_bias_forward: bias must be [num_experts, y.size(1)]")
+    if row_index is not None and (row_index.numel() != y.size(0) or row_index.dtype != torch.int64):
+        raise ValueError("expert_bias_forward: one int64 row index per row of y")
+    if bias.dtype != y.dtype or expert_offsets.dtype != torch.int64:
+        raise ValueError("expert_bias_forward: bias in y's dtype, int64 expert offsets")
+    if row_index is not None and not row_index.is_contiguous():
+        row_index = row_index.contiguous()
+    with _Launch(y, bias, row_index, expert_offsets) as L:
+        _check(
+            lib.ck_expert_bias_forward(_ptr(y), y.stride(0), _ptr(bias), bias.stride(0), _ptr(row_index),
+                                       _ptr(expert_offsets), y.size(0), y.size(1), bias.size(0), dtype_code(y.dtype),
+                                       L.stream),
+            "ck_expert_bias_forward",
+        )
+
+
+def expert_bias_backward(dy, expert_offsets, d_bias) -> None:
+    """d_bias[e] = sum of the expert-grouped rows of dy that belong to expert e (every element written)."""
+    lib = load_library()
+    if dy.stride(1) != 1 or d_bias.stride(1) != 1:
+        raise ValueError("expert_bias_backward needs unit column stride for dy and d_bias")
+    if d_bias.size(1) != dy.size(1) or d_bias.size(0) != expert_offsets.numel():
+        raise ValueError("expert_bias_backward: d_bias must be [num_experts, dy.size(1)]")
+    if d_bias.dtype != dy.dtype or expert_offsets.dtype != torch.int64:
+        raise ValueError("expert_bias_backward: d_bias in dy's dtype, int64 expert offsets")
+    with _Launch(dy, expert_offsets, d_bias) as L:
+        _check(
+            lib.ck_expert_bias_backward(_ptr(dy), dy.stride(0), _ptr(expert_offsets), _ptr(d_bias), d_bias.stride(0),
+                                        dy.size(0), dy.size(1), d_bias.size(0), dtype_code(dy.dtype), L.stream),
+            "ck_expert_bias_backward",
         )
 
 

@@ -51,6 +51,10 @@ def moe_sort(selected_experts: torch.Tensor, num_experts: int) -> tuple[torch.Te
 
 
 class Experts_HIP(Experts_Torch):
+    """The grouped linears on the HIP kernels.  ``add_bias=True`` applies the ``[E, out]`` bias as the plain-torch
+    experts do (torch_implementation.py:35-43); the reference's ``Experts_Triton`` holds the same parameter and
+    leaves it out of the product (triton_implementation/__init__.py:24-34), which only shows once it is non-zero."""
+
     def forward(
         self,
         inputs,
@@ -62,7 +66,6 @@ class Experts_HIP(Experts_Torch):
         grouped_in=False,
         grouped_out=False,
     ):
-        # bias is not applied on this path, as in the reference's Experts_Triton
         return scattered_experts(
             inputs,
             self.weight.permute(0, 2, 1),
@@ -73,6 +76,7 @@ class Experts_HIP(Experts_Torch):
             gates,
             grouped_in,
             grouped_out,
+            self.bias,
         )
 
 
@@ -88,9 +92,12 @@ class MoE_HIP(MoE_Torch):
     ) -> torch.Tensor:
         sorted_expert_idxs, sorted_scattered_idxs, expert_offsets = moe_sort(selected_experts, self.num_experts)
 
-        # the fused kernels take 16-bit storage with I a multiple of 128 and H a multiple of 8
+        # the fused kernels take 16-bit storage with I a multiple of 128 and H a multiple of 8, and no bias (it
+        # would have to enter before the activation)
         fusable = (
-            hidden_states.dtype in (torch.float16, torch.bfloat16)
+            self.c_fc.bias is None
+            and self.c_proj.bias is None
+            and hidden_states.dtype in (torch.float16, torch.bfloat16)
             and self.intermediate_size % 128 == 0
             and self.hidden_size % 8 == 0
         )

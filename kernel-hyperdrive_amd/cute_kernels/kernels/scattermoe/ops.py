@@ -3,7 +3,8 @@
 ``scatter2scatter``, ``group_bwd_W`` and ``group`` keep the names, argument order and ``cute::`` custom-op
 registration of cute_kernels/kernels/scattermoe/triton_implementation/ops.py:16-130, and
 ``_ScatteredExperts`` / ``scattered_experts`` the autograd contract of ops.py:133-301 (same inputs, same
-saved tensors, same nine gradient slots).  Differences that do not change results:
+saved tensors, same nine gradient slots, plus an optional tenth argument: the per-expert bias).  Differences that
+do not change results:
   * ``scatter2scatter`` takes the expert offsets as an optional trailing argument (the tile scheduler works
     per expert); without it they are recomputed from the sorted expert ids;
   * the two ``torch.bmm`` calls that mix expert outputs with the routing weights (ops.py:160-164, 204) are
@@ -11,6 +12,10 @@ saved tensors, same nine gradient slots).  Differences that do not change result
     gradient over a token's k slots (ops.py:261) runs on the first of them without weights;
   * the weight gradient is written completely by the kernel (zeros for experts without rows), so it is
     allocated with ``empty_like`` instead of ``zeros_like`` (ops.py:237).
+One difference that does: ``expert_biases`` ([E, out], default None).  The reference's Triton experts own a bias
+parameter and never apply it (triton_implementation/__init__.py:24-34), unlike its plain-torch experts
+(torch_implementation.py:35-43); with the argument given, the bias is added to every row's product before the
+routing weights mix the k outputs, and its gradient is the per-expert sum of the grouped output gradient.
 
 ``scattered_glu_experts`` is the whole expert MLP with a SwiGLU in between (c_fc -> swiglu_unchunked -> c_proj,
 triton_implementation/__init__.py:83-98) as one autograd node: the activation and its derivative run in the
@@ -140,6 +145,23 @@ def moe_combine_backward_gates(expanded: torch.Tensor, grad_out: torch.Tensor, d
     _C.moe_combine_backward_gates(expanded.contiguous(), grad_out.contiguous(), d_gates)
 
 
+@cute_op(f"{LIBRARY_NAME}::expert_bias_forward", mutates_args={"y"})
+def expert_bias_forward(
+    y: torch.Tensor, bias: torch.Tensor, expert_offsets: torch.Tensor, row_index: torch.Tensor | None = None
+) -> None:
+    """y[r] += bias[expert of r] in place: the bias term of the reference's F.linear(rows_e, W[e], bias[e])
+    (torch_implementation.py:35-43).  ``row_index`` None: y is expert-grouped; sorted_scattered_idxs: (token, slot) order."""
+    _C.expert_bias_forward(y, bias, row_index, expert_offsets)
+
+
+@cute_op(f"{LIBRARY_NAME}::expert_bias_backward", mutates_args={"d_bias"})
+def expert_bias_backward(DY: torch.Tensor, expert_offsets: torch.Tensor, d_bias: torch.Tensor) -> None:
+    """d_bias[e] = sum over expert e's rows of the expert-grouped DY."""
+    if DY.stride(1) != 1:
+        DY = DY.contiguous()
+    _C.expert_bias_backward(DY, expert_offsets, d_bias)
+
+
 class _ScatteredExperts(torch.autograd.Function):
     @staticmethod
     def forward(
@@ -153,8 +175,9 @@ class _ScatteredExperts(torch.autograd.Function):
         gates=None,
         grouped_in=False,
         grouped_out=False,
+        expert_biases=None,
     ):
-        # expert_weights: view [E, in, out] of the [E, out, in] parameter
+        # expert_weights: view [E, in, out] of the [E, out, in] parameter; expert_biases: [E, out] or None
         output = torch.empty(sorted_expert_idxs.size(0), expert_weights.size(-1), device=x.device, dtype=x.dtype)
         scatter2scatter(
             X=x,
@@ -167,6 +190,14 @@ class _ScatteredExperts(torch.autograd.Function):
             y_grouped=grouped_out,
             expert_offsets=expert_offsets,
         )
+        if expert_biases is not None:
+            # before the routing weights mix the k outputs, as F.linear(rows, W[e], bias[e]) has it
+            expert_bias_forward(
+                y=output,
+                bias=expert_biases,
+                expert_offsets=expert_offsets,
+                row_index=None if grouped_out else sorted_scattered_idxs,
+            )
 
         if gates is None:
             output_expanded = None
@@ -182,6 +213,7 @@ class _ScatteredExperts(torch.autograd.Function):
         ctx.grouped_in = grouped_in
         ctx.grouped_out = grouped_out
         ctx.k = k
+        ctx.has_bias = expert_biases is not None
         return output
 
     @staticmethod
@@ -227,6 +259,14 @@ class _ScatteredExperts(torch.autograd.Function):
                 fan_out=gate_fan,
             )
 
+        # --- bias gradient: the grouped (routing-weighted) output gradient summed per expert -------------
+        d_biases = None
+        if ctx.has_bias:
+            d_biases = torch.empty(
+                expert_weights.size(0), expert_weights.size(-1), device=grad_out.device, dtype=grad_out.dtype
+            )
+            expert_bias_backward(DY=grouped_grad_out, expert_offsets=expert_offsets, d_bias=d_biases)
+
         # --- expert-grouped input rows ----------------------------------------------------------------
         if grouped_in:
             grouped_x = x
@@ -257,8 +297,9 @@ class _ScatteredExperts(torch.autograd.Function):
 
         d_input = _sum_over_slots(d_expanded_input, x.size(0), k)
 
-        # x, expert_weights, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, gates, grouped_in, grouped_out
-        return d_input, d_weights, None, None, None, None, d_gates, None, None
+        # x, expert_weights, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, gates, grouped_in,
+        # grouped_out, expert_biases
+        return d_input, d_weights, None, None, None, None, d_gates, None, None, d_biases
 
 
 class _ScatteredGLUExperts(torch.autograd.Function):
@@ -370,6 +411,7 @@ def scattered_experts(
     gates=None,
     grouped_in=False,
     grouped_out=False,
+    expert_biases=None,
 ):
     return _ScatteredExperts.apply(
         inputs,
@@ -381,4 +423,5 @@ def scattered_experts(
         gates,
         grouped_in,
         grouped_out,
+        expert_biases,
     )

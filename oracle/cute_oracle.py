@@ -20,13 +20,16 @@ stock torch ops on random inputs):
   moe_sort            stable argsort; checked against a brute-force insertion on tiny inputs
   moe_combine_*       the two torch.bmm calls of scattermoe/triton_implementation/ops.py:160-164, 204; checked
                       against torch.bmm in fp64
+  expert_bias_*       the bias term of F.linear(rows_e, W[e], bias[e]) (scattermoe/torch_implementation.py:35-43);
+                      checked against F.linear per expert and its autograd in fp64
   scatter2scatter, group_bwd_W, group
                       per-slot / per-expert loops straight from the kernel docstrings
                       (scattermoe/triton_implementation/kernels.py:66-102, 152-240, 243-298)
   moe_forward_backward
                       restatement of MoE_Torch (scattermoe/torch_implementation.py:101-199) with bincount in
                       place of the Triton histogram; checked against an independent per-token dense
-                      formulation (y_t = sum_j softmax_j * FFN_{e_j}(x_t)) and its autograd in fp64
+                      formulation (y_t = sum_j softmax_j * FFN_{e_j}(x_t)) and its autograd in fp64, with and
+                      without the per-expert biases
 No function here is "parity unpinned".
 
 Precision policy: inputs are values of the storage dtype (bf16 / fp16 / fp32).  ``compute_dtype=float32``
@@ -235,6 +238,29 @@ def moe_combine_backward_gates(expanded, grad_out, compute_dtype=torch.float32):
 # =====================================================================================================
 # the MoE layer   (scattermoe/torch_implementation.py:101-199)
 # =====================================================================================================
+def expert_bias_forward(y, bias, expert_offsets, row_index=None, compute_dtype=torch.float32):
+    """y[r(i)] + bias[e(i)] for every expert-sorted position i (e(i) from the inclusive offsets, r(i) = row_index[i]
+    or i): the bias term of F.linear(rows_e, W[e], bias[e]), torch_implementation.py:35-43, added to an already
+    rounded product.  Returns a new tensor."""
+    expert = torch.from_numpy(_expert_of_slot(expert_offsets, y.size(0)))
+    rows = torch.arange(y.size(0)) if row_index is None else row_index
+    out = y.clone()
+    out[rows] = (y[rows].to(compute_dtype) + bias[expert].to(compute_dtype)).to(y.dtype)
+    return out
+
+
+def expert_bias_backward(dy, expert_offsets, compute_dtype=torch.float32):
+    """d_bias[e] = sum of the expert-grouped rows of dy in expert e's range (what autograd gives F.linear's bias)."""
+    ends = expert_offsets.tolist()
+    out = torch.zeros(len(ends), dy.size(1), dtype=compute_dtype)
+    start = 0
+    for e, end in enumerate(ends):
+        if end > start:
+            out[e] = dy[start:end].to(compute_dtype).sum(0)
+        start = end
+    return out.to(dy.dtype)
+
+
 def _acc_dtype(x: torch.Tensor) -> torch.dtype:
     """fp32 for 16- and 32-bit inputs; fp64 stays fp64 (used when the oracle itself is being pinned)."""
     return torch.float64 if x.dtype == torch.float64 else torch.float32
@@ -247,10 +273,12 @@ def swiglu_unchunked_activation(x: torch.Tensor) -> torch.Tensor:
     return (up.to(acc) * F.silu(gate.to(acc))).to(x.dtype)
 
 
-def moe_forward(x, w_gate, w_fc, w_proj, top_k: int, activation=swiglu_unchunked_activation, selected=None):
+def moe_forward(x, w_gate, w_fc, w_proj, top_k: int, activation=swiglu_unchunked_activation, selected=None,
+                b_fc=None, b_proj=None):
     """Forward of MoE_Torch on tensors of one dtype; returns (y [T, H], router_logits [T, E]).
 
-    x [T, H]; w_gate [E, H]; w_fc [E, F, H] (F = 2I for a GLU activation); w_proj [E, H, I].
+    x [T, H]; w_gate [E, H]; w_fc [E, F, H] (F = 2I for a GLU activation); w_proj [E, H, I]; optional per-expert
+    biases b_fc [E, F] and b_proj [E, H] (``add_bias=True``, :31 and :42).
     ``selected`` ([T, k] expert ids) replaces the top-k decision: logits rounded to 16 bits tie often, and
     two correct implementations may break a tie differently, so a test passes the decision of the run under
     test.  The values at the selected positions still come from this function's own logits.
@@ -276,9 +304,9 @@ def moe_forward(x, w_gate, w_fc, w_proj, top_k: int, activation=swiglu_unchunked
     splits = expert_frequency.tolist()
     outs = []
     for e, rows in enumerate(grouped.split(splits, dim=0)):                   # :36-43, 154-158
-        h = F.linear(rows, w_fc[e])
+        h = F.linear(rows, w_fc[e], None if b_fc is None else b_fc[e])
         h = activation(h)
-        outs.append(F.linear(h, w_proj[e]))
+        outs.append(F.linear(h, w_proj[e], None if b_proj is None else b_proj[e]))
     grouped = torch.cat(outs) * batch_gates.unsqueeze(-1)                     # :161
     # :162-163; the accumulation is done in fp32 and rounded once
     acc = _acc_dtype(x)
@@ -287,16 +315,20 @@ def moe_forward(x, w_gate, w_fc, w_proj, top_k: int, activation=swiglu_unchunked
 
 
 def moe_forward_backward(x, w_gate, w_fc, w_proj, dy, top_k: int, compute_dtype=torch.float32,
-                         activation=swiglu_unchunked_activation, selected=None) -> dict:
+                         activation=swiglu_unchunked_activation, selected=None, b_fc=None, b_proj=None) -> dict:
     """Forward and all gradients for loss = sum(y * dy), torch ops run in ``compute_dtype``.
 
-    Results are returned in the dtype of ``x``.
+    Results are returned in the dtype of ``x``; with biases given, their gradients are ``db_fc`` / ``db_proj``.
     """
     leaves = [t.detach().to(compute_dtype).clone().requires_grad_(True) for t in (x, w_gate, w_fc, w_proj)]
-    y, router_logits = moe_forward(*leaves, top_k=top_k, activation=activation, selected=selected)
+    biases = [None if b is None else b.detach().to(compute_dtype).clone().requires_grad_(True) for b in (b_fc, b_proj)]
+    y, router_logits = moe_forward(*leaves, top_k=top_k, activation=activation, selected=selected,
+                                   b_fc=biases[0], b_proj=biases[1])
     (y * dy.to(compute_dtype)).sum().backward()
     out_dtype = x.dtype
+    bias_grads = {name: b.grad.to(out_dtype) for name, b in zip(("db_fc", "db_proj"), biases) if b is not None}
     return {
+        **bias_grads,
         "y": y.detach().to(out_dtype),
         "router_logits": router_logits.detach().to(out_dtype),
         "dx": leaves[0].grad.to(out_dtype),
@@ -306,10 +338,11 @@ def moe_forward_backward(x, w_gate, w_fc, w_proj, dy, top_k: int, compute_dtype=
     }
 
 
-def moe_dense_per_token(x, w_gate, w_fc, w_proj, top_k: int, activation=swiglu_unchunked_activation):
+def moe_dense_per_token(x, w_gate, w_fc, w_proj, top_k: int, activation=swiglu_unchunked_activation,
+                        b_fc=None, b_proj=None):
     """Independent formulation used to pin ``moe_forward``: no sorting, no grouping.
 
-    y_t = sum_j softmax(top-k logits)_j * W_proj[e_j] act(W_fc[e_j] x_t)
+    y_t = sum_j softmax(top-k logits)_j * (W_proj[e_j] act(W_fc[e_j] x_t + b_fc[e_j]) + b_proj[e_j])
     """
     logits = x @ w_gate.T
     vals, sel = logits.topk(top_k, dim=-1) if top_k > 1 else logits.max(dim=-1, keepdim=True)
@@ -319,7 +352,13 @@ def moe_dense_per_token(x, w_gate, w_fc, w_proj, top_k: int, activation=swiglu_u
         acc = torch.zeros(x.size(1), dtype=x.dtype)
         for j in range(top_k):
             e = int(sel[t, j])
-            acc = acc + p[t, j] * (w_proj[e] @ activation((w_fc[e] @ x[t]).unsqueeze(0)).squeeze(0))
+            h = w_fc[e] @ x[t]
+            if b_fc is not None:
+                h = h + b_fc[e]
+            out = w_proj[e] @ activation(h.unsqueeze(0)).squeeze(0)
+            if b_proj is not None:
+                out = out + b_proj[e]
+            acc = acc + p[t, j] * out
         rows.append(acc)
     return torch.stack(rows), logits
 

@@ -121,6 +121,23 @@ def test_grouped_gemm_argument_checks(lib):
     assert lib.ck_moe_combine_forward(P, P, P, 16, 0, 64, BF16, None) == SHAPE  # k = 0
     assert lib.ck_moe_combine_forward(None, P, P, 16, 2, 64, BF16, None) == NULL  # (gates may be NULL: plain sum)
     assert lib.ck_moe_combine_backward_gates(P, P, None, 16, 2, 64, BF16, None) == NULL
+    bias = lib.ck_expert_bias_forward
+    #         y  ldy bias ldb idx  off rows N  E  dtype stream
+    assert bias(P, 64, P, 64, None, P, 16, 64, 0, BF16, None) == SHAPE  # E = 0
+    assert bias(P, 32, P, 64, None, P, 16, 64, 2, BF16, None) == SHAPE  # row stride below the row length
+    assert bias(P, 64, None, 64, None, P, 16, 64, 2, BF16, None) == NULL
+    assert bias(P, 64, P, 64, None, None, 16, 64, 2, BF16, None) == NULL  # no offsets
+    assert bias(P, 64, P, 64, None, P, 16, 64, 2, 6, None) == DTYPE
+    assert bias(P + 1, 64, P, 64, None, P, 16, 64, 2, BF16, None) == ALIGN
+    assert bias(P, 64, P, 64, None, P, 0, 64, 2, BF16, None) == OK  # no rows
+    bias_bwd = lib.ck_expert_bias_backward
+    #             dy ldy off d_bias ldb rows N  E  dtype stream
+    assert bias_bwd(P, 64, P, P, 64, 16, 64, 70000, BF16, None) == SHAPE  # more experts than grid rows
+    assert bias_bwd(P, 64, P, None, 64, 16, 64, 2, BF16, None) == NULL
+    assert bias_bwd(P, 64, None, P, 64, 16, 64, 2, BF16, None) == NULL
+    assert bias_bwd(P, 64, P, P, 64, 16, 64, 2, 3, None) == DTYPE
+    assert bias_bwd(P, 64, P, P + 2, 64, 16, 64, 2, F32, None) == ALIGN
+    assert bias_bwd(P, 64, P, P, 64, 16, 0, 2, BF16, None) == OK  # no columns
     assert lib.ck_probe_mfma(None, 10, 1, P, None) == NULL
     assert lib.ck_probe_mfma(P, 10, 0, P, None) == SHAPE
 

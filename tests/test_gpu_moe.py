@@ -206,6 +206,40 @@ def test_moe_combine(gpu, dtype, shape):
         assert_close(d_gates, expected, dtype, "d_gates")
 
 
+# ---- per-expert bias -------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("T,k,E,N,empty", [(16, 2, 4, 128, ()), (300, 3, 7, 200, (0, 6)), (257, 2, 5, 36, (2,)),
+                                           (50, 1, 3, 21, ()), (5000, 2, 8, 1032, ())])
+def test_expert_bias_ops(gpu, dtype, T, k, E, N, empty):
+    from cute_kernels.kernels.scattermoe.ops import expert_bias_backward, expert_bias_forward
+
+    announce("expert bias", dtype, T, k, E, N, empty)
+    _, scattered_idxs, offsets = routing(T, k, E, seed=71, empty=empty)
+    M = T * k
+    y = randn((M, N), dtype, seed=72)
+    bias = randn((E, N), dtype, seed=73)
+    # expert-grouped rows, then rows in (token, slot) order; a row stride wider than N in the second case
+    got = y.to(gpu)
+    expert_bias_forward(got, bias.to(gpu), offsets.to(gpu))
+    assert torch.equal(got.cpu(), O.expert_bias_forward(y, bias, offsets)), "grouped: one fp32 add, one rounding"
+    wide = torch.zeros(M, N + 8, dtype=dtype, device=gpu)
+    view = wide[:, :N]
+    view.copy_(y)
+    expert_bias_forward(view, bias.to(gpu), offsets.to(gpu), scattered_idxs.to(gpu))
+    assert torch.equal(view.cpu(), O.expert_bias_forward(y, bias, offsets, row_index=scattered_idxs)), "scattered"
+    assert torch.count_nonzero(wide[:, N:]) == 0
+
+    d_bias = torch.full((E, N), float("nan"), dtype=dtype, device=gpu)
+    expert_bias_backward(y.to(gpu), offsets.to(gpu), d_bias)
+    expected = O.expert_bias_backward(y, offsets, compute_dtype=torch.float64 if dtype == torch.float32 else torch.float32)
+    if dtype == torch.float32:
+        assert_norm_close(d_bias, expected, 1e-6, "d_bias")  # sums of up to 1250 terms of O(1) in fp32
+    else:
+        assert_close_long_sums(d_bias, expected, dtype, "d_bias")
+    for e in empty:
+        assert torch.count_nonzero(d_bias[e]) == 0
+
+
 # ---- the whole layer ----------------------------------------------------------------------------------
 def build_moe(cls, gpu, dtype, E, k, H, I, w_gate, w_fc, w_proj):
     from cute_kernels import swiglu_unchunked_cute
@@ -290,6 +324,76 @@ def test_moe_layer_against_oracle(gpu, dtype, case):
         tol = O.tolerance(dtype)
         for key in ("y", "dx", "dw_fc", "dw_proj"):
             assert O.fraction_outside(got[key], exact[key], **tol) < (2e-3 if k <= 4 else 5e-3), key  # more terms per row at top-6
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case", MOE_CASES[:4], ids=[c[0] for c in MOE_CASES[:4]])
+def test_moe_layer_with_expert_biases(gpu, dtype, case):
+    """``add_bias=True``: the layer on the HIP kernels applies the per-expert biases as the plain-torch layer does
+    (torch_implementation.py:35-43), here with non-zero values so that they are felt, and returns their gradients."""
+    from cute_kernels import MoE_Torch, MoE_Triton
+
+    name, T, H, I, E, k, skew = case
+    announce("moe layer with biases", dtype, case)
+    x, w_gate, w_fc, w_proj, dy = O.moe_inputs(T, H, I, E, dtype, seed=65)
+    if skew is not None:
+        w_gate, x = O.skewed_router(w_gate, x, 1.2, seed=66, scale=skew)
+    b_fc = randn((E, 2 * I), dtype, seed=67) * 0.5
+    b_proj = randn((E, H), dtype, seed=68) * 0.5
+
+    def build(cls):
+        from cute_kernels import swiglu_unchunked_cute
+
+        moe = cls(num_experts=E, num_experts_per_tok=k, hidden_size=H, intermediate_size=I,
+                  activation_function=swiglu_unchunked_cute, is_glu=True, add_bias=True, std=0.02)
+        moe = moe.to(device=gpu, dtype=dtype)
+        with torch.no_grad():
+            for param, value in ((moe.gate.weight, w_gate), (moe.c_fc.weight, w_fc), (moe.c_proj.weight, w_proj),
+                                 (moe.c_fc.bias, b_fc), (moe.c_proj.bias, b_proj)):
+                param.copy_(value)
+        return moe
+
+    def run(moe):
+        got, selected = run_moe(moe, x, dy, gpu)
+        got["db_fc"], got["db_proj"] = moe.c_fc.bias.grad, moe.c_proj.bias.grad
+        return got, selected
+
+    got, selected = run(build(MoE_Triton))
+    compute = dtype if dtype != torch.float32 else torch.float64
+    expected = O.moe_forward_backward(x, w_gate, w_fc, w_proj, dy, k, compute_dtype=compute, selected=selected,
+                                      b_fc=b_fc, b_proj=b_proj)
+    without = O.moe_forward_backward(x, w_gate, w_fc, w_proj, dy, k, compute_dtype=compute, selected=selected)
+    assert O.fraction_outside(without["y"], expected["y"], **O.tolerance(dtype)) > 0.5, "biases too small to matter"
+    for key in ("router_logits", "y", "dx", "dw_fc", "dw_proj", "db_fc", "db_proj"):
+        a, e = got[key], expected[key]
+        if key == "dx" and skew is not None:
+            a, e = a[:, 1:], e[:, 1:]  # feature 0 is the router's (see the test above)
+        if key in ("router_logits", "y"):
+            assert_close(a, e, dtype, f"{name}/{key}")
+            continue
+        # Gradients.  The bias is added to the product after it was rounded to the storage type, so in 16 bits
+        # about a quarter of the elements of h sit one unit in the last place beside a bias added before the
+        # rounding (the CPU's F.linear).  Both are as far from the exact value, but the gradients that read h,
+        # sums over hundreds of rows, then differ by more than two implementations with the same roundings do:
+        # the whole within one percent, and all but a small share of the elements within the tolerance (measured:
+        # bf16 up to 1.2e-2 of dw_proj, fp16 up to 8e-6).  fp32: sums of thousands of terms, held norm-wise, and
+        # element-wise except for the bias gradients (unscaled sums of O(1) rows).
+        assert_norm_close(a, e, 1e-5 if dtype == torch.float32 else 1e-2, f"{name}/{key}")
+        if dtype != torch.float32 or key not in ("db_fc", "db_proj"):
+            limit = {torch.float32: 1e-5, torch.float16: 1e-4, torch.bfloat16: 2.5e-2}[dtype]
+            assert O.fraction_outside(a, e, **O.tolerance(dtype)) <= limit, f"{name}/{key}"
+    if dtype == torch.bfloat16:
+        # where the bias enters before any 16-bit rounding on neither side, the sums agree to the bit
+        assert_close_long_sums(got["db_proj"], expected["db_proj"], dtype, f"{name}/db_proj")
+
+    # and the plain-torch layer on the GPU, the reference's own way of testing (tests/kernels/scattermoe_test.py)
+    ref, selected_ref = run(build(MoE_Torch))
+    if torch.equal(selected, selected_ref):
+        for key in ("y", "dx", "db_fc", "db_proj"):
+            if dtype == torch.float32:
+                assert_norm_close(got[key], ref[key], 1e-5, f"{name}/{key} vs MoE_Torch")
+            else:
+                assert O.fraction_outside(got[key], ref[key], **O.tolerance(dtype)) < 2.5e-2, key
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])

@@ -278,6 +278,55 @@ def test_moe_restatement_against_dense_per_token(top_k):
         assert torch.count_nonzero(res["dw_gate"]) == 0
 
 
+def test_moe_with_expert_biases_matches_per_token_formulation():
+    T, H, I, E, top_k = 19, 8, 6, 4, 2
+    x, wg, wfc, wproj, dy = (t.double() for t in O.moe_inputs(T, H, I, E, torch.float32, seed=8))
+    wg = wg * 20
+    g = torch.Generator().manual_seed(9)
+    b_fc = torch.randn(E, 2 * I, generator=g, dtype=F64)
+    b_proj = torch.randn(E, H, generator=g, dtype=F64)
+    res = O.moe_forward_backward(x, wg, wfc, wproj, dy, top_k, compute_dtype=F64, b_fc=b_fc, b_proj=b_proj)
+    without = O.moe_forward_backward(x, wg, wfc, wproj, dy, top_k, compute_dtype=F64)
+    assert not torch.allclose(res["y"], without["y"], atol=1e-3)  # the biases are felt
+
+    leaves = [t.clone().requires_grad_(True) for t in (x, wg, wfc, wproj, b_fc, b_proj)]
+    y, _ = O.moe_dense_per_token(*leaves[:4], top_k=top_k, b_fc=leaves[4], b_proj=leaves[5])
+    (y * dy).sum().backward()
+    assert torch.allclose(res["y"], y.detach(), rtol=1e-10, atol=1e-12)
+    for name, leaf in zip(("dx", "dw_gate", "dw_fc", "dw_proj", "db_fc", "db_proj"), leaves):
+        assert torch.allclose(res[name], leaf.grad, rtol=1e-9, atol=1e-11), name
+    # every selected slot adds its routing weight times b_proj[e]: d b_proj[e] = sum of weight * dy over e's slots,
+    # and the weights of one token sum to 1, so the b_proj gradients of all experts add up to the column sums of dy
+    assert torch.allclose(res["db_proj"].sum(0), dy.sum(0), rtol=1e-10, atol=1e-12)
+
+
+def test_expert_bias_ops_against_linear_per_expert():
+    g = torch.Generator().manual_seed(10)
+    E, N, K = 5, 12, 7
+    counts = torch.tensor([3, 0, 6, 1, 4])
+    offsets = counts.cumsum(0)
+    M = int(offsets[-1])
+    rows = torch.randn(M, K, generator=g, dtype=F64)
+    W = torch.randn(E, N, K, generator=g, dtype=F64)
+    bias = torch.randn(E, N, generator=g, dtype=F64).requires_grad_(True)
+    dy = torch.randn(M, N, generator=g, dtype=F64)
+    expected = torch.cat([F.linear(r, W[e], bias[e]) for e, r in enumerate(rows.split(counts.tolist()))])
+    (expected * dy).sum().backward()
+
+    product = torch.cat([F.linear(r, W[e]) for e, r in enumerate(rows.split(counts.tolist()))])
+    got = O.expert_bias_forward(product, bias.detach(), offsets, compute_dtype=F64)
+    assert torch.allclose(got, expected.detach(), rtol=1e-13, atol=1e-13)
+    assert torch.allclose(O.expert_bias_backward(dy, offsets, compute_dtype=F64), bias.grad, rtol=1e-13, atol=1e-13)
+    assert torch.count_nonzero(O.expert_bias_backward(dy, offsets)[1]) == 0  # the expert without rows
+
+    # rows held in another order: position i of the sorted order lives in row perm[i]
+    perm = torch.randperm(M, generator=g)
+    scattered = torch.empty_like(product)
+    scattered[perm] = product
+    got = O.expert_bias_forward(scattered, bias.detach(), offsets, row_index=perm, compute_dtype=F64)
+    assert torch.allclose(got[perm], expected.detach(), rtol=1e-13, atol=1e-13)
+
+
 def test_moe_single_expert_is_a_plain_mlp():
     T, H, I = 7, 8, 5
     x, wg, wfc, wproj, dy = (t.double() for t in O.moe_inputs(T, H, I, 1, torch.float32, seed=4))
