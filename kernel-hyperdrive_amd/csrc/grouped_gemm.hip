@@ -12,6 +12,8 @@
 // never mixes rows of two experts (the reference lets a 128-row block straddle experts and repeats the
 // product once per expert present in it).  fp32, and shapes whose contiguous dimensions are not
 // multiples of 8 elements, go through a plain kernel with exact (fp64) accumulation.
+#include <type_traits>
+
 #include "ck_device.h"
 
 namespace ck {
@@ -543,14 +545,20 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
     static_assert(WM == 2, "the epilogue stages one half of the rows per stage buffer");
     constexpr bool A_KC = !GROUP_K;
     constexpr bool B_KCC = GROUP_K ? false : B_KC;
-    typedef DtlOperand<S, BM, A_KC, NWAVES> AOp;
-    typedef DtlOperand<S, BN, B_KCC, NWAVES> BOp;
-    constexpr int STAGE_BYTES = AOp::STAGE_BYTES + BOp::STAGE_BYTES;
+    // Each operand tile lies in LDS as two halves of 128 lines, [A lower | A upper | B lower | B upper], 16 KB each.
+    // "Lower" holds the first half of every wave's rows (columns): line l of the lower A half is tile row
+    // (l / RW) * 2 RW + l % RW, of the upper half RW more; for B the same with CW.
+    typedef DtlOperand<S, BM / 2, A_KC, NWAVES> AOp;
+    typedef DtlOperand<S, BN / 2, B_KCC, NWAVES> BOp;
+    static_assert(AOp::IPW == BOp::IPW && AOp::IPW == 2, "square tile; the wait counts of the loop assume two copies per M phase");
+    constexpr int IPW = AOp::IPW;  // copy instructions per wave and half operand
+    constexpr int A_HALF = AOp::STAGE_BYTES, B_HALF = BOp::STAGE_BYTES, B_AT = 2 * A_HALF;
+    constexpr int STAGE_BYTES = 2 * A_HALF + 2 * B_HALF;
+    constexpr int RW = BM / WM / 2, CW = BN / WN / 2;  // lines of one half that belong to one wave
+    constexpr int TNH = TN / 2;
     constexpr int C_LD = BN + 8;
     constexpr int HALF_C_BYTES = (BM / 2) * C_LD * 2;  // staged output rows of one wave row-group
     constexpr int BUF_BYTES = STAGE_BYTES > HALF_C_BYTES ? STAGE_BYTES : HALF_C_BYTES;
-    // Two separate LDS objects, one per stage: a read of one stage then provably does not touch the other, so
-    // the compiler does not make fragment reads wait for the copies that are filling the other stage.
     __shared__ __attribute__((aligned(1024))) char lds0[BUF_BYTES];
     __shared__ __attribute__((aligned(1024))) char lds1[BUF_BYTES];
     __shared__ int sh_info[4];
@@ -589,73 +597,85 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
     const int cols_valid = GLU == 1 ? BN : min(BN, p.N - n_base);  // > 0 and a multiple of 8
 
     // ---- global sources of the LDS slots this lane fills ---------------------------------------------
-    // address = wave-uniform base of the tile (scalar registers, advanced by a fixed step per tile) + a 32-bit
-    // byte offset per lane and copy instruction.  Lines / chunks outside the problem are redirected to a valid
-    // one (their LDS content never reaches a stored output), so tiles inside the contraction range need no
-    // predicate at all.
     typedef __attribute__((address_space(1))) const char* gchar_t;
-    typedef __attribute__((address_space(1))) const void* gptr_t;
     typedef __attribute__((address_space(3))) void* lptr_t;
     const gchar_t a_base = (gchar_t)p.A + (A_KC ? (int64_t)k_begin : (int64_t)k_begin * p.lda + i_base) * 2;
     const gchar_t b_base = (gchar_t)p.B + ((GROUP_K ? 0 : (int64_t)expert * p.b_stride_e) +
                                           (B_KCC ? (int64_t)k_begin : (int64_t)k_begin * p.ldb + n_base)) * 2;
     const int64_t a_step = (A_KC ? (int64_t)BK : (int64_t)BK * p.lda) * 2;
     const int64_t b_step = (B_KCC ? (int64_t)BK : (int64_t)BK * p.ldb) * 2;
-    uint32_t a_voff[AOp::IPW], b_voff[BOp::IPW];
+    uint32_t a_voff[2][IPW], b_voff[2][IPW];
     {
         const int lane = lane_id();
 #pragma unroll
-        for (int j = 0; j < AOp::IPW; ++j) {
-            int line, chunk;
-            AOp::slot_source((wave * AOp::IPW + j) * CK_WAVE + lane, line, chunk);
-            if (A_KC) {
-                const int64_t slot = row_start + min(line, rows_valid - 1);
-                const int64_t src_row = p.x_grouped ? slot : (int64_t)((uint32_t)p.row_idx[slot] / (uint32_t)p.fan_out);
-                a_voff[j] = (uint32_t)((src_row * p.lda + chunk * 8) * 2);
-            } else {
-                const int cc = (chunk * 8 < rows_valid) ? chunk * 8 : 0;
-                a_voff[j] = (uint32_t)(((int64_t)line * p.lda + cc) * 2);
-            }
-        }
+        for (int h = 0; h < 2; ++h)
 #pragma unroll
-        for (int j = 0; j < BOp::IPW; ++j) {
-            int line, chunk;
-            BOp::slot_source((wave * BOp::IPW + j) * CK_WAVE + lane, line, chunk);
-            if (B_KCC) {
-                const int r = min(line, cols_valid - 1);
-                const int w_row = (GLU == 1 && r >= BN / 2) ? p.glu_half + n_base + r - BN / 2 : n_base + r;
-                b_voff[j] = (uint32_t)(((int64_t)w_row * p.ldb + chunk * 8) * 2);
-            } else {
-                const int cc = (chunk * 8 < cols_valid) ? chunk * 8 : 0;
-                b_voff[j] = (uint32_t)(((int64_t)line * p.ldb + cc) * 2);
+            for (int j = 0; j < IPW; ++j) {
+                int line, chunk;
+                AOp::slot_source((wave * IPW + j) * CK_WAVE + lane, line, chunk);
+                if (A_KC) {
+                    const int trow = (line / RW) * (2 * RW) + h * RW + line % RW;
+                    const int64_t slot = row_start + min(trow, rows_valid - 1);
+                    const int64_t src_row = p.x_grouped ? slot : (int64_t)((uint32_t)p.row_idx[slot] / (uint32_t)p.fan_out);
+                    a_voff[h][j] = (uint32_t)((src_row * p.lda + chunk * 8) * 2);
+                } else {
+                    const int l0 = chunk * 8;
+                    const int tcol = (l0 / RW) * (2 * RW) + h * RW + l0 % RW;
+                    const int cc = tcol < rows_valid ? tcol : 0;
+                    a_voff[h][j] = (uint32_t)(((int64_t)line * p.lda + cc) * 2);
+                }
             }
-        }
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int j = 0; j < IPW; ++j) {
+                int line, chunk;
+                BOp::slot_source((wave * IPW + j) * CK_WAVE + lane, line, chunk);
+                if (B_KCC) {
+                    const int tcol = (line / CW) * (2 * CW) + h * CW + line % CW;
+                    const int r = min(tcol, cols_valid - 1);
+                    const int w_row = (GLU == 1 && r >= BN / 2) ? p.glu_half + n_base + r - BN / 2 : n_base + r;
+                    b_voff[h][j] = (uint32_t)(((int64_t)w_row * p.ldb + chunk * 8) * 2);
+                } else {
+                    const int l0 = chunk * 8;
+                    const int tcol = (l0 / CW) * (2 * CW) + h * CW + l0 % CW;
+                    const int cc = tcol < cols_valid ? tcol : 0;
+                    b_voff[h][j] = (uint32_t)(((int64_t)line * p.ldb + cc) * 2);
+                }
+            }
     }
 
-    constexpr int LOADS = AOp::IPW + BOp::IPW;  // copy instructions per wave per tile, A first
-    // copy instructions [j0, j1) of tile t, which lies completely inside the contraction range
-    auto issue_range = [&](char* st, int j0, int j1, int t) __attribute__((always_inline)) {
-        // the tile bases are made opaque so that they stay in scalar registers and each copy is addressed as
-        // scalar base + 32-bit lane offset, instead of being folded into 64-bit per-lane pointers
-        const gchar_t at = (gchar_t)opaque_s64((uint64_t)(a_base + (int64_t)t * a_step));
-        const gchar_t bt = (gchar_t)opaque_s64((uint64_t)(b_base + (int64_t)t * b_step));
+    // One copy instruction: 64 lanes x 16 bytes from (wave-uniform base + 32-bit lane offset) to 1 KB of LDS at dst.
+    // Written as assembly so that the compiler's wait-count bookkeeping does not see the LDS writes: the waits for
+    // them are placed by hand below.
+    // (m0 carries the LDS address of the copy; nothing else in this kernel uses it)
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+    auto dma = [&](gchar_t base, uint32_t voff, const char* dst) __attribute__((always_inline)) {
+        const uint32_t la = (uint32_t)(uintptr_t)((lptr_t)dst);
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(la), "v"(voff), "s"((uint64_t)base)
+                     : "memory", "m0");
+    };
+#pragma clang diagnostic pop
+    // one half operand (0: A lower, 1: A upper, 2: B lower, 3: B upper) of tile t, which lies inside the contraction range
+    auto issue_part = [&](char* st, int part, int t) __attribute__((always_inline)) {
+        if (part < 2) {
+            const gchar_t at = a_base + (int64_t)t * a_step;
 #pragma unroll
-        for (int j = 0; j < LOADS; ++j) {
-            if (j < j0 || j >= j1) continue;
-            if (j < AOp::IPW) {
-                __builtin_amdgcn_global_load_lds((gptr_t)(at + a_voff[j]), (lptr_t)(st + (wave * AOp::IPW + j) * 1024), 16, 0, 0);
-            } else {
-                const int jb = j - AOp::IPW;
-                __builtin_amdgcn_global_load_lds((gptr_t)(bt + b_voff[jb]),
-                                                 (lptr_t)(st + AOp::STAGE_BYTES + (wave * BOp::IPW + jb) * 1024), 16, 0, 0);
-            }
+            for (int j = 0; j < IPW; ++j) dma(at, a_voff[part][j], st + part * A_HALF + (wave * IPW + j) * 1024);
+        } else {
+            const gchar_t bt = b_base + (int64_t)t * b_step;
+#pragma unroll
+            for (int j = 0; j < IPW; ++j)
+                dma(bt, b_voff[part - 2][j], st + B_AT + (part - 2) * B_HALF + (wave * IPW + j) * 1024);
         }
     };
     // tile t whatever its position: slots past the end of the contraction range are cleared instead of copied
     auto issue = [&](int t, char* st) __attribute__((always_inline)) {
         const int k0 = k_begin + t * BK;
         if (k0 + BK <= k_end) {
-            issue_range(st, 0, LOADS, t);
+#pragma unroll
+            for (int part = 0; part < 4; ++part) issue_part(st, part, t);
             return;
         }
         const gchar_t at = a_base + (int64_t)t * a_step;
@@ -663,35 +683,32 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
         const int lane = opaque(lane_id());
         const u32x4_t zero = {0u, 0u, 0u, 0u};
 #pragma unroll
-        for (int j = 0; j < AOp::IPW; ++j) {
-            int line, chunk;
-            AOp::slot_source((wave * AOp::IPW + j) * CK_WAVE + lane, line, chunk);
-            char* dst = st + (wave * AOp::IPW + j) * 1024;
-            if (k0 + (A_KC ? chunk * 8 : line) < k_end)
-                __builtin_amdgcn_global_load_lds((gptr_t)(at + a_voff[j]), (lptr_t)dst, 16, 0, 0);
-            else
-                *reinterpret_cast<u32x4_t*>(dst + lane * 16) = zero;
-        }
+        for (int h = 0; h < 2; ++h)
 #pragma unroll
-        for (int j = 0; j < BOp::IPW; ++j) {
-            int line, chunk;
-            BOp::slot_source((wave * BOp::IPW + j) * CK_WAVE + lane, line, chunk);
-            char* dst = st + AOp::STAGE_BYTES + (wave * BOp::IPW + j) * 1024;
-            if (k0 + (B_KCC ? chunk * 8 : line) < k_end)
-                __builtin_amdgcn_global_load_lds((gptr_t)(bt + b_voff[j]), (lptr_t)dst, 16, 0, 0);
-            else
-                *reinterpret_cast<u32x4_t*>(dst + lane * 16) = zero;
-        }
+            for (int j = 0; j < IPW; ++j) {
+                int line, chunk;
+                AOp::slot_source((wave * IPW + j) * CK_WAVE + lane, line, chunk);
+                char* dst = st + h * A_HALF + (wave * IPW + j) * 1024;
+                if (k0 + (A_KC ? chunk * 8 : line) < k_end)
+                    dma(at, a_voff[h][j], dst);
+                else
+                    *reinterpret_cast<u32x4_t*>(dst + lane * 16) = zero;
+            }
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int j = 0; j < IPW; ++j) {
+                int line, chunk;
+                BOp::slot_source((wave * IPW + j) * CK_WAVE + lane, line, chunk);
+                char* dst = st + B_AT + h * B_HALF + (wave * IPW + j) * 1024;
+                if (k0 + (B_KCC ? chunk * 8 : line) < k_end)
+                    dma(bt, b_voff[h][j], dst);
+                else
+                    *reinterpret_cast<u32x4_t*>(dst + lane * 16) = zero;
+            }
     };
 
     // ---- fragment addresses (bytes inside a stage) -----------------------------------------------------
-    // v_mfma_f32_16x16x32: lane l holds row (or column) l % 16 and the 8 contraction indices 8 * (l / 16) .. + 7.
-    // k-contiguous operand: row r starts at r * 128, chunk c sits in slot c ^ ((r >> 1) & 7).  A lane reads chunk
-    //   kk / 8 + l / 16 of row l % 16 + 16 * i; kk / 8 is 0 or 4 and l / 16 < 4, so the slot is
-    //   (lane-dependent part) ^ (kk / 8) and i adds a compile-time multiple of 2048 bytes.
-    // other layout (contraction row = ROWS * 2 bytes, chunk c of row k in slot c ^ ((k & 3) << 2)): two transposing
-    //   reads; in each group of 16 lanes, lane q fetches elements 4 (q % 4) .. + 3 of contraction row q / 4 (then
-    //   + 4) of the 16-wide block, and receives element q of each of the four rows.
     int frag_row, frag_swz;
     int a_off[TM], b_off[TN];
     {
@@ -701,61 +718,70 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
         const int g = lane / 16, q = lane % 16;
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
-            const int r0 = wm * (BM / WM) + i * 16;
+            const int l0 = wm * RW + (i % TH) * 16;
             if (A_KC) {
-                a_off[i] = r0 * 128;
+                a_off[i] = (i / TH) * A_HALF + l0 * 128;
             } else {
-                const int col = r0 + (q % 4) * 4;
-                a_off[i] = (g * 8 + q / 4) * (BM * 2) + ((((col / 8) ^ ((q / 4) << 2))) << 4) + (col % 8) * 2;
+                const int col = l0 + (q % 4) * 4;
+                a_off[i] = (i / TH) * A_HALF + (g * 8 + q / 4) * BM + ((((col / 8) ^ ((q / 4) << 2))) << 4) + (col % 8) * 2;
             }
         }
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-            const int c0 = wn * (BN / WN) + j * 16;
+            const int l0 = wn * CW + (j % TNH) * 16;
             if (B_KCC) {
-                b_off[j] = AOp::STAGE_BYTES + c0 * 128;
+                b_off[j] = B_AT + (j / TNH) * B_HALF + l0 * 128;
             } else {
-                const int col = c0 + (q % 4) * 4;
-                b_off[j] = AOp::STAGE_BYTES + (g * 8 + q / 4) * (BN * 2) + ((((col / 8) ^ ((q / 4) << 2))) << 4) + (col % 8) * 2;
+                const int col = l0 + (q % 4) * 4;
+                b_off[j] = B_AT + (j / TNH) * B_HALF + (g * 8 + q / 4) * BN + ((((col / 8) ^ ((q / 4) << 2))) << 4) + (col % 8) * 2;
             }
         }
     }
-    // fragments of rows [16 * TH * half, + 16 * TH) of the wave's block, contraction indices kk .. kk + 31
-    auto read_a = [&](const char* st, int kk, int half, frag_t* af) __attribute__((always_inline)) {
-        const int kc = frag_row + (opaque(frag_swz) ^ ((kk / 8) << 4));
+    // fragments of one half of the wave's rows, both contraction groups of 32: af[kk / 32][i]
+    auto read_a = [&](const char* st, int h, frag_t (*af)[TH]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < TH; ++i) {
-            if (A_KC) {
-                af[i] = *reinterpret_cast<const frag_t*>(st + kc + a_off[half * TH + i]);
-            } else {
-                // blocks 2m and 2m + 1 differ in bit 1 of the chunk index only, below the swizzled bits: + 32 bytes
-                const int ii = half * TH + i;
-                const char* q = st + a_off[ii & ~1] + (ii & 1) * 32 + kk * (BM * 2);
-                union {
-                    v4i16_t h[2];
-                    frag_t f;
-                } u;
-                u.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(q));
-                u.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(q + 4 * (BM * 2)));
-                af[i] = u.f;
+        for (int kki = 0; kki < 2; ++kki) {
+            const int kk = kki * 32;
+            const int kc = frag_row + (opaque(frag_swz) ^ ((kk / 8) << 4));
+#pragma unroll
+            for (int i = 0; i < TH; ++i) {
+                const int ii = h * TH + i;
+                if (A_KC) {
+                    af[kki][i] = *reinterpret_cast<const frag_t*>(st + kc + a_off[ii]);
+                } else {
+                    // a contraction row of a half operand is BM / 2 elements = BM bytes
+                    const char* q = st + a_off[ii & ~1] + (ii & 1) * 32 + kk * BM;
+                    union {
+                        v4i16_t h2[2];
+                        frag_t f;
+                    } u;
+                    u.h2[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(q));
+                    u.h2[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(q + 4 * BM));
+                    af[kki][i] = u.f;
+                }
             }
         }
     };
-    auto read_b = [&](const char* st, int kk, frag_t* bf) __attribute__((always_inline)) {
-        const int kc = frag_row + (opaque(frag_swz) ^ ((kk / 8) << 4));
+    auto read_b = [&](const char* st, int h, frag_t (*bf)[TNH]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            if (B_KCC) {
-                bf[j] = *reinterpret_cast<const frag_t*>(st + kc + b_off[j]);
-            } else {
-                const char* q = st + b_off[j & ~1] + (j & 1) * 32 + kk * (BN * 2);
-                union {
-                    v4i16_t h[2];
-                    frag_t f;
-                } u;
-                u.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(q));
-                u.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(q + 4 * (BN * 2)));
-                bf[j] = u.f;
+        for (int kki = 0; kki < 2; ++kki) {
+            const int kk = kki * 32;
+            const int kc = frag_row + (opaque(frag_swz) ^ ((kk / 8) << 4));
+#pragma unroll
+            for (int j = 0; j < TNH; ++j) {
+                const int jj = h * TNH + j;
+                if (B_KCC) {
+                    bf[kki][j] = *reinterpret_cast<const frag_t*>(st + kc + b_off[jj]);
+                } else {
+                    const char* q = st + b_off[jj & ~1] + (jj & 1) * 32 + kk * BN;
+                    union {
+                        v4i16_t h2[2];
+                        frag_t f;
+                    } u;
+                    u.h2[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(q));
+                    u.h2[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(q + 4 * BN));
+                    bf[kki][j] = u.f;
+                }
             }
         }
     };
@@ -768,106 +794,129 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
 
-    auto mma_half = [&](int half, const frag_t* af, const frag_t* bf) __attribute__((always_inline)) {
+    // one quarter of the wave's block: rows of half ha times columns of half hb, over the whole tile depth
+    auto mma_quad = [&](int ha, int hb, frag_t (*af)[TH], frag_t (*bf)[TNH]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < TH; ++i)
+        for (int kki = 0; kki < 2; ++kki)
 #pragma unroll
-            for (int j = 0; j < TN; ++j) acc[half * TH + i][j] = Mma16<T>::mma(af[i], bf[j], acc[half * TH + i][j]);
+            for (int i = 0; i < TH; ++i)
+#pragma unroll
+                for (int j = 0; j < TNH; ++j)
+                    acc[ha * TH + i][hb * TNH + j] = Mma16<T>::mma(af[kki][i], bf[kki][j], acc[ha * TH + i][hb * TNH + j]);
     };
-    // Order inside one group of TH * TN MFMAs: each MFMA is followed by at most one LDS read of the group and at
-    // most one copy instruction.  Nothing crosses the group boundary.
-    static_assert((TH * (A_KC ? 1 : 2) + TN * (B_KCC ? 1 : 2)) <= TH * TN, "one LDS read per MFMA must be enough");
-    auto pin_group = [&](int copies) __attribute__((always_inline)) {
-#pragma unroll
-        for (int m = 0; m < TH * TN; ++m) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            if (m < copies) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-    };
-    // one whole tile, fragments read as they are needed (used outside the pipelined loop)
+    frag_t fa[2][TH], fb0[2][TNH], fb1[2][TNH];
+    // one whole tile, outside the pipelined loop
     auto multiply_tile = [&](const char* st) __attribute__((always_inline)) {
-#pragma unroll
-        for (int kk = 0; kk < BK; kk += 32) {
-            frag_t bf[TN];
-            read_b(st, kk, bf);
-#pragma unroll
-            for (int half = 0; half < 2; ++half) {
-                frag_t af[TH];
-                read_a(st, kk, half, af);
-                mma_half(half, af, bf);
-            }
-        }
-    };
-    // unpipelined step: request tile kt + 1 (whole, clipped to the contraction range), multiply tile kt
-    auto plain_step = [&](int kt, int k_tiles, const char* cur, char* fill) __attribute__((always_inline)) {
-        if (kt + 1 < k_tiles) issue(kt + 1, fill);
-        multiply_tile(cur);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
+        read_a(st, 0, fa);
+        read_b(st, 0, fb0);
+        read_b(st, 1, fb1);
+        mma_quad(0, 0, fa, fb0);
+        mma_quad(0, 1, fa, fb1);
+        __builtin_amdgcn_sched_barrier(0);
+        read_a(st, 1, fa);
+        mma_quad(1, 1, fa, fb1);
+        mma_quad(1, 0, fa, fb0);
     };
 
-    // Pipelined step over tile kt in X while tile kt + 1 arrives in Y.  A tile is two contraction groups of 32,
-    // each multiplied in two halves of the wave's rows: four groups of TH * TN MFMAs.  On entry the fragments of
-    // the first group (lower rows + columns of contraction group 0) are in registers.
-    //   group 0   reads the upper rows of contraction group 0
-    //   group 1   reads the lower rows and the columns of contraction group 1
-    //   group 2   reads the upper rows of contraction group 1 - the last fragments of X
-    //   then every wave waits for its copies and meets the others: tile kt + 1 is complete in Y, X is free
-    //   group 3   multiplies those last fragments while the first fragments of Y are read and the copies of tile
-    //             kt + 2 start filling X: three groups of matrix work pass before anybody waits for them
-    frag_t a_lo[TH], a_hi[TH], b_0[TN], b_1[TN];
-    auto pipe_step = [&](int kt, char* X, char* Y) __attribute__((always_inline)) {
-        read_a(X, 0, 1, a_hi);
-        mma_half(0, a_lo, b_0);
-        pin_group(0);
-        read_a(X, 32, 0, a_lo);
-        read_b(X, 32, b_1);
-        mma_half(1, a_hi, b_0);
-        pin_group(0);
-        read_a(X, 32, 1, a_hi);
-        mma_half(0, a_lo, b_1);
-        pin_group(0);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        read_a(Y, 0, 0, a_lo);
-        read_b(Y, 0, b_0);
-        issue_range(X, 0, LOADS, kt + 2);
-        mma_half(1, a_hi, b_1);
-        pin_group(LOADS);
-    };
-
+    // ---- the pipelined loop ----------------------------------------------------------------------------
+    // The waves of the lower row group (0 .. 3, one per SIMD) and of the upper row group (4 .. 7) run the same
+    // sequence of phases, the upper group one phase behind: while one wave of a SIMD issues a quarter of its
+    // matrix instructions (C phase), the other reads the next fragments and requests copies (M phase).  A wave
+    // that waits for the copy path to take its request then never holds up matrix instructions.  Every phase ends
+    // at a workgroup barrier.  Tile kt is read from X while tile kt + 2 is copied over the halves of X as they
+    // fall free:
+    //   M0 reads A lower of X           copies B lower (last read in M3 of the step before)
+    //   M1 reads B upper                copies A lower
+    //   M2 reads A upper                copies B upper
+    //   M3 reads B lower of Y           copies A upper
+    // so every copy has seven M phases until its half is read again, and a wait that leaves the twelve most recent
+    // copies of the wave outstanding (two per M phase) at the end of each M phase covers it: what the next M phase
+    // of either group reads was requested at least six M phases before this one, and the barrier that ends the
+    // phase passes that on to the other waves.
+#define CK_PHASE_END()                           \
+    do {                                         \
+        __builtin_amdgcn_sched_barrier(0);       \
+        __builtin_amdgcn_s_barrier();            \
+        __builtin_amdgcn_sched_barrier(0);       \
+    } while (0)
+    // An M phase ends with a wait that leaves the twelve most recent copies of the wave outstanding.
+#define CK_M_END(PART)                                        \
+    do {                                                      \
+        issue_part(X, PART, tf);                              \
+        asm volatile("s_waitcnt vmcnt(12)" ::: "memory");     \
+        __builtin_amdgcn_s_waitcnt(0xC07F); /* lgkmcnt(0) */  \
+        CK_PHASE_END();                                       \
+    } while (0)
     const int k_tiles = (k_end - k_begin + BK - 1) / BK;
     const int n_full = (k_end - k_begin) / BK;  // leading tiles that lie completely inside the range
-    const bool primed = n_full >= 2;
+    auto pp_step = [&](int kt, char* X, char* Y, frag_t (*bl)[TNH], frag_t (*bu)[TNH]) __attribute__((always_inline)) {
+        // The last two steps of a range have no tile left to request; they request the last tile once more, into
+        // halves that nobody reads again, which keeps the count of outstanding copies the same in every step (a
+        // branch around the copies, with its own wait, measured slower than the 2 / 64 of copy work it saves).
+        const int tf = min(kt + 2, n_full - 1);
+        read_a(X, 0, fa);
+        CK_M_END(2);
+        __builtin_amdgcn_s_setprio(1);
+        mma_quad(0, 0, fa, bl);
+        __builtin_amdgcn_s_setprio(0);
+        CK_PHASE_END();
+        read_b(X, 1, bu);
+        CK_M_END(0);
+        __builtin_amdgcn_s_setprio(1);
+        mma_quad(0, 1, fa, bu);
+        __builtin_amdgcn_s_setprio(0);
+        CK_PHASE_END();
+        read_a(X, 1, fa);
+        CK_M_END(3);
+        __builtin_amdgcn_s_setprio(1);
+        mma_quad(1, 1, fa, bu);
+        __builtin_amdgcn_s_setprio(0);
+        CK_PHASE_END();
+        // lower columns of the next tile, over the registers of this tile's upper columns (after the last tile of a
+        // range this reads a stage that nobody uses any more)
+        read_b(Y, 0, bu);
+        CK_M_END(1);
+        __builtin_amdgcn_s_setprio(1);
+        mma_quad(1, 0, fa, bl);
+        __builtin_amdgcn_s_setprio(0);
+        CK_PHASE_END();
+    };
+
     int kt = 0;
-    if (primed) {
-        issue_range(lds0, 0, LOADS, 0);
-        issue_range(lds1, 0, LOADS, 1);
+    if (n_full >= 2) {
+#pragma unroll
+        for (int part = 0; part < 4; ++part) issue_part(lds0, part, 0);
+#pragma unroll
+        for (int part = 0; part < 4; ++part) issue_part(lds1, part, 1);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        read_a(lds0, 0, 0, a_lo);
-        read_b(lds0, 0, b_0);
-        // two steps per turn so that each names its buffers statically; the loop leaves with tile kt complete in
-        // lds0, the copies of tile kt + 1 under way and at most three more tiles to go
-        for (; kt + 3 < n_full; kt += 2) {
-            pipe_step(kt, lds0, lds1);
-            pipe_step(kt + 1, lds1, lds0);
+        read_b(lds0, 0, fb0);
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+        CK_PHASE_END();
+        if (wm == 1) CK_PHASE_END();  // the upper group falls one phase behind
+        // two steps per turn so that each names its buffers and registers statically
+        for (; kt + 1 < n_full; kt += 2) {
+            pp_step(kt, lds0, lds1, fb0, fb1);
+            pp_step(kt + 1, lds1, lds0, fb1, fb0);
         }
-    } else {
-        if (k_tiles > 0) issue(0, lds0);
+        if (wm == 0) CK_PHASE_END();
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if (1 < k_tiles) issue(1, lds1);
+        if (kt < n_full) {  // an odd number of full tiles: the last one is complete in lds0
+            multiply_tile(lds0);
+            ++kt;
+            __syncthreads();
+        }
     }
-    if (k_tiles > 0) multiply_tile(lds0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    for (int t = kt + 1; t < k_tiles; t += 2) {
-        plain_step(t, k_tiles, lds1, lds0);
-        if (t + 1 < k_tiles) plain_step(t + 1, k_tiles, lds0, lds1);
+    for (; kt < k_tiles; ++kt) {
+        issue(kt, lds0);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        multiply_tile(lds0);
+        __syncthreads();
     }
+#undef CK_M_END
+#undef CK_PHASE_END
 
     // ---- epilogue -----------------------------------------------------------------------------------
     // Accumulators (lane: column lane % 16, rows 4 * (lane / 16) + r of each 16x16 tile) are
