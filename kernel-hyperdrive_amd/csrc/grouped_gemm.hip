@@ -546,8 +546,10 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
     constexpr bool A_KC = !GROUP_K;
     constexpr bool B_KCC = GROUP_K ? false : B_KC;
     // Each operand tile lies in LDS as two halves of 128 lines, [A lower | A upper | B lower | B upper], 16 KB each.
-    // "Lower" holds the first half of every wave's rows (columns): line l of the lower A half is tile row
-    // (l / RW) * 2 RW + l % RW, of the upper half RW more; for B the same with CW.
+    // The halves are the tile's rows [0, BM / 2) and [BM / 2, BM), columns [0, BN / 2) and [BN / 2, BN): where rows or
+    // columns are the contiguous dimension in memory, a half's lines are then whole 256-byte runs (interleaved
+    // 32-column groups split every 128-byte line between the halves and measured 47 % more requests to L2).  Wave
+    // (wm, wn) owns rows wm * RW .. + RW of either A half and columns wn * CW .. + CW of either B half.
     typedef DtlOperand<S, BM / 2, A_KC, NWAVES> AOp;
     typedef DtlOperand<S, BN / 2, B_KCC, NWAVES> BOp;
     static_assert(AOp::IPW == BOp::IPW && AOp::IPW == 2, "square tile; the wait counts of the loop assume two copies per M phase");
@@ -614,13 +616,12 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
                 int line, chunk;
                 AOp::slot_source((wave * IPW + j) * CK_WAVE + lane, line, chunk);
                 if (A_KC) {
-                    const int trow = (line / RW) * (2 * RW) + h * RW + line % RW;
+                    const int trow = h * (BM / 2) + line;
                     const int64_t slot = row_start + min(trow, rows_valid - 1);
                     const int64_t src_row = p.x_grouped ? slot : (int64_t)((uint32_t)p.row_idx[slot] / (uint32_t)p.fan_out);
                     a_voff[h][j] = (uint32_t)((src_row * p.lda + chunk * 8) * 2);
                 } else {
-                    const int l0 = chunk * 8;
-                    const int tcol = (l0 / RW) * (2 * RW) + h * RW + l0 % RW;
+                    const int tcol = h * (BM / 2) + chunk * 8;
                     const int cc = tcol < rows_valid ? tcol : 0;
                     a_voff[h][j] = (uint32_t)(((int64_t)line * p.lda + cc) * 2);
                 }
@@ -632,13 +633,12 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
                 int line, chunk;
                 BOp::slot_source((wave * IPW + j) * CK_WAVE + lane, line, chunk);
                 if (B_KCC) {
-                    const int tcol = (line / CW) * (2 * CW) + h * CW + line % CW;
+                    const int tcol = h * (BN / 2) + line;
                     const int r = min(tcol, cols_valid - 1);
                     const int w_row = (GLU == 1 && r >= BN / 2) ? p.glu_half + n_base + r - BN / 2 : n_base + r;
                     b_voff[h][j] = (uint32_t)(((int64_t)w_row * p.ldb + chunk * 8) * 2);
                 } else {
-                    const int l0 = chunk * 8;
-                    const int tcol = (l0 / CW) * (2 * CW) + h * CW + l0 % CW;
+                    const int tcol = h * (BN / 2) + chunk * 8;
                     const int cc = tcol < cols_valid ? tcol : 0;
                     b_voff[h][j] = (uint32_t)(((int64_t)line * p.ldb + cc) * 2);
                 }
@@ -920,26 +920,46 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
 
     // ---- epilogue -----------------------------------------------------------------------------------
     // Accumulators (lane: column lane % 16, rows 4 * (lane / 16) + r of each 16x16 tile) are
-    // rounded and staged in LDS - the upper half of the rows in one stage buffer, the lower half in the other -
+    // rounded and staged in LDS - the tile's upper half of the rows in one stage buffer, the lower half in the other -
     // then written out as 16-byte packets along rows, rows going to their mapped position.
     const int lane = opaque(lane_id());
-    S* Ch = reinterpret_cast<S*>(wm == 0 ? lds0 : lds1);
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+    for (int i = 0; i < TM; ++i) {
+        S* Ch = reinterpret_cast<S*>(i / TH == 0 ? lds0 : lds1);  // tile rows [0, BM / 2) are staged in lds0, the rest in lds1
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const int row = i * 16 + 4 * (lane / 16) + r;  // inside this half
-                const int col = wn * (BN / WN) + j * 16 + lane % 16;
+                const int row = wm * RW + (i % TH) * 16 + 4 * (lane / 16) + r;  // inside this half of the tile
+                const int col = (j / TNH) * (BN / 2) + wn * CW + (j % TNH) * 16 + lane % 16;
                 Ch[row * C_LD + col] = T::down(acc[i][j][r]);
             }
-    __syncthreads();
+    }
     S* Cbase = reinterpret_cast<S*>(p.C) + (GROUP_K ? (int64_t)expert * p.c_stride_e : 0);
     typedef VPack<T, 8> P8;
     // GLU == 1: a lane takes an "up" packet together with its "gate" packet, so packets are counted over half a row
     constexpr int C_CHUNKS_PER_ROW = (GLU == 1 ? BN / 2 : BN) / 8;
     constexpr int C_CH = BM * C_CHUNKS_PER_ROW / THREADS;
+    // GLU == 2: the up / gate packets of h that this lane's packets need are requested here, all of them at once and
+    // without branches (positions outside the tile are redirected to a valid one), while the accumulator registers
+    // are free and the workgroup is on its way to the barrier; inside the store loop each packet would wait for its
+    // own two loads in turn.
+    constexpr int H_CH = GLU == 2 ? C_CH : 1;
+    P8 h_up[H_CH], h_gate[H_CH];
+    if (GLU == 2) {
+#pragma unroll
+        for (int i = 0; i < C_CH; ++i) {
+            const int c = tid + i * THREADS;
+            const int row = min(c / C_CHUNKS_PER_ROW, rows_valid - 1);
+            const int col = min((c % C_CHUNKS_PER_ROW) * 8, cols_valid - 8);
+            const int64_t slot = row_start + row;
+            const int64_t out_row = p.y_grouped ? slot : p.row_idx[slot];
+            const S* hrow = reinterpret_cast<const S*>(p.aux) + out_row * p.ld_aux + n_base + col;
+            h_up[i] = nt_load(reinterpret_cast<const P8*>(hrow));
+            h_gate[i] = nt_load(reinterpret_cast<const P8*>(hrow + p.glu_half));
+        }
+    }
+    __syncthreads();
 #pragma unroll
     for (int i = 0; i < C_CH; ++i) {
         const int c = tid + i * THREADS;
@@ -971,9 +991,8 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
             } else {
                 // the staged tile is d_act (rounded, as the separate kernels would hand it over); h supplies up
                 // and gate of the same positions, and d_h receives both derivatives
-                const S* hrow = reinterpret_cast<const S*>(p.aux) + out_row * p.ld_aux + n_base + col;
-                const P8 u = nt_load(reinterpret_cast<const P8*>(hrow));
-                const P8 g = nt_load(reinterpret_cast<const P8*>(hrow + p.glu_half));
+                const P8 u = h_up[GLU == 2 ? i : 0];
+                const P8 g = h_gate[GLU == 2 ? i : 0];
                 const P8 d = *reinterpret_cast<const P8*>(src);
                 P8 du, dg;
 #pragma unroll
