@@ -214,6 +214,25 @@ int ck_moe_combine_backward_gates(const void* expanded, const void* grad_out, vo
                                   int64_t k, int64_t H, int dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * Routing weights: top-k of the router logits and the softmax over the k selected values
+ * replaces the stock torch ops of MoE_Torch._compute_routing_weights / _get_topk
+ * (scattermoe/torch_implementation.py:121-132, 193-199: topk or max, .float(), softmax, type_as) and the
+ * backward ops autograd derives from them.
+ *   forward : logits [tokens, E] (row stride logits_stride, unit column stride) ->
+ *             selected [tokens, k] int64: positions of the k largest logits, largest first (ties: the lower
+ *             position first; NaN counts as the largest value, as in torch.topk),
+ *             weights [tokens, k] (storage type) and weights_f32 [tokens, k]: softmax over the k values in fp32.
+ *   backward: d_logits [tokens, E] = softmax backward of d_weights on weights_f32, placed at the selected
+ *             positions, zero elsewhere; every element is written.
+ * E <= 1024, k <= min(E, 64); weights, weights_f32, selected and d_weights are dense.
+ * ------------------------------------------------------------------------------------------- */
+int ck_router_topk_softmax_forward(const void* logits, int64_t logits_stride, void* weights, float* weights_f32,
+                                   int64_t* selected, int64_t tokens, int64_t E, int64_t k, int dtype, void* stream);
+int ck_router_topk_softmax_backward(const void* d_weights, const float* weights_f32, const int64_t* selected,
+                                    void* d_logits, int64_t d_logits_stride, int64_t tokens, int64_t E, int64_t k,
+                                    int dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
  * Per-expert bias of the grouped linears
  * replaces the bias term of F.linear(rows_e, W[e], bias[e]) in scattermoe/torch_implementation.py:35-43 (the
  * reference's Triton experts, triton_implementation/__init__.py:24-34, do not read their bias parameter).

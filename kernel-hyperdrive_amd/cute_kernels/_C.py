@@ -70,6 +70,8 @@ _SIGNATURES = {
     "ck_moe_combine_backward_gates": (_i32, [_p, _p, _p, _i64, _i64, _i64, _i32, _p]),
     "ck_expert_bias_forward": (_i32, [_p, _i64, _p, _i64, _p, _p, _i64, _i64, _i64, _i32, _p]),
     "ck_expert_bias_backward": (_i32, [_p, _i64, _p, _p, _i64, _i64, _i64, _i64, _i32, _p]),
+    "ck_router_topk_softmax_forward": (_i32, [_p, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, _p]),
+    "ck_router_topk_softmax_backward": (_i32, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i32, _p]),
     "ck_probe_mfma": (_i32, [_p, _i64, _i32, _p, _p]),
 }
 
@@ -498,6 +500,50 @@ def expert_bias_backward(dy, expert_offsets, d_bias) -> None:
             lib.ck_expert_bias_backward(_ptr(dy), dy.stride(0), _ptr(expert_offsets), _ptr(d_bias), d_bias.stride(0),
                                         dy.size(0), dy.size(1), d_bias.size(0), dtype_code(dy.dtype), L.stream),
             "ck_expert_bias_backward",
+        )
+
+
+ROUTER_MAX_EXPERTS = 1024
+ROUTER_MAX_TOP_K = 64
+
+
+def router_topk_softmax_forward(logits, weights, weights_f32, selected) -> None:
+    """logits [T, E] -> selected [T, k] int64 (largest first), weights [T, k] in logits' dtype and in fp32."""
+    lib = load_library()
+    T, E = logits.shape
+    k = selected.size(1)
+    if logits.stride(1) != 1:
+        raise ValueError("router_topk_softmax_forward needs unit column stride for the logits")
+    if weights.dtype != logits.dtype or weights_f32.dtype != torch.float32 or selected.dtype != torch.int64:
+        raise ValueError("router_topk_softmax_forward: weights in the logits' dtype, weights_f32 fp32, selected int64")
+    for out in (weights, weights_f32, selected):
+        if tuple(out.shape) != (T, k) or not out.is_contiguous():
+            raise ValueError("router_topk_softmax_forward: outputs must be dense [tokens, k]")
+    with _Launch(logits, weights, weights_f32, selected) as L:
+        _check(
+            lib.ck_router_topk_softmax_forward(_ptr(logits), logits.stride(0), _ptr(weights), _ptr(weights_f32),
+                                               _ptr(selected), T, E, k, dtype_code(logits.dtype), L.stream),
+            "ck_router_topk_softmax_forward",
+        )
+
+
+def router_topk_softmax_backward(d_weights, weights_f32, selected, d_logits) -> None:
+    """d_logits [T, E] from d_weights [T, k], the fp32 weights and the selected positions of the forward."""
+    lib = load_library()
+    T, E = d_logits.shape
+    k = selected.size(1)
+    if d_logits.stride(1) != 1:
+        raise ValueError("router_topk_softmax_backward needs unit column stride for d_logits")
+    if d_weights.dtype != d_logits.dtype or weights_f32.dtype != torch.float32 or selected.dtype != torch.int64:
+        raise ValueError("router_topk_softmax_backward: d_weights in d_logits' dtype, weights_f32 fp32, selected int64")
+    for t in (d_weights, weights_f32, selected):
+        if tuple(t.shape) != (T, k) or not t.is_contiguous():
+            raise ValueError("router_topk_softmax_backward: d_weights, weights_f32 and selected must be dense [tokens, k]")
+    with _Launch(d_weights, weights_f32, selected, d_logits) as L:
+        _check(
+            lib.ck_router_topk_softmax_backward(_ptr(d_weights), _ptr(weights_f32), _ptr(selected), _ptr(d_logits),
+                                                d_logits.stride(0), T, E, k, dtype_code(d_logits.dtype), L.stream),
+            "ck_router_topk_softmax_backward",
         )
 
 

@@ -50,6 +50,66 @@ def moe_sort(selected_experts: torch.Tensor, num_experts: int) -> tuple[torch.Te
     return moe_sort_hip(flat, num_experts)
 
 
+def _router_forward_fake(router_logits: torch.Tensor, top_k: int):
+    T = router_logits.size(0)
+    return (
+        torch.empty(T, top_k, dtype=router_logits.dtype, device=router_logits.device),
+        torch.empty(T, top_k, dtype=torch.float32, device=router_logits.device),
+        torch.empty(T, top_k, dtype=torch.int64, device=router_logits.device),
+    )
+
+
+@cute_op(f"{LIBRARY_NAME}::router_topk_softmax_forward_hip", mutates_args={}, fake_func=_router_forward_fake)
+def router_topk_softmax_forward_hip(
+    router_logits: torch.Tensor, top_k: int
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    T = router_logits.size(0)
+    device = router_logits.device
+    weights = torch.empty(T, top_k, dtype=router_logits.dtype, device=device)
+    weights_f32 = torch.empty(T, top_k, dtype=torch.float32, device=device)
+    selected = torch.empty(T, top_k, dtype=torch.int64, device=device)
+    _C.router_topk_softmax_forward(router_logits, weights, weights_f32, selected)
+    return weights, weights_f32, selected
+
+
+def _router_backward_fake(d_weights: torch.Tensor, weights_f32: torch.Tensor, selected: torch.Tensor, num_experts: int):
+    return torch.empty(d_weights.size(0), num_experts, dtype=d_weights.dtype, device=d_weights.device)
+
+
+@cute_op(f"{LIBRARY_NAME}::router_topk_softmax_backward_hip", mutates_args={}, fake_func=_router_backward_fake)
+def router_topk_softmax_backward_hip(
+    d_weights: torch.Tensor, weights_f32: torch.Tensor, selected: torch.Tensor, num_experts: int
+) -> torch.Tensor:
+    d_logits = torch.empty(d_weights.size(0), num_experts, dtype=d_weights.dtype, device=d_weights.device)
+    _C.router_topk_softmax_backward(d_weights.contiguous(), weights_f32, selected, d_logits)
+    return d_logits
+
+
+class _RouterTopKSoftmax(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, router_logits, top_k):
+        if router_logits.stride(1) != 1:
+            router_logits = router_logits.contiguous()
+        weights, weights_f32, selected = router_topk_softmax_forward_hip(router_logits, top_k)
+        ctx.save_for_backward(weights_f32, selected)
+        ctx.num_experts = router_logits.size(1)
+        ctx.mark_non_differentiable(selected)
+        return weights, selected
+
+    @staticmethod
+    def backward(ctx, d_weights, _d_selected):
+        weights_f32, selected = ctx.saved_tensors
+        return router_topk_softmax_backward_hip(d_weights, weights_f32, selected, ctx.num_experts), None
+
+
+def router_topk_softmax(router_logits: torch.Tensor, top_k: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """``(router_weights [T, k], selected_experts [T, k])`` from ``router_logits [T, E]``: what
+    ``MoE_Torch._compute_routing_weights`` makes of the logits with topk (max for k = 1), ``.float()``, softmax and
+    ``type_as`` (torch_implementation.py:121-132, 193-199), forward and backward one launch each.  Equal logits are
+    taken in the order of their positions (torch.topk leaves that order open)."""
+    return _RouterTopKSoftmax.apply(router_logits, top_k)
+
+
 class Experts_HIP(Experts_Torch):
     """The grouped linears on the HIP kernels.  ``add_bias=True`` applies the ``[E, out]`` bias as the plain-torch
     experts do (torch_implementation.py:35-43); the reference's ``Experts_Triton`` holds the same parameter and
@@ -86,6 +146,19 @@ class MoE_HIP(MoE_Torch):
     # GEMMs' epilogues (same values, two passes over the intermediate activations fewer).  False keeps the three
     # separate autograd nodes of the reference layer.
     fuse_swiglu = True
+    # Top-k, softmax and their backward as one launch each instead of the stock torch ops (False: inherited routing).
+    fuse_router = True
+
+    def _compute_routing_weights(self, hidden_states: torch.Tensor):
+        if not (
+            self.fuse_router
+            and self.num_experts <= _C.ROUTER_MAX_EXPERTS
+            and self.top_k <= min(self.num_experts, _C.ROUTER_MAX_TOP_K)
+        ):
+            return super()._compute_routing_weights(hidden_states)
+        router_logits = self.gate(hidden_states)  # [T, E]
+        router_weights, selected_experts = router_topk_softmax(router_logits, self.top_k)
+        return router_logits, router_weights, selected_experts
 
     def _compute_experts(
         self, hidden_states: torch.Tensor, router_weights: torch.Tensor, selected_experts: torch.Tensor

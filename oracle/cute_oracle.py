@@ -20,6 +20,9 @@ stock torch ops on random inputs):
   moe_sort            stable argsort; checked against a brute-force insertion on tiny inputs
   moe_combine_*       the two torch.bmm calls of scattermoe/triton_implementation/ops.py:160-164, 204; checked
                       against torch.bmm in fp64
+  router_topk_softmax the routing of MoE_Torch (scattermoe/torch_implementation.py:121-132, 193-199); checked against
+                      torch.topk + softmax on tie-free logits, a brute-force selection on tiny inputs with ties, and
+                      the closed form of the softmax gradient in fp64
   expert_bias_*       the bias term of F.linear(rows_e, W[e], bias[e]) (scattermoe/torch_implementation.py:35-43);
                       checked against F.linear per expert and its autograd in fp64
   scatter2scatter, group_bwd_W, group
@@ -259,6 +262,28 @@ def expert_bias_backward(dy, expert_offsets, compute_dtype=torch.float32):
             out[e] = dy[start:end].to(compute_dtype).sum(0)
         start = end
     return out.to(dy.dtype)
+
+
+def router_topk_softmax(router_logits: torch.Tensor, top_k: int, compute_dtype=torch.float32):
+    """(weights [T, k], selected [T, k]) of MoE_Torch._compute_routing_weights / _get_topk
+    (scattermoe/torch_implementation.py:121-132, 193-199): the k largest logits per token, largest first, and the
+    softmax over them in fp32 rounded to the logits' dtype.  Equal logits are taken in the order of their positions
+    (a stable descending sort); torch.topk leaves that order open."""
+    order = torch.sort(router_logits.to(torch.float64), dim=-1, descending=True, stable=True).indices
+    selected = order[:, :top_k].contiguous()
+    values = router_logits.gather(1, selected)
+    weights = F.softmax(values.to(compute_dtype), dim=-1).to(router_logits.dtype)
+    return weights, selected
+
+
+def router_topk_softmax_backward(d_weights, router_logits, selected, compute_dtype=torch.float32):
+    """d_logits of ``router_topk_softmax`` for fixed ``selected``: autograd through gather, .float(), softmax and the
+    cast back, the result in the logits' dtype."""
+    logits = router_logits.detach().clone().requires_grad_(True)
+    values = logits.gather(1, selected)
+    weights = F.softmax(values.to(compute_dtype), dim=-1).to(router_logits.dtype)
+    weights.backward(d_weights)
+    return logits.grad
 
 
 def _acc_dtype(x: torch.Tensor) -> torch.dtype:

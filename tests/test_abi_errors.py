@@ -138,6 +138,25 @@ def test_grouped_gemm_argument_checks(lib):
     assert bias_bwd(P, 64, P, P, 64, 16, 64, 2, 3, None) == DTYPE
     assert bias_bwd(P, 64, P, P + 2, 64, 16, 64, 2, F32, None) == ALIGN
     assert bias_bwd(P, 64, P, P, 64, 16, 0, 2, BF16, None) == OK  # no columns
+    router = lib.ck_router_topk_softmax_forward
+    #           logits ld w  w32 sel T  E   k  dtype stream
+    assert router(P, 8, P, P, P, 16, 0, 1, BF16, None) == SHAPE  # no experts
+    assert router(P, 8, P, P, P, 16, 8, 9, BF16, None) == SHAPE  # k > E
+    assert router(P, 2048, P, P, P, 16, 2048, 2, BF16, None) == SHAPE  # more experts than the kernel takes
+    assert router(P, 128, P, P, P, 16, 128, 65, BF16, None) == SHAPE  # k above one wavefront
+    assert router(P, 4, P, P, P, 16, 8, 2, BF16, None) == SHAPE  # row stride below the row length
+    assert router(None, 8, P, P, P, 16, 8, 2, BF16, None) == NULL
+    assert router(P, 8, P, None, P, 16, 8, 2, BF16, None) == NULL
+    assert router(P, 8, P, P, P, 16, 8, 2, 7, None) == DTYPE
+    assert router(P + 1, 8, P, P, P, 16, 8, 2, BF16, None) == ALIGN
+    assert router(P, 8, P, P, P, 0, 8, 2, BF16, None) == OK  # no tokens
+    router_bwd = lib.ck_router_topk_softmax_backward
+    #               dw w32 sel d_logits ld T  E  k  dtype stream
+    assert router_bwd(P, P, P, P, 8, 16, 8, 0, BF16, None) == SHAPE
+    assert router_bwd(P, P, None, P, 8, 16, 8, 2, BF16, None) == NULL
+    assert router_bwd(P, P, P, None, 8, 16, 8, 2, BF16, None) == NULL
+    assert router_bwd(P, P, P, P, 8, 16, 8, 2, 9, None) == DTYPE
+    assert router_bwd(P, P, P, P + 2, 8, 16, 8, 2, F32, None) == ALIGN
     assert lib.ck_probe_mfma(None, 10, 1, P, None) == NULL
     assert lib.ck_probe_mfma(P, 10, 0, P, None) == SHAPE
 

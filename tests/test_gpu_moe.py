@@ -206,6 +206,66 @@ def test_moe_combine(gpu, dtype, shape):
         assert_close(d_gates, expected, dtype, "d_gates")
 
 
+# ---- router ---------------------------------------------------------------------------------------------
+ROUTER_CASES = [
+    # T, E, k, ties
+    (64, 8, 2, False),
+    (1000, 8, 2, True),
+    (333, 64, 6, True),
+    (50, 5, 5, False),
+    (129, 100, 3, True),   # two values per lane
+    (77, 1024, 64, True),  # the limits of the kernel
+    (9, 1, 1, False),
+    (16384, 8, 1, True),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("T,E,k,ties", ROUTER_CASES)
+def test_router_topk_softmax(gpu, dtype, T, E, k, ties):
+    from cute_kernels.kernels.scattermoe import router_topk_softmax
+
+    announce("router", dtype, T, E, k, ties)
+    logits = randn((T, E), dtype, seed=81)
+    if ties:
+        logits = (logits * 2).round() / 2  # values from a small set: many equal logits in a row
+    d_weights = randn((T, k), dtype, seed=82)
+    # a view with a row stride wider than E, as a slice of a larger tensor would be
+    wide = torch.zeros(T, E + 3, dtype=dtype, device=gpu)
+    wide[:, :E] = logits.to(gpu)
+    for source in (logits.to(gpu), wide[:, :E]):
+        x = source.detach().requires_grad_(True)
+        weights, selected = router_topk_softmax(x, k)
+        exp_w, exp_sel = O.router_topk_softmax(logits, k)
+        assert torch.equal(selected.cpu(), exp_sel), "positions: largest first, equal values in the order of their positions"
+        assert_close(weights, exp_w, dtype, "routing weights")
+        weights.backward(d_weights.to(gpu))
+        expected = O.router_topk_softmax_backward(d_weights, logits, exp_sel)
+        assert_close(x.grad, expected, dtype, "d_logits")
+        outside = torch.ones(T, E, dtype=torch.bool).scatter_(1, exp_sel, False)
+        assert torch.count_nonzero(x.grad.cpu()[outside]) == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_router_matches_the_stock_ops_on_the_device(gpu, dtype):
+    """Without equal logits the fused routing selects what torch.topk selects, and its weights are those of
+    softmax(topk(.).float()).type_as(.) computed by torch on the same device."""
+    from cute_kernels.kernels.scattermoe import router_topk_softmax
+
+    logits = (randn((4096, 64), torch.float32, seed=83) * 3).to(gpu)
+    if dtype != torch.float32:
+        # spread the values so that the 16-bit roundings of a row stay distinct
+        logits = (torch.argsort(torch.argsort(logits, dim=-1), dim=-1).float() * 0.125 - 4).to(dtype)
+    logits = logits.to(dtype)
+    weights, selected = router_topk_softmax(logits, 6)
+    vals, idx = logits.topk(6, dim=-1)
+    assert torch.equal(selected, idx)
+    stock = torch.softmax(vals.float(), dim=-1).type_as(logits)
+    assert_close(weights, stock, dtype, "weights against the stock ops")
+    if dtype != torch.float32:
+        assert (weights != stock).float().mean().item() < 1e-3  # the two exp implementations round alike
+
+
 # ---- per-expert bias -------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("T,k,E,N,empty", [(16, 2, 4, 128, ()), (300, 3, 7, 200, (0, 6)), (257, 2, 5, 36, (2,)),

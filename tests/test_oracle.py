@@ -327,6 +327,33 @@ def test_expert_bias_ops_against_linear_per_expert():
     assert torch.allclose(got[perm], expected.detach(), rtol=1e-13, atol=1e-13)
 
 
+def test_router_topk_softmax_against_topk_brute_force_and_closed_form():
+    g = torch.Generator().manual_seed(11)
+    logits = torch.randn(37, 12, generator=g, dtype=F64)  # fp64 random values: no ties
+    for k in (1, 2, 5, 12):
+        weights, selected = O.router_topk_softmax(logits, k, compute_dtype=F64)
+        vals, idx = logits.topk(k, dim=-1)
+        assert torch.equal(selected, idx)
+        assert torch.allclose(weights, torch.softmax(vals, -1), rtol=1e-14, atol=0)
+        assert torch.allclose(weights.sum(-1), torch.ones(37, dtype=F64), rtol=1e-14, atol=0)
+    # ties: values from a set of three, brute force "largest value first, lower position first"
+    tied = torch.randint(0, 3, (50, 7), generator=g).double()
+    _, selected = O.router_topk_softmax(tied, 4, compute_dtype=F64)
+    for t in range(50):
+        row = tied[t].tolist()
+        expected = sorted(range(7), key=lambda e: (-row[e], e))[:4]
+        assert selected[t].tolist() == expected
+    # gradient: d_v_j = w_j (g_j - sum_i g_i w_i) at the selected positions, zero elsewhere
+    k = 3
+    weights, selected = O.router_topk_softmax(logits, k, compute_dtype=F64)
+    d_weights = torch.randn(37, k, generator=g, dtype=F64)
+    d_logits = O.router_topk_softmax_backward(d_weights, logits, selected, compute_dtype=F64)
+    d_v = weights * (d_weights - (d_weights * weights).sum(-1, keepdim=True))
+    assert torch.allclose(d_logits.gather(1, selected), d_v, rtol=1e-12, atol=1e-15)
+    assert torch.count_nonzero(d_logits) == 37 * k
+    assert torch.allclose(d_logits.sum(-1), torch.zeros(37, dtype=F64), atol=1e-15)  # softmax gradients sum to zero
+
+
 def test_moe_single_expert_is_a_plain_mlp():
     T, H, I = 7, 8, 5
     x, wg, wfc, wproj, dy = (t.double() for t in O.moe_inputs(T, H, I, 1, torch.float32, seed=4))
