@@ -146,6 +146,19 @@ int ck_scatter2scatter(const void* X, int64_t x_stride, const void* W, int64_t w
                        int64_t K, int64_t N, int64_t E, int64_t fan_out, int x_grouped, int y_grouped,
                        int dtype, void* stream);
 
+/* The same product with the tail of the tile grid split along the contraction (no counterpart in the reference).
+ * A product with few column tiles leaves most CUs idle during its last round of tiles; given a workspace of
+ * ck_scatter2scatter_workspace_size() bytes (16-byte aligned; 0: the shape is not eligible - fp32, or K below 4096),
+ * the tiles of every XCD's last round are cut into pieces of the contraction range, summed by a second launch on the
+ * same stream.  Results differ from ck_scatter2scatter in the order of the fp32 additions only.  workspace == NULL
+ * is ck_scatter2scatter. */
+int64_t ck_scatter2scatter_workspace_size(int64_t num_slots, int64_t K, int64_t N, int64_t E, int dtype);
+int ck_scatter2scatter_ws(const void* X, int64_t x_stride, const void* W, int64_t w_stride_e, int64_t w_stride_k,
+                          int64_t w_stride_n, const int64_t* sorted_scattered_idxs, const int64_t* expert_offsets,
+                          void* out, int64_t out_stride, int64_t num_slots, int64_t K, int64_t N, int64_t E,
+                          int64_t fan_out, int x_grouped, int y_grouped, int dtype, void* workspace,
+                          int64_t workspace_bytes, void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * scatter2scatter with the SwiGLU of the MoE layer in its epilogue.
  * replaces, in one launch each, the pairs of calls the reference layer makes around its activation

@@ -71,6 +71,9 @@ struct GemmParams {
     void* aux;
     int64_t ld_aux;
     int glu_half;
+    // Tail splitting of the per-expert products (kernel template argument MODE, see find_tile_split): fp32 partial
+    // tiles, kSplitSlots of them, BM * BN floats each
+    float* partials;
 };
 
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -195,6 +198,106 @@ __device__ __forceinline__ void find_tile_balanced(const int64_t* __restrict__ o
             sh_info[1] = found_start;
             sh_info[2] = found_rows;
             sh_info[3] = nt;
+        }
+    }
+    __syncthreads();
+}
+
+// The same search with the last, partly filled round of every XCD split along the contraction.  A product with few
+// column tiles has only a few rounds of tiles per CU (1088 tiles of a Mixtral c_proj over 256 CUs: 4.25), and the
+// CUs without a tile in the last round idle for a whole tile time.  Every XCD (32 CUs) takes an even share of the
+// tiles; if the share leaves a last round of rem <= 16 tiles, each of them is cut into s = 32 / rem pieces of the
+// contraction range, worked on by s workgroups that write fp32 partial tiles to a workspace; a second launch
+// (MODE 2) adds the pieces up and runs the epilogue.  Pieces are at least 32 contraction tiles long (the partial
+// tiles cost two passes over 256 KB per piece and the second launch a few microseconds).
+//   sh_info: 0 expert (< 0: nothing to do), 1 first row, 2 valid rows, 3 column tile, 4 / 5 first and end
+//   contraction tile of this workgroup, 6 partial slot (< 0: a whole tile), 7 pieces per tile in this XCD's tail
+// fixup = true (MODE 2): workgroup (x, i) = (blockIdx.x % 8, blockIdx.x / 8) owns tail tile i of XCD x, if there is one.
+constexpr int kSplitSlots = 256, kSplitMinTiles = 32, kSplitMax = 8;
+
+template <int BM, int BK>
+__device__ __forceinline__ void find_tile_split(const int64_t* __restrict__ offsets, int E, int n_tiles, int K, bool fixup,
+                                                int* sh_info) {
+    if (threadIdx.x < CK_WAVE) {
+        constexpr int XCDS = 8, GROUP_M = 8, CUS = 32;
+        const int lane = lane_id();
+        int m_tiles = 0;
+        for (int e0 = 0; e0 < E; e0 += CK_WAVE) {
+            const int e = e0 + lane;
+            int tiles = 0;
+            if (e < E) tiles = ((int)offsets[e] - (e == 0 ? 0 : (int)offsets[e - 1]) + BM - 1) / BM;
+            m_tiles += wave_sum_i(tiles);
+        }
+        const int total = m_tiles * n_tiles;
+        const int per_xcd = (total + XCDS - 1) / XCDS;
+        const int xcd = blockIdx.x % XCDS, pos = blockIdx.x / XCDS;
+        const int base = xcd * per_xcd;
+        const int mine = max(0, min(per_xcd, total - base));  // tiles of this XCD
+        const int full = mine / CUS * CUS, rem = mine - full;
+        const int k_tiles = (K + BK - 1) / BK;
+        int pieces = 1;
+        if (rem > 0 && rem <= CUS / 2) pieces = max(1, min(min(CUS / rem, kSplitMax), k_tiles / kSplitMinTiles));
+        int L = -1, kt_b = 0, kt_e = k_tiles, slot = -1;
+        if (fixup) {
+            if (pieces > 1 && pos < rem) {
+                L = base + full + pos;
+                slot = xcd * CUS + pos * pieces;  // the first of the tile's pieces
+            }
+        } else if (pos < full) {
+            L = base + pos;
+        } else {
+            const int i = pos - full;
+            if (i < rem * pieces) {
+                L = base + full + i / pieces;
+                if (pieces > 1) {
+                    const int c = i % pieces;
+                    kt_b = (int)((int64_t)c * k_tiles / pieces);
+                    kt_e = (int)((int64_t)(c + 1) * k_tiles / pieces);
+                    slot = xcd * CUS + i;
+                }
+            }
+        }
+        int found_e = -1, found_start = 0, found_rows = 0, nt = 0;
+        if (L >= 0) {
+            const int group_span = GROUP_M * n_tiles;
+            const int group = L / group_span;
+            const int first_m = group * GROUP_M;
+            const int gm = min(GROUP_M, m_tiles - first_m);
+            const int in_group = L - group * group_span;
+            const int mt = first_m + in_group % gm;
+            nt = in_group / gm;
+            int base_tiles = 0;
+            for (int e0 = 0; e0 < E && found_e < 0; e0 += CK_WAVE) {
+                const int e = e0 + lane;
+                int begin = 0, end = 0;
+                if (e < E) {
+                    end = (int)offsets[e];
+                    begin = e == 0 ? 0 : (int)offsets[e - 1];
+                }
+                const int tiles = (end - begin + BM - 1) / BM;
+                const int incl = wave_inclusive_scan_i(tiles) + base_tiles;
+                const uint64_t hit = __ballot(e < E && incl > mt);
+                if (hit != 0) {
+                    const int src = __ffsll((unsigned long long)hit) - 1;
+                    const int excl = __shfl(incl - tiles, src, CK_WAVE);
+                    const int b = __shfl(begin, src, CK_WAVE);
+                    const int en = __shfl(end, src, CK_WAVE);
+                    found_e = e0 + src;
+                    found_start = b + (mt - excl) * BM;
+                    found_rows = min(BM, en - found_start);
+                }
+                base_tiles = __shfl(incl, CK_WAVE - 1, CK_WAVE);
+            }
+        }
+        if (lane == 0) {
+            sh_info[0] = found_e;
+            sh_info[1] = found_start;
+            sh_info[2] = found_rows;
+            sh_info[3] = nt;
+            sh_info[4] = kt_b;
+            sh_info[5] = kt_e;
+            sh_info[6] = slot;
+            sh_info[7] = pieces;
         }
     }
     __syncthreads();
@@ -530,11 +633,15 @@ __device__ __forceinline__ uint64_t opaque_s64(uint64_t v) {  // same for a wave
     return v;
 }
 
-template <typename T, typename TL, bool B_KC, bool GROUP_K, int GLU = 0>
+// MODE 0: one workgroup per tile.  MODE 1: tiles dealt by find_tile_split; a workgroup with a piece of a tile writes its
+// fp32 accumulators to p.partials instead of running the epilogue.  MODE 2: the launch that follows MODE 1 - one
+// workgroup per split tile adds the pieces up and runs the epilogue.
+template <typename T, typename TL, bool B_KC, bool GROUP_K, int GLU = 0, int MODE = 0>
 // Two waves per SIMD is all the LDS footprint allows; telling the compiler keeps it from spilling to reach a
 // higher occupancy that cannot happen.
 __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
     grouped_gemm_m16_kernel(GemmParams p) {
+    static_assert(MODE == 0 || (GLU == 0 && !GROUP_K), "tail splitting is for the plain per-expert products");
     typedef typename T::storage_t S;
     typedef typename Mma16<T>::frag_t frag_t;
     constexpr int BM = TL::BM, BN = TL::BN, BK = 64, WM = TL::WM, WN = TL::WN;
@@ -563,7 +670,7 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
     constexpr int BUF_BYTES = STAGE_BYTES > HALF_C_BYTES ? STAGE_BYTES : HALF_C_BYTES;
     __shared__ __attribute__((aligned(1024))) char lds0[BUF_BYTES];
     __shared__ __attribute__((aligned(1024))) char lds1[BUF_BYTES];
-    __shared__ int sh_info[4];
+    __shared__ int sh_info[8];
 
     int nt = 0;
     const int tid = threadIdx.x;
@@ -571,8 +678,12 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
     const int wm = wave / WN, wn = wave % WN;
 
     int expert, row_start, rows_valid, k_begin, k_end, i_base;
+    int part_slot = -1, part_pieces = 1;
     if (!GROUP_K) {
-        find_tile_balanced<BM>(p.offsets, p.E, p.n_tiles, sh_info);
+        if (MODE == 0)
+            find_tile_balanced<BM>(p.offsets, p.E, p.n_tiles, sh_info);
+        else
+            find_tile_split<BM, BK>(p.offsets, p.E, p.n_tiles, p.K, MODE == 2, sh_info);
         expert = __builtin_amdgcn_readfirstlane(sh_info[0]);
         row_start = __builtin_amdgcn_readfirstlane(sh_info[1]);
         rows_valid = __builtin_amdgcn_readfirstlane(sh_info[2]);
@@ -580,6 +691,14 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
         if (expert < 0) return;
         k_begin = 0;
         k_end = p.K;
+        if (MODE != 0) {
+            part_slot = __builtin_amdgcn_readfirstlane(sh_info[6]);
+            part_pieces = __builtin_amdgcn_readfirstlane(sh_info[7]);
+            if (MODE == 1 && part_slot >= 0) {
+                k_begin = __builtin_amdgcn_readfirstlane(sh_info[4]) * BK;
+                k_end = min(p.K, __builtin_amdgcn_readfirstlane(sh_info[5]) * BK);
+            }
+        }
         i_base = 0;
     } else {
         int rank, it;
@@ -883,7 +1002,8 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
     };
 
     int kt = 0;
-    if (n_full >= 2) {
+    if (MODE == 2) kt = k_tiles;  // nothing to multiply: the accumulators come from the partial tiles below
+    if (MODE != 2 && n_full >= 2) {
 #pragma unroll
         for (int part = 0; part < 4; ++part) issue_part(lds0, part, 0);
 #pragma unroll
@@ -917,6 +1037,33 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
     }
 #undef CK_M_END
 #undef CK_PHASE_END
+
+    // ---- pieces of a split tile ------------------------------------------------------------------------
+    // A partial tile is stored the way the accumulators lie in the registers: float4 number
+    // ((wave * TM + i) * TN + j) * 64 + lane of the slot, so both directions move 1 KB per wave instruction.
+    if (MODE == 1 && part_slot >= 0) {
+        f32x4_t* dst = reinterpret_cast<f32x4_t*>(p.partials) + (int64_t)part_slot * (BM * BN / 4);
+        const int l = lane_id();
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) dst[((wave * TM + i) * TN + j) * CK_WAVE + l] = acc[i][j];
+        return;
+    }
+    if (MODE == 2) {
+        const f32x4_t* src = reinterpret_cast<const f32x4_t*>(p.partials) + (int64_t)part_slot * (BM * BN / 4);
+        const int l = lane_id();
+        for (int c = 0; c < part_pieces; ++c) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    const f32x4_t v = src[(int64_t)c * (BM * BN / 4) + ((wave * TM + i) * TN + j) * CK_WAVE + l];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[i][j][r] += v[r];
+                }
+        }
+    }
 
     // ---- epilogue -----------------------------------------------------------------------------------
     // Accumulators (lane: column lane % 16, rows 4 * (lane / 16) + r of each 16x16 tile) are
@@ -1151,6 +1298,21 @@ void launch_mfma(const ck::GemmParams& p, hipStream_t s) {
                            dim3(MainTile::THREADS), 0, s, p);
 }
 
+// per-expert product whose last round of tiles is split along the contraction (see find_tile_split): the tiles,
+// then the sums of the split ones
+template <typename T, bool B_KC>
+void launch_mfma_split(const ck::GemmParams& p, hipStream_t s) {
+    const int64_t per_xcd = ((int64_t)p.m_tiles * p.n_tiles + 7) / 8 + 32;  // the pieces of a tail take up to 32 places
+    hipLaunchKernelGGL((ck::grouped_gemm_m16_kernel<T, MainTile, B_KC, false, 0, 1>), dim3((unsigned)(8 * per_xcd)),
+                       dim3(MainTile::THREADS), 0, s, p);
+    hipLaunchKernelGGL((ck::grouped_gemm_m16_kernel<T, MainTile, B_KC, false, 0, 2>), dim3(8 * 16),
+                       dim3(MainTile::THREADS), 0, s, p);
+}
+
+constexpr int64_t kSplitWorkspaceBytes = (int64_t)ck::kSplitSlots * kBM * kBN * 4;
+// contraction lengths from which a tile can be cut into two pieces of kSplitMinTiles contraction tiles
+constexpr int64_t kSplitMinK = 2 * ck::kSplitMinTiles * 64;
+
 // per-expert product with the SwiGLU epilogue GLU (1: forward, 2: backward); never the wide kernel
 template <typename T, bool B_KC, int GLU>
 void launch_mfma_glu(const ck::GemmParams& p, hipStream_t s) {
@@ -1162,11 +1324,26 @@ bool mult8(int64_t v) { return (v & 7) == 0; }
 
 }  // namespace
 
+extern "C" int64_t ck_scatter2scatter_workspace_size(int64_t num_slots, int64_t K, int64_t N, int64_t E, int dtype) {
+    if (num_slots <= 0 || N <= 0 || E <= 0 || dtype == CK_F32 || K < kSplitMinK) return 0;
+    return kSplitWorkspaceBytes;
+}
+
 extern "C" int ck_scatter2scatter(const void* X, int64_t x_stride, const void* W, int64_t w_stride_e,
                                   int64_t w_stride_k, int64_t w_stride_n, const int64_t* sorted_scattered_idxs,
                                   const int64_t* expert_offsets, void* out, int64_t out_stride, int64_t num_slots,
                                   int64_t K, int64_t N, int64_t E, int64_t fan_out, int x_grouped, int y_grouped,
                                   int dtype, void* stream) {
+    return ck_scatter2scatter_ws(X, x_stride, W, w_stride_e, w_stride_k, w_stride_n, sorted_scattered_idxs, expert_offsets,
+                                 out, out_stride, num_slots, K, N, E, fan_out, x_grouped, y_grouped, dtype, nullptr, 0,
+                                 stream);
+}
+
+extern "C" int ck_scatter2scatter_ws(const void* X, int64_t x_stride, const void* W, int64_t w_stride_e,
+                                     int64_t w_stride_k, int64_t w_stride_n, const int64_t* sorted_scattered_idxs,
+                                     const int64_t* expert_offsets, void* out, int64_t out_stride, int64_t num_slots,
+                                     int64_t K, int64_t N, int64_t E, int64_t fan_out, int x_grouped, int y_grouped,
+                                     int dtype, void* workspace, int64_t workspace_bytes, void* stream) {
     if (num_slots < 0 || K < 0 || N < 0 || E <= 0 || fan_out <= 0) return CK_ERR_SHAPE;
     if (num_slots > 0x7fffffff || K > 0x7fffffff || N > 0x7fffffff || E > 0x7fffffff) return CK_ERR_SHAPE;
     if (dtype != CK_F32 && dtype != CK_F16 && dtype != CK_BF16) return CK_ERR_DTYPE;
@@ -1202,7 +1379,20 @@ extern "C" int ck_scatter2scatter(const void* X, int64_t x_stride, const void* W
         p.wide = num_slots * x_stride * 2 >= (int64_t)1 << 32 || (b_kc ? N : K) * p.ldb * 2 >= (int64_t)1 << 32;
         p.m_tiles = (int)(num_slots / kBM + E);
         p.n_tiles = (int)ck_ceil_div(N, kBN);
-        if ((int64_t)(p.m_tiles + 8) * p.n_tiles > 0x7ffffff0) return CK_ERR_SHAPE;
+        if ((int64_t)(p.m_tiles + 8) * p.n_tiles > 0x7ffffff0 - 256) return CK_ERR_SHAPE;
+        // with a workspace, the last round of tiles of every XCD is split along the contraction
+        if (workspace != nullptr && !p.wide && K >= kSplitMinK) {
+            if (workspace_bytes < kSplitWorkspaceBytes || !ck_aligned16(workspace)) return CK_ERR_WORKSPACE;
+            p.partials = static_cast<float*>(workspace);
+            if (dtype == CK_BF16) {
+                if (b_kc) launch_mfma_split<ck::BF16, true>(p, s);
+                else launch_mfma_split<ck::BF16, false>(p, s);
+            } else {
+                if (b_kc) launch_mfma_split<ck::F16, true>(p, s);
+                else launch_mfma_split<ck::F16, false>(p, s);
+            }
+            return ck_launch_status();
+        }
         if (dtype == CK_BF16) {
             if (b_kc) launch_mfma<ck::BF16, true, false>(p, s);
             else launch_mfma<ck::BF16, false, false>(p, s);

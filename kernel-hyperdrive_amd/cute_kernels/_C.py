@@ -55,6 +55,12 @@ _SIGNATURES = {
         _i32,
         [_p, _i64, _p, _i64, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _p],
     ),
+    "ck_scatter2scatter_ws": (
+        _i32,
+        [_p, _i64, _p, _i64, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _p, _i64,
+         _p],
+    ),
+    "ck_scatter2scatter_workspace_size": (_i64, [_i64, _i64, _i64, _i64, _i32]),
     "ck_scatter2scatter_glu": (
         _i32,
         [_p, _i64, _p, _i64, _i64, _i64, _p, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _p],
@@ -361,20 +367,27 @@ def offsets_from_sorted(sorted_expert_idxs, expert_offsets) -> None:
         )
 
 
+def scatter2scatter_workspace_size(num_slots: int, K: int, N: int, E: int, dtype) -> int:
+    """Bytes of workspace with which ``scatter2scatter`` splits the tail of its tile grid (0: not for this shape)."""
+    return int(load_library().ck_scatter2scatter_workspace_size(num_slots, K, N, E, dtype_code(dtype)))
+
+
 def scatter2scatter(X, W, sorted_scattered_idxs, expert_offsets, out, fan_out: int, x_grouped: bool,
-                    y_grouped: bool) -> None:
-    """X [*, K] (unit column stride), W strided view [E, K, N], out [slots, N] (unit column stride)."""
+                    y_grouped: bool, workspace=None) -> None:
+    """X [*, K] (unit column stride), W strided view [E, K, N], out [slots, N] (unit column stride); ``workspace``:
+    uint8 tensor of ``scatter2scatter_workspace_size`` bytes or None."""
     lib = load_library()
     if X.stride(1) != 1 or out.stride(1) != 1:
         raise ValueError("scatter2scatter needs unit column stride for X and out")
     flop = 2.0 * out.size(0) * X.size(1) * out.size(1)
-    with _Launch(X, W, sorted_scattered_idxs, expert_offsets, out) as L, _Timed("scatter2scatter", flop):
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    with _Launch(X, W, sorted_scattered_idxs, expert_offsets, out, workspace) as L, _Timed("scatter2scatter", flop):
         _check(
-            lib.ck_scatter2scatter(_ptr(X), X.stride(0), _ptr(W), W.stride(0), W.stride(1), W.stride(2),
-                                   _ptr(sorted_scattered_idxs), _ptr(expert_offsets), _ptr(out), out.stride(0),
-                                   out.size(0), X.size(1), out.size(1), W.size(0), fan_out, int(x_grouped),
-                                   int(y_grouped), dtype_code(X.dtype), L.stream),
-            "ck_scatter2scatter",
+            lib.ck_scatter2scatter_ws(_ptr(X), X.stride(0), _ptr(W), W.stride(0), W.stride(1), W.stride(2),
+                                      _ptr(sorted_scattered_idxs), _ptr(expert_offsets), _ptr(out), out.stride(0),
+                                      out.size(0), X.size(1), out.size(1), W.size(0), fan_out, int(x_grouped),
+                                      int(y_grouped), dtype_code(X.dtype), _ptr(workspace), ws_bytes, L.stream),
+            "ck_scatter2scatter_ws",
         )
 
 

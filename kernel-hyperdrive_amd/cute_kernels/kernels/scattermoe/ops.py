@@ -32,6 +32,10 @@ from ...utils import cute_op
 
 torch._dynamo.config.capture_scalar_outputs = True
 
+# scatter2scatter splits the tail of its tile grid along the contraction when the shape allows it (False: one
+# workgroup per tile throughout)
+SPLIT_TILE_TAIL = True
+
 
 @cute_op(f"{LIBRARY_NAME}::scatter2scatter", mutates_args={"out"})
 def scatter2scatter(
@@ -56,7 +60,14 @@ def scatter2scatter(
         _C.offsets_from_sorted(sorted_expert_idxs.contiguous(), expert_offsets)
     if X.stride(1) != 1:
         X = X.contiguous()
-    _C.scatter2scatter(X, W, sorted_scattered_idxs, expert_offsets, out, FAN_OUT, x_grouped, y_grouped)
+    # long contractions over few column tiles: the last round of tiles is split over the idle CUs (needs room for
+    # the pieces' partial sums)
+    workspace = None
+    if SPLIT_TILE_TAIL:
+        nbytes = _C.scatter2scatter_workspace_size(out.size(0), X.size(1), out.size(1), W.size(0), X.dtype)
+        if nbytes > 0:
+            workspace = torch.empty(nbytes, dtype=torch.uint8, device=X.device)
+    _C.scatter2scatter(X, W, sorted_scattered_idxs, expert_offsets, out, FAN_OUT, x_grouped, y_grouped, workspace)
 
 
 @cute_op(f"{LIBRARY_NAME}::scatter2scatter_glu", mutates_args={"h", "act"})

@@ -61,6 +61,52 @@ def test_scatter2scatter(gpu, dtype, w_layout, mode, shape):
     assert torch.equal(out2, out)
 
 
+# ---- scatter2scatter with the tail of the tile grid split along the contraction ----------------------------
+SPLIT_SHAPES = [
+    # T, k, E, K, N, empty experts: few tiles, so every tile is the "last round" of its XCD and is cut into pieces
+    (300, 2, 3, 4096, 256, ()),    # two pieces of 32 contraction tiles
+    (100, 2, 4, 8192, 512, (1,)),  # four pieces, two column tiles, an empty expert
+    (260, 1, 2, 4160, 264, ()),    # contraction and columns not multiples of the tile
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("w_layout", ["k_contiguous", "n_contiguous"])
+@pytest.mark.parametrize("mode", ["gather_in", "scatter_out", "grouped_both"])
+@pytest.mark.parametrize("shape", SPLIT_SHAPES)
+def test_scatter2scatter_split_tail(gpu, dtype, w_layout, mode, shape):
+    """Long contractions take the variant that cuts the tiles of the last round into pieces: against the oracle,
+    and against the one-workgroup-per-tile launch (same products, fp32 sums formed in a different order)."""
+    from cute_kernels import _C
+    from cute_kernels.kernels.scattermoe import ops
+
+    T, k, E, K, N, empty = shape
+    announce("scatter2scatter split", dtype, w_layout, mode, shape)
+    s_e, s_idx, off = routing(T, k, E, 91, empty)
+    x_grouped = mode != "gather_in"
+    y_grouped = mode != "scatter_out"
+    fan_out = 1 if x_grouped else k
+    X = randn((T * k if x_grouped else T, K), dtype, 92, 0.25)
+    if w_layout == "k_contiguous":
+        W = randn((E, N, K), dtype, 93, 0.05).permute(0, 2, 1)
+        Wg = W.permute(0, 2, 1).contiguous().to(gpu).permute(0, 2, 1)
+    else:
+        W = randn((E, K, N), dtype, 93, 0.05)
+        Wg = W.to(gpu)
+    assert _C.scatter2scatter_workspace_size(T * k, K, N, E, dtype) > 0
+    assert ops.SPLIT_TILE_TAIL
+    out = torch.full((T * k, N), float("nan"), dtype=dtype, device=gpu)
+    ops.scatter2scatter(X.to(gpu), Wg, s_e.to(gpu), s_idx.to(gpu), out, fan_out, x_grouped, y_grouped, off.to(gpu))
+    expected = O.scatter2scatter(X, W, s_idx, off, fan_out, x_grouped, y_grouped, acc_dtype(dtype))
+    assert_close(out, expected, dtype, "out (split)")
+    whole = torch.full_like(out, float("nan"))
+    _C.scatter2scatter(X.to(gpu), Wg, s_idx.to(gpu), off.to(gpu), whole, fan_out, x_grouped, y_grouped, None)
+    assert_close(whole, expected, dtype, "out (one workgroup per tile)")
+    # the two differ by the rounding of fp32 sums added in another order: at most the last bit of a few elements
+    assert (out != whole).float().mean().item() < 0.02
+    assert_close(out, whole, dtype, "split against whole")
+
+
 # ---- grouped products with the SwiGLU in the epilogue ----------------------------------------------------
 GLU_SHAPES = [
     # T, k, E, K (hidden), I, empty experts
