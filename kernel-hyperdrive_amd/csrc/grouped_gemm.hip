@@ -913,7 +913,10 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
 
-    // one quarter of the wave's block: rows of half ha times columns of half hb, over the whole tile depth
+    // one quarter of the wave's block: rows of half ha times columns of half hb, over the whole tile depth.  The
+    // MFMA gets the column fragment as its first operand, i.e. it computes the 16 x 16 block transposed: a lane
+    // then holds four consecutive columns of one row (row lane % 16, columns 4 * (lane / 16) + r), which the
+    // epilogue stages with one 8-byte LDS store instead of four 2-byte ones.
     auto mma_quad = [&](int ha, int hb, frag_t (*af)[TH], frag_t (*bf)[TNH]) __attribute__((always_inline)) {
 #pragma unroll
         for (int kki = 0; kki < 2; ++kki)
@@ -921,7 +924,7 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
             for (int i = 0; i < TH; ++i)
 #pragma unroll
                 for (int j = 0; j < TNH; ++j)
-                    acc[ha * TH + i][hb * TNH + j] = Mma16<T>::mma(af[kki][i], bf[kki][j], acc[ha * TH + i][hb * TNH + j]);
+                    acc[ha * TH + i][hb * TNH + j] = Mma16<T>::mma(bf[kki][j], af[kki][i], acc[ha * TH + i][hb * TNH + j]);
     };
     frag_t fa[2][TH], fb0[2][TNH], fb1[2][TNH];
     // one whole tile, outside the pipelined loop
@@ -1066,7 +1069,7 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
     }
 
     // ---- epilogue -----------------------------------------------------------------------------------
-    // Accumulators (lane: column lane % 16, rows 4 * (lane / 16) + r of each 16x16 tile) are
+    // Accumulators (lane: row lane % 16, columns 4 * (lane / 16) + r of each 16x16 tile) are
     // rounded and staged in LDS - the tile's upper half of the rows in one stage buffer, the lower half in the other -
     // then written out as 16-byte packets along rows, rows going to their mapped position.
     const int lane = opaque(lane_id());
@@ -1074,13 +1077,14 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
     for (int i = 0; i < TM; ++i) {
         S* Ch = reinterpret_cast<S*>(i / TH == 0 ? lds0 : lds1);  // tile rows [0, BM / 2) are staged in lds0, the rest in lds1
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+        for (int j = 0; j < TN; ++j) {
+            const int row = wm * RW + (i % TH) * 16 + lane % 16;  // inside this half of the tile
+            const int col = (j / TNH) * (BN / 2) + wn * CW + (j % TNH) * 16 + 4 * (lane / 16);
+            VPack<T, 4> four;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int row = wm * RW + (i % TH) * 16 + 4 * (lane / 16) + r;  // inside this half of the tile
-                const int col = (j / TNH) * (BN / 2) + wn * CW + (j % TNH) * 16 + lane % 16;
-                Ch[row * C_LD + col] = T::down(acc[i][j][r]);
-            }
+            for (int r = 0; r < 4; ++r) four.v[r] = T::down(acc[i][j][r]);
+            *reinterpret_cast<VPack<T, 4>*>(Ch + row * C_LD + col) = four;
+        }
     }
     S* Cbase = reinterpret_cast<S*>(p.C) + (GROUP_K ? (int64_t)expert * p.c_stride_e : 0);
     typedef VPack<T, 8> P8;
