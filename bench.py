@@ -32,9 +32,9 @@ BF16_MFMA_PEAK_TFLOPS = 2500.0
 HBM_PEAK_GBS = 8000.0
 # HBM-side bytes per grouped-GEMM launch at the Mixtral shape, from two rocprofv3 --pmc runs of this file
 # (FETCH_SIZE, then WRITE_SIZE, each scaled by what the same counter reads for the 1 GiB copies of
-# --copy-calibration): 36.1 GB read + 5.4 GB written per step over 6 launches.  Summary:
+# --copy-calibration): 38.2 GB read + 5.6 GB written per step over 6 products.  Summary:
 # profiles/grouped_gemm_hbm_traffic_moe_mixtral_bf16.txt
-GEMM_HBM_BYTES_PER_LAUNCH = 6.93e9
+GEMM_HBM_BYTES_PER_LAUNCH = 7.29e9
 
 
 def parse_args():
