@@ -264,7 +264,16 @@ def bench_extras(device):
     ms = _time_rotating(lambda i: RN._backward(x=xs[i % sets], weight=w, eps=1e-5, rmsnorm_denominator=rstd,
                                                output_grad=dys[i % sets], kernel_backend=hip, BLOCK_SIZE_B=1, BLOCK_SIZE_H=H), sets)
     out["rmsnorm_bwd"] = gbs(3 * B * H * 2 + 2 * H * 2 + B * 4, ms)
-    del xs, dys
+    # residual addition + RMSNorm in one pass on the same shape: two rows read, two written
+    from cute_kernels.kernels.fused_residual_add_rmsnorm import fused_residual_add_rmsnorm_forward_hip
+
+    y, s_out = torch.empty_like(xs[0]), torch.empty_like(xs[0])
+    rstd_out = torch.empty(B, device=device, dtype=torch.float32)
+    ms = _time_rotating(lambda i: fused_residual_add_rmsnorm_forward_hip(
+        x=xs[i % sets], residual=dys[i % sets], weight=w, output=y, residual_output=s_out, eps=1e-5,
+        rmsnorm_denominator=rstd_out), sets)
+    out["residual_rmsnorm_fwd"] = gbs(4 * B * H * 2 + H * 2 + B * 4, ms)
+    del xs, dys, y, s_out
 
     # SwiGLU, BASELINE configs[2]: gate, up [16384, 14336]; 470 MB per tensor already exceeds the cache
     N = 16384 * 14336

@@ -74,6 +74,16 @@ int ck_swiglu_unchunked_backward(const void* x, const void* output_grad, void* x
  * ------------------------------------------------------------------------------------------- */
 int ck_rmsnorm_forward(const void* x, const void* weight, void* output, float* rstd, int64_t B, int64_t H,
                        float eps, int dtype, void* stream);
+
+/* Residual addition and RMSNorm in one pass (no counterpart in the reference, whose transformer blocks would run
+ * x + residual through add_tensor (kernels/add/add_tensor/__init__.py) and then rmsnorm (kernels/rmsnorm/__init__.py)):
+ *   residual_out = x + residual  (fp32 sum, rounded to the storage type),  output = rmsnorm(residual_out) as above.
+ * Same values as ck_add_tensor_forward followed by ck_rmsnorm_forward, with one read of the sum less.  All tensors
+ * are dense [B, H]; rstd as in ck_rmsnorm_forward.  The gradient of the pair is ck_rmsnorm_backward on residual_out
+ * plus whatever gradient reaches residual_out (ck_add_tensor_forward). */
+int ck_residual_rmsnorm_forward(const void* x, const void* residual, const void* weight, void* output,
+                                void* residual_out, float* rstd, int64_t B, int64_t H, float eps, int dtype,
+                                void* stream);
 int64_t ck_rmsnorm_backward_workspace_size(int64_t B, int64_t H);
 int ck_rmsnorm_backward(const void* x, const void* weight, const void* output_grad, const float* rstd,
                         void* x_grad, void* weight_grad, void* workspace, int64_t workspace_bytes,

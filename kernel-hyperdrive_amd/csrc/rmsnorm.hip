@@ -48,11 +48,14 @@ __device__ __forceinline__ void forget(P& p) {
 
 #define CK_RMS_BOUNDS(TPR) __launch_bounds__((TPR) > 256 ? (TPR) : 256, (TPR) > 256 ? 1 : 2)
 
-template <typename T, int TPR>
+// RES: the row that is normalised is x + res, rounded to the storage type and written to res_out as well (the
+// residual stream of a transformer block: one pass instead of an addition followed by a normalisation).
+template <typename T, int TPR, bool RES = false>
 __global__ void CK_RMS_BOUNDS(TPR)
     rmsnorm_fwd_kernel(const typename T::storage_t* __restrict__ x, const typename T::storage_t* __restrict__ w,
                        typename T::storage_t* __restrict__ y, float* __restrict__ rstd_out, int64_t B, int H,
-                       float eps) {
+                       float eps, const typename T::storage_t* __restrict__ res = nullptr,
+                       typename T::storage_t* __restrict__ res_out = nullptr) {
     typedef VPack<T, T::kVec> P;
     __shared__ float red[16];
     const int teams_per_block = blockDim.x / TPR;
@@ -65,23 +68,46 @@ __global__ void CK_RMS_BOUNDS(TPR)
     // rows are dealt round-robin; the next row is requested before the current one is reduced.
     // With TPR > 64 the block is one team, so the trip count is uniform across the barriers in team_sum.
     P cur[kMaxPacks], nxt[kMaxPacks];
+    P rcur[RES ? kMaxPacks : 1], rnxt[RES ? kMaxPacks : 1];
     int64_t row = team;
     if (row < B) {
         const P* xr = reinterpret_cast<const P*>(x + row * H);
+        const P* rr = RES ? reinterpret_cast<const P*>(res + row * H) : nullptr;
 #pragma unroll
         for (int i = 0; i < kMaxPacks; ++i) {
             const int p = t + i * TPR;
-            if (p < packs) cur[i] = nt_load(xr + p);
+            if (p < packs) {
+                cur[i] = nt_load(xr + p);
+                if (RES) rcur[i] = nt_load(rr + p);
+            }
         }
     }
     for (; row < B; row += num_teams) {
         const int64_t next_row = row + num_teams;
         if (next_row < B) {
             const P* xr = reinterpret_cast<const P*>(x + next_row * H);
+            const P* rr = RES ? reinterpret_cast<const P*>(res + next_row * H) : nullptr;
 #pragma unroll
             for (int i = 0; i < kMaxPacks; ++i) {
                 const int p = t + i * TPR;
-                if (p < packs) nxt[i] = nt_load(xr + p);
+                if (p < packs) {
+                    nxt[i] = nt_load(xr + p);
+                    if (RES) rnxt[i] = nt_load(rr + p);
+                }
+            }
+        }
+        if (RES) {
+            // the sum is rounded to the storage type first: that value is both the new residual and the row that
+            // is normalised, exactly as an addition kernel followed by the normalisation would have it
+            P* so = reinterpret_cast<P*>(res_out + row * H);
+#pragma unroll
+            for (int i = 0; i < kMaxPacks; ++i) {
+                const int p = t + i * TPR;
+                if (p < packs) {
+#pragma unroll
+                    for (int j = 0; j < T::kVec; ++j) cur[i].v[j] = T::down(T::up(cur[i].v[j]) + T::up(rcur[i].v[j]));
+                    nt_store(cur[i], so + p);
+                }
             }
         }
         float ss = 0.f;
@@ -118,7 +144,10 @@ __global__ void CK_RMS_BOUNDS(TPR)
             }
         }
 #pragma unroll
-        for (int i = 0; i < kMaxPacks; ++i) cur[i] = nxt[i];
+        for (int i = 0; i < kMaxPacks; ++i) {
+            cur[i] = nxt[i];
+            if (RES) rcur[i] = rnxt[i];
+        }
     }
 }
 
@@ -513,6 +542,42 @@ extern "C" int ck_rmsnorm_forward(const void* x, const void* weight, void* outpu
             const int64_t grid = B < 65536 ? B : 65536;
             hipLaunchKernelGGL((ck::rmsnorm_fwd_generic_kernel<T>), dim3((unsigned)grid), dim3(256), 0, s, (const S*)x,
                                (const S*)weight, (S*)output, rstd, B, (int)H, eps);
+        }
+    });
+    return ck_launch_status();
+}
+
+extern "C" int ck_residual_rmsnorm_forward(const void* x, const void* residual, const void* weight, void* output,
+                                           void* residual_out, float* rstd, int64_t B, int64_t H, float eps, int dtype,
+                                           void* stream) {
+    if (B < 0 || H < 0 || H > 65536) return CK_ERR_SHAPE;
+    if (B == 0 || H == 0) return CK_OK;
+    if (!x || !residual || !output || !residual_out) return CK_ERR_NULL;
+    if (!ck_aligned_elem(x, dtype) || !ck_aligned_elem(residual, dtype) || !ck_aligned_elem(output, dtype) ||
+        !ck_aligned_elem(residual_out, dtype) || (weight && !ck_aligned_elem(weight, dtype)))
+        return CK_ERR_ALIGN;
+    hipStream_t s = (hipStream_t)stream;
+    const bool aligned = ck_aligned16(x) && ck_aligned16(residual) && ck_aligned16(output) && ck_aligned16(residual_out) &&
+                         (!weight || ck_aligned16(weight));
+    const int tpr = aligned ? fast_tpr(H, dtype) : 0;
+    if (tpr != 64 && tpr != 256) {
+        // rows outside the register budget of the one-pass kernel (or unaligned): the sum, then the normalisation
+        const int st = ck_add_tensor_forward(x, residual, residual_out, B * H, dtype, 256, stream);
+        if (st != CK_OK) return st;
+        return ck_rmsnorm_forward(residual_out, weight, output, rstd, B, H, eps, dtype, stream);
+    }
+    CK_DISPATCH_DTYPE(dtype, {
+        typedef typename T::storage_t S;
+        if (tpr == 64) {
+            int64_t grid = (int64_t)cu_count() * 4;
+            if (grid > ck_ceil_div(B, 4)) grid = ck_ceil_div(B, 4);
+            hipLaunchKernelGGL((ck::rmsnorm_fwd_kernel<T, 64, true>), dim3((unsigned)grid), dim3(256), 0, s, (const S*)x,
+                               (const S*)weight, (S*)output, rstd, B, (int)H, eps, (const S*)residual, (S*)residual_out);
+        } else {
+            int64_t grid = (int64_t)cu_count() * 4;
+            if (grid > B) grid = B;
+            hipLaunchKernelGGL((ck::rmsnorm_fwd_kernel<T, 256, true>), dim3((unsigned)grid), dim3(256), 0, s, (const S*)x,
+                               (const S*)weight, (S*)output, rstd, B, (int)H, eps, (const S*)residual, (S*)residual_out);
         }
     });
     return ck_launch_status();

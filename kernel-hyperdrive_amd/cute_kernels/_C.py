@@ -43,6 +43,7 @@ _SIGNATURES = {
     "ck_swiglu_unchunked_forward": (_i32, [_p, _p, _i64, _i64, _i32, _i32, _p]),
     "ck_swiglu_unchunked_backward": (_i32, [_p, _p, _p, _i64, _i64, _i32, _i32, _p]),
     "ck_rmsnorm_forward": (_i32, [_p, _p, _p, _p, _i64, _i64, _f32, _i32, _p]),
+    "ck_residual_rmsnorm_forward": (_i32, [_p, _p, _p, _p, _p, _p, _i64, _i64, _f32, _i32, _p]),
     "ck_rmsnorm_backward_workspace_size": (_i64, [_i64, _i64]),
     "ck_rmsnorm_backward": (_i32, [_p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _f32, _i32, _p]),
     "ck_embedding_forward": (_i32, [_p, _i32, _p, _p, _i64, _i64, _i64, _i32, _p]),
@@ -282,6 +283,24 @@ def rmsnorm_forward(x, weight, output, rstd, eps: float) -> None:
             lib.ck_rmsnorm_forward(_ptr(x), _ptr(weight), _ptr(output), _ptr(rstd), B, H, eps, dtype_code(x.dtype),
                                    L.stream),
             "ck_rmsnorm_forward",
+        )
+
+
+def residual_rmsnorm_forward(x, residual, weight, output, residual_out, rstd, eps: float) -> None:
+    """residual_out = x + residual, output = rmsnorm(residual_out); all dense and of one shape and dtype."""
+    lib = load_library()
+    H = x.size(-1)
+    B = x.numel() // H if H > 0 else 0
+    for t in (residual, output, residual_out):
+        if t.shape != x.shape or t.dtype != x.dtype or not t.is_contiguous():
+            raise ValueError("residual_rmsnorm_forward: x, residual, output and residual_out must be dense and alike")
+    if not x.is_contiguous():
+        raise ValueError("residual_rmsnorm_forward: x must be dense")
+    with _Launch(x, residual, weight, output, residual_out, rstd) as L:
+        _check(
+            lib.ck_residual_rmsnorm_forward(_ptr(x), _ptr(residual), _ptr(weight), _ptr(output), _ptr(residual_out),
+                                            _ptr(rstd), B, H, eps, dtype_code(x.dtype), L.stream),
+            "ck_residual_rmsnorm_forward",
         )
 
 

@@ -23,6 +23,8 @@ from .kernels import (
     contiguous_count_cute,
     embedding_cute,
     embedding_torch,
+    fused_residual_add_rmsnorm_cute,
+    fused_residual_add_rmsnorm_torch,
     rmsnorm_cute,
     rmsnorm_torch,
     scattered_experts,

@@ -14,6 +14,8 @@ stock torch ops on random inputs):
                       ``up * F.silu(gate)`` in fp64 and the limits g -> +-inf, g = 0
   rmsnorm_*           closed form cute_kernels/kernels/rmsnorm/README.md:3-25; checked against autograd of
                       ``F.rms_norm`` in fp64, scale invariance and the dx.x identity
+  residual_rmsnorm_*  add_tensor followed by rmsnorm_* (no operator of its own in the reference); checked against autograd
+                      of ``F.rms_norm(x + residual)`` with the sum used twice, in fp64
   embedding_*         one_hot(ids)^T @ dy (cute_kernels/kernels/embedding/README.md:7-15); checked against a
                       dense one-hot matmul and ``F.embedding`` autograd in fp64
   contiguous_count    numpy.bincount(minlength) (tests/kernels/contiguous_count_test.py:35)
@@ -136,6 +138,24 @@ def rmsnorm_forward(x, weight, eps, compute_dtype=torch.float32):
     if weight is not None:
         y = y * weight.to(compute_dtype)
     return y.to(x.dtype), rstd.squeeze(-1)
+
+
+def residual_rmsnorm_forward(x, residual, weight, eps, compute_dtype=torch.float32):
+    """(rmsnorm(s), s) with s = x + residual rounded to the storage type first: ``add_tensor`` followed by
+    ``rmsnorm_forward``, the two reference operators a pre-norm block runs on its residual stream."""
+    s = add_tensor(x, residual)
+    return rmsnorm_forward(s, weight, eps, compute_dtype)[0], s
+
+
+def residual_rmsnorm_backward(x, residual, weight, output_grad, sum_grad, eps, compute_dtype=torch.float32):
+    """Gradients of ``residual_rmsnorm_forward`` for loss = <y, output_grad> + <s, sum_grad>: the normalisation's
+    input gradient, rounded, plus ``sum_grad``, rounded again (as two separate operators hand it on); the same for
+    both terms of the sum.  Returns (d_x = d_residual, d_weight)."""
+    s = add_tensor(x, residual)
+    dx, dw = rmsnorm_backward(s, weight, output_grad, eps, compute_dtype)
+    if sum_grad is not None:
+        dx = (dx.to(compute_dtype) + sum_grad.to(compute_dtype)).to(x.dtype)  # add_tensor at compute_dtype = fp32
+    return dx, dw
 
 
 def rmsnorm_backward(x, weight, output_grad, eps, compute_dtype=torch.float32):

@@ -62,6 +62,17 @@ def test_rmsnorm_argument_checks(lib):
     assert lib.ck_rmsnorm_backward(P, P, P + 2, None, P, P, P, need, 4, 64, 1e-5, F32, None) == ALIGN
 
 
+def test_residual_rmsnorm_argument_checks(lib):
+    f = lib.ck_residual_rmsnorm_forward
+    #        x  res w     y  res_out rstd  B  H   eps   dtype stream
+    assert f(P, P, None, P, P, None, 4, 65537, 1e-5, BF16, None) == SHAPE
+    assert f(P, None, None, P, P, None, 4, 64, 1e-5, BF16, None) == NULL
+    assert f(P, P, None, P, None, None, 4, 64, 1e-5, BF16, None) == NULL
+    assert f(P, P, None, P, P, None, 4, 64, 1e-5, 9, None) == DTYPE
+    assert f(P, P + 1, None, P, P, None, 4, 64, 1e-5, BF16, None) == ALIGN
+    assert f(P, P, None, P, P, None, 0, 64, 1e-5, BF16, None) == OK  # no rows
+
+
 def test_embedding_argument_checks(lib):
     assert lib.ck_embedding_forward(P, 0, P, P, -1, 10, 8, BF16, None) == SHAPE
     assert lib.ck_embedding_forward(None, 0, P, P, 4, 10, 8, BF16, None) == NULL

@@ -189,6 +189,57 @@ def test_rmsnorm_config2_shape_slice_and_eps_default(gpu):
     torch.testing.assert_close(rstd.cpu(), O.rmsnorm_forward(x, None, 1e-5)[1], rtol=1e-5, atol=1e-6)
 
 
+# ---- residual addition + rmsnorm in one pass --------------------------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("has_weight", [True, False])
+@pytest.mark.parametrize("memory_efficient", [False, True])
+@pytest.mark.parametrize("size", [(37, 4096), (5, 72), (3, 70), (2, 40000), (300, 8192), (4096,), (6, 7, 512)])
+def test_fused_residual_add_rmsnorm(gpu, dtype, has_weight, memory_efficient, size):
+    """Outputs and gradients equal, bit for bit, add_tensor_cute followed by rmsnorm_cute (the two reference
+    operators the fused one stands for); both are held to the oracle as well."""
+    from cute_kernels import add_tensor_cute, fused_residual_add_rmsnorm_cute, rmsnorm_cute
+
+    announce("residual + rmsnorm", dtype, has_weight, memory_efficient, size)
+    H = size[-1]
+    x, r = randn(size, dtype, 14), randn(size, dtype, 15)
+    w = randn((H,), dtype, 16, 0.1, 1.0) if has_weight else None
+    dy, ds = randn(size, dtype, 17), randn(size, dtype, 18)
+    eps = 1e-5
+
+    def leaves():
+        return (x.to(gpu).requires_grad_(True), r.to(gpu).requires_grad_(True),
+                w.to(gpu).requires_grad_(True) if has_weight else None)
+
+    xf, rf, wf = leaves()
+    y, s = fused_residual_add_rmsnorm_cute(xf, rf, wf, eps, memory_efficient=memory_efficient)
+    torch.autograd.backward([y, s], [dy.to(gpu), ds.to(gpu)])
+    xs, rs, ws = leaves()
+    s_ref = add_tensor_cute(xs, rs)
+    y_ref = rmsnorm_cute(s_ref, ws, eps, memory_efficient=memory_efficient)
+    torch.autograd.backward([y_ref, s_ref], [dy.to(gpu), ds.to(gpu)])
+    assert y.shape == x.shape and s.shape == x.shape
+    assert torch.equal(y, y_ref) and torch.equal(s, s_ref)
+    assert torch.equal(xf.grad, xs.grad) and torch.equal(rf.grad, rs.grad) and torch.equal(xf.grad, rf.grad)
+    if has_weight:
+        assert torch.equal(wf.grad, ws.grad)
+
+    x2, r2, dy2, ds2 = (t.reshape(-1, H) for t in (x, r, dy, ds))
+    y_o, s_o = O.residual_rmsnorm_forward(x2, r2, w, eps)
+    assert torch.equal(s.cpu().reshape(-1, H), s_o), "the sum: one fp32 addition, one rounding"
+    assert_close(y.reshape(-1, H), y_o, dtype, "y")
+    dx_o, dw_o = O.residual_rmsnorm_backward(x2, r2, w, dy2, ds2, eps)
+    assert_close(xf.grad.reshape(-1, H), dx_o, dtype, "x_grad")
+    if has_weight:
+        assert_close(wf.grad, dw_o, dtype, "weight_grad")
+
+    # only the normalised output used: no addition in the backward, the gradient is the normalisation's
+    xf, rf, wf = leaves()
+    y, _ = fused_residual_add_rmsnorm_cute(xf, rf, wf, eps, memory_efficient=memory_efficient)
+    y.backward(dy.to(gpu))
+    dx_o, _ = O.residual_rmsnorm_backward(x2, r2, w, dy2, None, eps)
+    assert_close(xf.grad.reshape(-1, H), dx_o, dtype, "x_grad without a gradient on the sum")
+
+
 # ---- embedding ----------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize(

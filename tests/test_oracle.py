@@ -354,6 +354,28 @@ def test_router_topk_softmax_against_topk_brute_force_and_closed_form():
     assert torch.allclose(d_logits.sum(-1), torch.zeros(37, dtype=F64), atol=1e-15)  # softmax gradients sum to zero
 
 
+def test_residual_rmsnorm_against_autograd_of_the_composition():
+    g = torch.Generator().manual_seed(12)
+    B, H, eps = 9, 24, 1e-5
+    # (x and r on the bf16 grid: their sum is then exact in the fp32 addition the oracle's add_tensor performs)
+    x, r = (torch.randn(B, H, generator=g).bfloat16().double() for _ in range(2))
+    dy, ds = (torch.randn(B, H, generator=g, dtype=F64) for _ in range(2))
+    w = torch.randn(H, generator=g, dtype=F64)
+    leaves = [t.clone().requires_grad_(True) for t in (x, r, w)]
+    s = leaves[0] + leaves[1]
+    y = F.rms_norm(s, (H,), weight=leaves[2], eps=eps)
+    ((y * dy).sum() + (s * ds).sum()).backward()
+    y_o, s_o = O.residual_rmsnorm_forward(x, r, w, eps, compute_dtype=F64)
+    assert torch.allclose(y_o, y.detach(), rtol=1e-12, atol=1e-13) and torch.equal(s_o, s.detach())
+    dx, dw = O.residual_rmsnorm_backward(x, r, w, dy, ds, eps, compute_dtype=F64)
+    assert torch.allclose(dx, leaves[0].grad, rtol=1e-11, atol=1e-12)
+    assert torch.allclose(dx, leaves[1].grad, rtol=1e-11, atol=1e-12)
+    assert torch.allclose(dw, leaves[2].grad, rtol=1e-11, atol=1e-12)
+    # without a gradient on the sum the pair reduces to the plain normalisation of x + r
+    dx0, _ = O.residual_rmsnorm_backward(x, r, None, dy, None, eps, compute_dtype=F64)
+    assert torch.allclose(dx0, O.rmsnorm_backward(x + r, None, dy, eps, compute_dtype=F64)[0], rtol=0, atol=0)
+
+
 def test_moe_single_expert_is_a_plain_mlp():
     T, H, I = 7, 8, 5
     x, wg, wfc, wproj, dy = (t.double() for t in O.moe_inputs(T, H, I, 1, torch.float32, seed=4))
