@@ -107,6 +107,67 @@ def test_scatter2scatter_split_tail(gpu, dtype, w_layout, mode, shape):
     assert_close(out, whole, dtype, "split against whole")
 
 
+def _random_gemm_cases(n, seed):
+    g = torch.Generator().manual_seed(seed)
+
+    def pick(lo, hi):
+        return int(torch.randint(lo, hi + 1, (1,), generator=g))
+
+    cases = []
+    for i in range(n):
+        E = pick(1, 12)
+        k = pick(1, min(3, E))
+        T = pick(40, 1500)
+        K = 8 * pick(8, 160) if i % 4 else 64 * pick(64, 160)  # every fourth case is long enough to be split
+        N = 8 * pick(4, 130)
+        empty = tuple(sorted(set(pick(0, E - 1) for _ in range(pick(0, 2))))) if E - k >= 3 else ()
+        cases.append((T, k, E, K, N, empty, pick(0, 2), pick(0, 1), i % 2))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_gemm_cases(32, 1234), ids=lambda c: "-".join(map(str, c[:5])))
+def test_grouped_products_on_random_shapes(gpu, case):
+    """scatter2scatter and group_bwd_W on shapes drawn at random (ragged experts, contraction tails, one to many
+    tiles, with and without the split tail), against fp32 products of stock torch on the device per expert."""
+    from cute_kernels.kernels.scattermoe import group_bwd_W, scatter2scatter
+
+    T, k, E, K, N, empty, mode, w_kc, use_f16 = case
+    dtype = torch.float16 if use_f16 else torch.bfloat16
+    announce("random grouped products", dtype, case)
+    s_e, s_idx, off = routing(T, k, E, 95, empty)
+    x_grouped, y_grouped = mode != 0, mode != 1
+    fan_out = 1 if x_grouped else k
+    M = T * k
+    X = randn((M if x_grouped else T, K), dtype, 96, 0.5).to(gpu)
+    W = (randn((E, N, K), dtype, 97, 0.05).to(gpu).permute(0, 2, 1) if w_kc else randn((E, K, N), dtype, 97, 0.05).to(gpu))
+    out = torch.full((M, N), float("nan"), dtype=dtype, device=gpu)
+    s_idx_g, off_g = s_idx.to(gpu), off.to(gpu)
+    scatter2scatter(X, W, s_e.to(gpu), s_idx_g, out, fan_out, x_grouped, y_grouped, off_g)
+
+    rows_in = X if x_grouped else X[s_idx_g // k]          # expert-grouped input rows
+    expected = torch.empty(M, N, dtype=torch.float32, device=gpu)
+    bounds = [0] + off.tolist()
+    for e in range(E):
+        a, b = bounds[e], bounds[e + 1]
+        if b > a:
+            expected[a:b] = rows_in[a:b].float() @ W[e].float()
+    if not y_grouped:
+        scattered = torch.empty_like(expected)
+        scattered[s_idx_g] = expected
+        expected = scattered
+    assert_close(out, expected.to(dtype), dtype, "scatter2scatter")
+
+    # weight gradient of the same rows: DW[e] = X_e^T DY_e
+    DY = randn((M, N), dtype, 98, 0.5).to(gpu)
+    Xg = rows_in.contiguous()
+    DW = torch.full((E, K, N), float("nan"), dtype=dtype, device=gpu)
+    group_bwd_W(DY, Xg, off_g, DW, E)
+    for e in range(E):
+        a, b = bounds[e], bounds[e + 1]
+        ref = (Xg[a:b].float().T @ DY[a:b].float()).to(dtype) if b > a else torch.zeros(K, N, dtype=dtype, device=gpu)
+        assert_close_long_sums(DW[e], ref, dtype, f"group_bwd_W expert {e}")
+
+
 # ---- grouped products with the SwiGLU in the epilogue ----------------------------------------------------
 GLU_SHAPES = [
     # T, k, E, K (hidden), I, empty experts
