@@ -1091,60 +1091,71 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
     // GLU == 1: a lane takes an "up" packet together with its "gate" packet, so packets are counted over half a row
     constexpr int C_CHUNKS_PER_ROW = (GLU == 1 ? BN / 2 : BN) / 8;
     constexpr int C_CH = BM * C_CHUNKS_PER_ROW / THREADS;
-    // GLU == 2: the up / gate packets of h that this lane's packets need are requested here, all of them at once and
-    // without branches (positions outside the tile are redirected to a valid one), while the accumulator registers
-    // are free and the workgroup is on its way to the barrier; inside the store loop each packet would wait for its
-    // own two loads in turn.
+    // The loads an output packet depends on are all requested before anything is stored, and without branches
+    // (positions outside the tile are redirected to a valid one): the destination rows of scattered outputs, the
+    // up / gate packets of h for GLU == 2 - both while the workgroup is on its way to the barrier - and, behind the
+    // barrier, the staged packets themselves.  Packet by packet, every store would wait for its own loads in turn
+    // (and, with one counter for loads and stores, for the store before it).
     constexpr int H_CH = GLU == 2 ? C_CH : 1;
     P8 h_up[H_CH], h_gate[H_CH];
+    int64_t out_row[C_CH];
+#pragma unroll
+    for (int i = 0; i < C_CH; ++i) {
+        const int row = min((tid + i * THREADS) / C_CHUNKS_PER_ROW, rows_valid - 1);
+        out_row[i] = GROUP_K ? i_base + row : row_start + row;
+    }
+    if (!GROUP_K && !p.y_grouped) {
+#pragma unroll
+        for (int i = 0; i < C_CH; ++i) out_row[i] = p.row_idx[out_row[i]];
+    }
     if (GLU == 2) {
 #pragma unroll
         for (int i = 0; i < C_CH; ++i) {
-            const int c = tid + i * THREADS;
-            const int row = min(c / C_CHUNKS_PER_ROW, rows_valid - 1);
-            const int col = min((c % C_CHUNKS_PER_ROW) * 8, cols_valid - 8);
-            const int64_t slot = row_start + row;
-            const int64_t out_row = p.y_grouped ? slot : p.row_idx[slot];
-            const S* hrow = reinterpret_cast<const S*>(p.aux) + out_row * p.ld_aux + n_base + col;
+            const int col = min(((tid + i * THREADS) % C_CHUNKS_PER_ROW) * 8, cols_valid - 8);
+            const S* hrow = reinterpret_cast<const S*>(p.aux) + out_row[i] * p.ld_aux + n_base + col;
             h_up[i] = nt_load(reinterpret_cast<const P8*>(hrow));
             h_gate[i] = nt_load(reinterpret_cast<const P8*>(hrow + p.glu_half));
         }
     }
     __syncthreads();
+    constexpr int G_CH = GLU == 1 ? C_CH : 1;
+    P8 staged[C_CH], staged_gate[G_CH];
+#pragma unroll
+    for (int i = 0; i < C_CH; ++i) {
+        const int c = tid + i * THREADS;
+        const int row = c / C_CHUNKS_PER_ROW;
+        const int col = (c % C_CHUNKS_PER_ROW) * 8;
+        const S* src = reinterpret_cast<const S*>(row < BM / 2 ? lds0 : lds1) + (row % (BM / 2)) * C_LD + col;
+        staged[i] = *reinterpret_cast<const P8*>(src);
+        // GLU == 1: columns [0, BN / 2) of the tile are "up", [BN / 2, BN) the matching "gate"
+        if (GLU == 1) staged_gate[i] = *reinterpret_cast<const P8*>(src + BN / 2);
+    }
 #pragma unroll
     for (int i = 0; i < C_CH; ++i) {
         const int c = tid + i * THREADS;
         const int row = c / C_CHUNKS_PER_ROW;
         const int col = (c % C_CHUNKS_PER_ROW) * 8;
         if (row < rows_valid && col < cols_valid) {
-            int64_t out_row;
-            if (GROUP_K) {
-                out_row = i_base + row;
-            } else {
-                const int64_t slot = row_start + row;
-                out_row = p.y_grouped ? slot : p.row_idx[slot];
-            }
-            const S* src = reinterpret_cast<const S*>(row < BM / 2 ? lds0 : lds1) + (row % (BM / 2)) * C_LD + col;
             if (GLU == 0) {
-                *reinterpret_cast<u32x4_t*>(Cbase + out_row * p.ldc + n_base + col) = *reinterpret_cast<const u32x4_t*>(src);
+                *reinterpret_cast<P8*>(Cbase + out_row[i] * p.ldc + n_base + col) = staged[i];
             } else if (GLU == 1) {
-                // columns [0, BN / 2) of the tile are "up", [BN / 2, BN) the matching "gate": both go to h, and the
-                // activation is computed from the rounded values exactly as the separate kernel would from h
-                const P8 u = *reinterpret_cast<const P8*>(src);
-                const P8 g = *reinterpret_cast<const P8*>(src + BN / 2);
+                // both halves go to h, and the activation is computed from the rounded values exactly as the
+                // separate kernel would from h
+                const P8 u = staged[i];
+                const P8 g = staged_gate[GLU == 1 ? i : 0];
                 P8 y;
 #pragma unroll
                 for (int e = 0; e < 8; ++e) y.v[e] = T::down(swiglu_fwd_1<T>(T::up(g.v[e]), T::up(u.v[e])));
-                S* hrow = Cbase + out_row * p.ldc + n_base + col;
+                S* hrow = Cbase + out_row[i] * p.ldc + n_base + col;
                 *reinterpret_cast<P8*>(hrow) = u;
                 *reinterpret_cast<P8*>(hrow + p.glu_half) = g;
-                *reinterpret_cast<P8*>(reinterpret_cast<S*>(p.aux) + out_row * p.ld_aux + n_base + col) = y;
+                *reinterpret_cast<P8*>(reinterpret_cast<S*>(p.aux) + out_row[i] * p.ld_aux + n_base + col) = y;
             } else {
                 // the staged tile is d_act (rounded, as the separate kernels would hand it over); h supplies up
                 // and gate of the same positions, and d_h receives both derivatives
                 const P8 u = h_up[GLU == 2 ? i : 0];
                 const P8 g = h_gate[GLU == 2 ? i : 0];
-                const P8 d = *reinterpret_cast<const P8*>(src);
+                const P8 d = staged[i];
                 P8 du, dg;
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
@@ -1153,7 +1164,7 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
                     dg.v[e] = T::down(fg);
                     du.v[e] = T::down(fu);
                 }
-                S* drow = Cbase + out_row * p.ldc + n_base + col;
+                S* drow = Cbase + out_row[i] * p.ldc + n_base + col;
                 *reinterpret_cast<P8*>(drow) = du;
                 *reinterpret_cast<P8*>(drow + p.glu_half) = dg;
             }
