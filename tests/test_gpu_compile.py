@@ -77,6 +77,36 @@ def test_compiled_additions(gpu, dtype):
     assert torch.equal(xs.grad.cpu(), dz)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_compiled_residual_rmsnorm_and_router(gpu, dtype):
+    from cute_kernels import fused_residual_add_rmsnorm_cute
+    from cute_kernels.kernels.scattermoe import router_topk_softmax
+
+    announce("compiled residual rmsnorm / router", dtype)
+    x, r, dy, ds = (randn((33, 520), dtype, 24 + i) for i in range(4))
+    w = randn((520,), dtype, 28, 0.1, 1.0)
+    xg, rg, wg = x.to(gpu).requires_grad_(True), r.to(gpu).requires_grad_(True), w.to(gpu).requires_grad_(True)
+    y, s = torch.compile(fused_residual_add_rmsnorm_cute, fullgraph=True)(xg, rg, wg, 1e-5)
+    torch.autograd.backward([y, s], [dy.to(gpu), ds.to(gpu)])
+    y_o, s_o = O.residual_rmsnorm_forward(x, r, w, 1e-5)
+    dx_o, dw_o = O.residual_rmsnorm_backward(x, r, w, dy, ds, 1e-5)
+    assert torch.equal(s.detach().cpu(), s_o)
+    assert_close(y, y_o, dtype, "y")
+    assert_close(xg.grad, dx_o, dtype, "x_grad")
+    assert torch.equal(xg.grad, rg.grad)
+    assert_close(wg.grad, dw_o, dtype, "weight_grad")
+
+    logits = randn((200, 16), dtype, 29)
+    lg = logits.to(gpu).requires_grad_(True)
+    weights, selected = torch.compile(router_topk_softmax, fullgraph=True)(lg, 4)
+    dw_ = randn((200, 4), dtype, 30)
+    weights.backward(dw_.to(gpu))
+    exp_w, exp_sel = O.router_topk_softmax(logits, 4)
+    assert torch.equal(selected.cpu(), exp_sel)
+    assert_close(weights, exp_w, dtype, "routing weights")
+    assert_close(lg.grad, O.router_topk_softmax_backward(dw_, logits, exp_sel), dtype, "d_logits")
+
+
 def test_compiled_contiguous_count(gpu):
     from cute_kernels import contiguous_count_cute
 
