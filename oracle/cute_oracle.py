@@ -5,7 +5,9 @@ that the HIP kernels can be checked against it.  Only tests, ``__graft_entry__.s
 ``cpu_baseline`` leg of ``bench.py`` may import it; nothing in the shipped package does.
 
 How each function is pinned (the reference holds no golden vectors for this path; its tests compare against
-stock torch ops on random inputs):
+stock torch ops on random inputs; the known-answer fixtures of tests/golden, written by code that shares nothing
+with this module, pin swiglu, rmsnorm, residual_rmsnorm, embedding, moe_sort, router_topk_softmax and the MoE layer
+with and without biases as well):
   add_tensor, add_scalar
                       ``x + y`` (cute_kernels/kernels/add/add_*/torch_implementation.py:4-5): the sum formed in fp32
                       and rounded once; checked against numpy float32 addition with a hand-written

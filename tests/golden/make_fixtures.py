@@ -11,6 +11,11 @@ with ``oracle/cute_oracle.py`` or the HIP kernels:
   rmsnorm.npz     y = x / sqrt(mean(x^2) + eps) * w and the closed-form dx, dw (rmsnorm/README.md:3-25), numpy
   embedding.npz   gather and dW = one_hot(ids)^T dy as explicit loops over tokens, duplicates included
   moe_sort.npz    hand-written stable counting sort of a small id list, offsets by counting
+  router.npz      per token: the k largest logits by an explicit sort (ties to the lower position), softmax over them
+                  and its closed-form gradient, element by element (torch_implementation.py:121-132, 193-199)
+  residual_rmsnorm.npz   s = x + r, then the rmsnorm formulas above on s; dx with a gradient arriving on s as well
+  moe_bias.npz    the loop of moe.npz with a bias added after each of the two matrix-vector products
+                  (Experts_Torch with add_bias=True, torch_implementation.py:18-20, 40)
   moe.npz         the MoE layer as a loop over tokens: every token's top-k experts evaluated as two dense
                   matrix-vector products with SwiGLU in between, mixed with softmax weights
                   (scattermoe/torch_implementation.py:101-199 of the reference, read per token); gradients by
@@ -124,6 +129,81 @@ def make_moe(rng):
              dw_proj=w_proj.grad.numpy())
 
 
+def make_router(rng):
+    T, E, k = 10, 6, 3
+    logits = dyadic(rng, (T, E), 1.0)
+    logits[0, :] = 1.5  # all equal: positions 0, 1, 2 win
+    logits[1, 4] = logits[1, 1]  # a tie that may straddle the cut
+    d_weights = dyadic(rng, (T, k), 1.0)
+    selected = np.zeros((T, k), dtype=np.int64)
+    weights = np.zeros((T, k))
+    d_logits = np.zeros((T, E))
+    for t in range(T):
+        order = sorted(range(E), key=lambda e: (-logits[t, e], e))[:k]
+        vals = [logits[t, e] for e in order]
+        ex = [np.exp(v - vals[0]) for v in vals]
+        w = [v / sum(ex) for v in ex]
+        dot = sum(d_weights[t, j] * w[j] for j in range(k))
+        for j, e in enumerate(order):
+            selected[t, j] = e
+            weights[t, j] = w[j]
+            d_logits[t, e] = w[j] * (d_weights[t, j] - dot)
+    np.savez(os.path.join(HERE, "router.npz"), logits=logits, top_k=np.int64(k), d_weights=d_weights, selected=selected,
+             weights=weights, d_logits=d_logits)
+
+
+def make_residual_rmsnorm(rng):
+    B, H, eps = 6, 48, 1e-5
+    x = dyadic(rng, (B, H), 1.0)
+    r = dyadic(rng, (B, H), 1.0)  # x + r = k / 16 with |k| <= 96: still exact in bfloat16
+    w = 1.0 + dyadic(rng, (H,), 1.0 / 8.0)
+    dy = dyadic(rng, (B, H), 0.5)
+    ds = dyadic(rng, (B, H), 0.5)
+    s = x + r
+    y = np.empty_like(s)
+    dx = np.empty_like(s)
+    dw = np.zeros(H)
+    for b in range(B):
+        rs = 1.0 / np.sqrt(float(np.dot(s[b], s[b])) / H + eps)
+        y[b] = s[b] * rs * w
+        g = dy[b] * w
+        dx[b] = rs * g - s[b] * (rs ** 3) * float(np.dot(g, s[b])) / H + ds[b]
+        dw += dy[b] * s[b] * rs
+    np.savez(os.path.join(HERE, "residual_rmsnorm.npz"), x=x, r=r, w=w, dy=dy, ds=ds, eps=np.float64(eps), s=s, y=y, dx=dx, dw=dw)
+
+
+def make_moe_bias(rng):
+    T, H, I, E, k = 10, 16, 24, 4, 2
+    leaf = lambda a: torch.tensor(a, requires_grad=True)
+    x = leaf(dyadic(rng, (T, H), 0.5))
+    w_gate = leaf(dyadic(rng, (E, H), 1.0 / 8.0))
+    w_fc = leaf(dyadic(rng, (E, 2 * I, H), 1.0 / 8.0))
+    w_proj = leaf(dyadic(rng, (E, H, I), 1.0 / 8.0))
+    b_fc = leaf(dyadic(rng, (E, 2 * I), 0.5))
+    b_proj = leaf(dyadic(rng, (E, H), 0.5))
+    dy = torch.tensor(dyadic(rng, (T, H), 1.0))
+    rows, selected = [], []
+    for t in range(T):
+        logits = w_gate @ x[t]
+        assert len(set(float(v) for v in logits.detach())) == E, "router tie in the fixture: change the seed"
+        order = sorted(range(E), key=lambda e: (-float(logits[e].detach()), e))[:k]
+        weights = torch.softmax(torch.stack([logits[e] for e in order]), dim=0)
+        acc = torch.zeros(H, dtype=torch.float64)
+        for j, e in enumerate(order):
+            h = w_fc[e] @ x[t] + b_fc[e]
+            up, gate = h[:I], h[I:]
+            acc = acc + weights[j] * (w_proj[e] @ (up * gate * torch.sigmoid(gate)) + b_proj[e])
+        rows.append(acc)
+        selected.append(order)
+    y = torch.stack(rows)
+    (y * dy).sum().backward()
+    np.savez(os.path.join(HERE, "moe_bias.npz"), x=x.detach().numpy(), w_gate=w_gate.detach().numpy(),
+             w_fc=w_fc.detach().numpy(), w_proj=w_proj.detach().numpy(), b_fc=b_fc.detach().numpy(),
+             b_proj=b_proj.detach().numpy(), dy=dy.numpy(), top_k=np.int64(k), selected=np.array(selected, dtype=np.int64),
+             y=y.detach().numpy(), dx=x.grad.numpy(), dw_gate=w_gate.grad.numpy(), dw_fc=w_fc.grad.numpy(),
+             dw_proj=w_proj.grad.numpy(), db_fc=b_fc.grad.numpy(), db_proj=b_proj.grad.numpy())
+
+
 def main():
     rng = np.random.default_rng(20240607)
     make_swiglu(rng)
@@ -131,6 +211,10 @@ def main():
     make_embedding(rng)
     make_moe_sort()
     make_moe(rng)
+    rng2 = np.random.default_rng(20240608)  # the later fixtures draw from their own stream: the files above stay as they are
+    make_router(rng2)
+    make_residual_rmsnorm(rng2)
+    make_moe_bias(rng2)
     for name in sorted(os.listdir(HERE)):
         if name.endswith(".npz"):
             print(name, os.path.getsize(os.path.join(HERE, name)), "bytes")

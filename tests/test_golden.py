@@ -24,7 +24,9 @@ def load(name):
 
 def test_fixture_inputs_are_exact_in_bfloat16():
     for name, keys in (("swiglu", ["gate", "up", "dy"]), ("rmsnorm", ["x", "w", "dy"]), ("embedding", ["table", "dy"]),
-                       ("moe", ["x", "w_gate", "w_fc", "w_proj", "dy"])):
+                       ("moe", ["x", "w_gate", "w_fc", "w_proj", "dy"]), ("router", ["logits", "d_weights"]),
+                       ("residual_rmsnorm", ["x", "r", "s", "w", "dy", "ds"]),
+                       ("moe_bias", ["x", "w_gate", "w_fc", "w_proj", "b_fc", "b_proj", "dy"])):
         f = load(name)
         for k in keys:
             assert torch.equal(f[k].to(torch.bfloat16).double(), f[k]), (name, k)
@@ -84,6 +86,99 @@ def test_oracle_moe_golden():
 
 
 # ---- GPU: the HIP path against the fixtures ---------------------------------------------------------------
+def test_oracle_router_golden():
+    f = load("router")
+    k = int(f["top_k"])
+    weights, selected = O.router_topk_softmax(f["logits"], k, torch.float64)
+    assert torch.equal(selected, f["selected"])
+    torch.testing.assert_close(weights, f["weights"], rtol=1e-13, atol=1e-14)
+    d_logits = O.router_topk_softmax_backward(f["d_weights"], f["logits"], selected, torch.float64)
+    torch.testing.assert_close(d_logits, f["d_logits"], rtol=1e-12, atol=1e-13)
+
+
+def test_oracle_residual_rmsnorm_golden():
+    f = load("residual_rmsnorm")
+    eps = float(f["eps"])
+    y, s = O.residual_rmsnorm_forward(f["x"], f["r"], f["w"], eps, torch.float64)
+    assert torch.equal(s, f["s"])
+    torch.testing.assert_close(y, f["y"], rtol=1e-12, atol=1e-12)
+    dx, dw = O.residual_rmsnorm_backward(f["x"], f["r"], f["w"], f["dy"], f["ds"], eps, torch.float64)
+    torch.testing.assert_close(dx, f["dx"], rtol=1e-11, atol=1e-11)
+    torch.testing.assert_close(dw, f["dw"], rtol=1e-11, atol=1e-11)
+
+
+def test_oracle_moe_bias_golden():
+    f = load("moe_bias")
+    res = O.moe_forward_backward(f["x"], f["w_gate"], f["w_fc"], f["w_proj"], f["dy"], int(f["top_k"]),
+                                 compute_dtype=torch.float64, b_fc=f["b_fc"], b_proj=f["b_proj"])
+    for key in ("y", "dx", "dw_gate", "dw_fc", "dw_proj", "db_fc", "db_proj"):
+        torch.testing.assert_close(res[key], f[key], rtol=1e-9, atol=1e-10, msg=lambda m, key=key: f"{key}: {m}")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_hip_router_golden(gpu, dtype):
+    from cute_kernels.kernels.scattermoe import router_topk_softmax
+
+    announce("golden router", dtype)
+    f = load("router")
+    logits = f["logits"].to(dtype).to(gpu).requires_grad_(True)
+    weights, selected = router_topk_softmax(logits, int(f["top_k"]))
+    weights.backward(f["d_weights"].to(dtype).to(gpu))
+    assert torch.equal(selected.cpu(), f["selected"]), "largest first, equal logits in the order of their positions"
+    assert_close(weights.detach(), f["weights"].to(dtype), dtype, "weights")
+    assert_close(logits.grad, f["d_logits"].to(dtype), dtype, "d_logits")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_hip_residual_rmsnorm_golden(gpu, dtype):
+    from cute_kernels import fused_residual_add_rmsnorm_cute
+
+    announce("golden residual rmsnorm", dtype)
+    f = load("residual_rmsnorm")
+    x, r, w = (f[key].to(dtype).to(gpu).requires_grad_(True) for key in ("x", "r", "w"))
+    y, s = fused_residual_add_rmsnorm_cute(x, r, w, float(f["eps"]))
+    torch.autograd.backward([y, s], [f["dy"].to(dtype).to(gpu), f["ds"].to(dtype).to(gpu)])
+    assert torch.equal(s.detach().cpu().double(), f["s"]), "the sum is exact in every storage type"
+    assert_close(y.detach(), f["y"].to(dtype), dtype, "y")
+    assert_close(x.grad, f["dx"].to(dtype), dtype, "dx")
+    assert torch.equal(x.grad, r.grad)
+    assert_close(w.grad, f["dw"].to(dtype), dtype, "dw")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_hip_moe_bias_golden(gpu, dtype):
+    from cute_kernels import MoE_Triton, swiglu_unchunked_cute
+
+    announce("golden moe with biases", dtype)
+    f = load("moe_bias")
+    T, H = f["x"].shape
+    E, I = f["w_proj"].shape[0], f["w_proj"].shape[2]
+    k = int(f["top_k"])
+    moe = MoE_Triton(num_experts=E, num_experts_per_tok=k, hidden_size=H, intermediate_size=I,
+                     activation_function=swiglu_unchunked_cute, is_glu=True, add_bias=True, std=0.02)
+    moe = moe.to(device=gpu, dtype=dtype)
+    with torch.no_grad():
+        for param, key in ((moe.gate.weight, "w_gate"), (moe.c_fc.weight, "w_fc"), (moe.c_proj.weight, "w_proj"),
+                           (moe.c_fc.bias, "b_fc"), (moe.c_proj.bias, "b_proj")):
+            param.copy_(f[key])
+    x = f["x"].to(dtype).to(gpu).requires_grad_(True)
+    y, _ = moe(x)
+    (y * f["dy"].to(dtype).to(gpu)).sum().backward()
+    with torch.no_grad():
+        _, _, selected = moe._compute_routing_weights(x)
+    assert torch.equal(selected.cpu(), f["selected"]), "routing"
+    got = {"y": y.detach(), "dx": x.grad, "dw_fc": moe.c_fc.weight.grad, "dw_proj": moe.c_proj.weight.grad,
+           "db_fc": moe.c_fc.bias.grad, "db_proj": moe.c_proj.bias.grad, "dw_gate": moe.gate.weight.grad}
+    for key, value in got.items():
+        # values reach a few tens and every intermediate is rounded to the storage type: norm-wise at its rounding
+        # level (fp32: the router gradient is made by stock torch ops from the routing weights' gradient)
+        limit = (1e-4 if key == "dw_gate" else 1e-5) if dtype == torch.float32 else 2e-2
+        assert_norm_close(value, f[key], limit, key)
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_hip_swiglu_golden(gpu, dtype):
