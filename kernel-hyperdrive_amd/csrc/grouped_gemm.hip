@@ -1009,9 +1009,15 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
     if (MODE != 2 && n_full >= 2) {
 #pragma unroll
         for (int part = 0; part < 4; ++part) issue_part(lds0, part, 0);
-#pragma unroll
-        for (int part = 0; part < 4; ++part) issue_part(lds1, part, 1);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        // Tile 1 is requested in the order in which the first two steps read it (B lower, A lower, B upper, A
+        // upper), so the waits of the loop (twelve copies outstanding, two more per M phase) cover each half in
+        // time, and only tile 0 has to be complete before the loop starts: the 128 copy instructions of the two
+        // tiles take the request path about 2 us, half of which now runs beside the first step.
+        issue_part(lds1, 2, 1);
+        issue_part(lds1, 0, 1);
+        issue_part(lds1, 3, 1);
+        issue_part(lds1, 1, 1);
+        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
         __syncthreads();
         read_b(lds0, 0, fb0);
         __builtin_amdgcn_s_waitcnt(0xC07F);
