@@ -954,7 +954,9 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
     // so every copy has seven M phases until its half is read again, and a wait that leaves the twelve most recent
     // copies of the wave outstanding (two per M phase) at the end of each M phase covers it: what the next M phase
     // of either group reads was requested at least six M phases before this one, and the barrier that ends the
-    // phase passes that on to the other waves.
+    // phase passes that on to the other waves.  The count only works because nothing but these copies is
+    // outstanding on the vector-memory counter inside the loop: the copies complete in the order they were
+    // issued, but an ordinary load issued among them can complete ahead of older copies (tried: wrong results).
 #define CK_PHASE_END()                           \
     do {                                         \
         __builtin_amdgcn_sched_barrier(0);       \
