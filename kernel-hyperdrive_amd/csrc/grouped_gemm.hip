@@ -136,6 +136,77 @@ __device__ __forceinline__ bool logical_tile(int m_tiles, int n_tiles, int& mt, 
     return true;
 }
 
+// Row tiles of all experts, and the expert that owns row tile mt.  Both are run by one wavefront.  With at most 64
+// experts lane e keeps the bounds and the running tile count of expert e from the first function, and the second
+// needs no further pass over the offsets (one round trip to memory per tile search instead of two).
+struct ExpertTiles {
+    int begin, end, tiles, incl;
+};
+
+template <int BM>
+__device__ __forceinline__ int count_row_tiles(const int64_t* __restrict__ offsets, int E, int lane, ExpertTiles& mine) {
+    if (E <= CK_WAVE) {
+        mine.begin = 0;
+        mine.end = 0;
+        if (lane < E) {
+            mine.end = (int)offsets[lane];
+            mine.begin = lane == 0 ? 0 : (int)offsets[lane - 1];
+        }
+        mine.tiles = (mine.end - mine.begin + BM - 1) / BM;
+        mine.incl = wave_inclusive_scan_i(mine.tiles);
+        return __shfl(mine.incl, CK_WAVE - 1, CK_WAVE);
+    }
+    int m_tiles = 0;
+    for (int e0 = 0; e0 < E; e0 += CK_WAVE) {
+        const int e = e0 + lane;
+        int tiles = 0;
+        if (e < E) tiles = ((int)offsets[e] - (e == 0 ? 0 : (int)offsets[e - 1]) + BM - 1) / BM;
+        m_tiles += wave_sum_i(tiles);
+    }
+    return m_tiles;
+}
+
+template <int BM>
+__device__ __forceinline__ void expert_of_row_tile(const int64_t* __restrict__ offsets, int E, int lane, int mt,
+                                                   const ExpertTiles& mine, int& found_e, int& found_start,
+                                                   int& found_rows) {
+    if (E <= CK_WAVE) {
+        const uint64_t hit = __ballot(lane < E && mine.incl > mt);
+        if (hit != 0) {
+            const int src = __ffsll((unsigned long long)hit) - 1;
+            const int excl = __shfl(mine.incl - mine.tiles, src, CK_WAVE);
+            const int b = __shfl(mine.begin, src, CK_WAVE);
+            const int en = __shfl(mine.end, src, CK_WAVE);
+            found_e = src;
+            found_start = b + (mt - excl) * BM;
+            found_rows = min(BM, en - found_start);
+        }
+        return;
+    }
+    int base_tiles = 0;
+    for (int e0 = 0; e0 < E && found_e < 0; e0 += CK_WAVE) {
+        const int e = e0 + lane;
+        int begin = 0, end = 0;
+        if (e < E) {
+            end = (int)offsets[e];
+            begin = e == 0 ? 0 : (int)offsets[e - 1];
+        }
+        const int tiles = (end - begin + BM - 1) / BM;
+        const int incl = wave_inclusive_scan_i(tiles) + base_tiles;
+        const uint64_t hit = __ballot(e < E && incl > mt);
+        if (hit != 0) {
+            const int src = __ffsll((unsigned long long)hit) - 1;
+            const int excl = __shfl(incl - tiles, src, CK_WAVE);
+            const int b = __shfl(begin, src, CK_WAVE);
+            const int en = __shfl(end, src, CK_WAVE);
+            found_e = e0 + src;
+            found_start = b + (mt - excl) * BM;
+            found_rows = min(BM, en - found_start);
+        }
+        base_tiles = __shfl(incl, CK_WAVE - 1, CK_WAVE);
+    }
+}
+
 // Tile of workgroup blockIdx.x for the products whose rows are cut per expert (forward and input gradient): the
 // XCD-aware order above, applied to the number of row tiles the experts really have.  The host can only bound
 // that number (rows / BM + E); dealing out the bound would leave the XCD that owns the end of the range with
@@ -146,14 +217,8 @@ __device__ __forceinline__ void find_tile_balanced(const int64_t* __restrict__ o
     if (threadIdx.x < CK_WAVE) {
         constexpr int XCDS = 8, GROUP_M = 8;
         const int lane = lane_id();
-        // row tiles of all experts
-        int m_tiles = 0;
-        for (int e0 = 0; e0 < E; e0 += CK_WAVE) {
-            const int e = e0 + lane;
-            int tiles = 0;
-            if (e < E) tiles = ((int)offsets[e] - (e == 0 ? 0 : (int)offsets[e - 1]) + BM - 1) / BM;
-            m_tiles += wave_sum_i(tiles);
-        }
+        ExpertTiles mine;
+        const int m_tiles = count_row_tiles<BM>(offsets, E, lane, mine);
         int found_e = -1, found_start = 0, found_rows = 0, nt = 0;
         const int total = m_tiles * n_tiles;
         // an even share of the tiles where rows of the tile grid are long; whole rows of it where they are short
@@ -170,28 +235,7 @@ __device__ __forceinline__ void find_tile_balanced(const int64_t* __restrict__ o
             const int in_group = L - group * group_span;
             const int mt = first_m + in_group % gm;
             nt = in_group / gm;
-            int base_tiles = 0;
-            for (int e0 = 0; e0 < E && found_e < 0; e0 += CK_WAVE) {
-                const int e = e0 + lane;
-                int begin = 0, end = 0;
-                if (e < E) {
-                    end = (int)offsets[e];
-                    begin = e == 0 ? 0 : (int)offsets[e - 1];
-                }
-                const int tiles = (end - begin + BM - 1) / BM;
-                const int incl = wave_inclusive_scan_i(tiles) + base_tiles;
-                const uint64_t hit = __ballot(e < E && incl > mt);
-                if (hit != 0) {
-                    const int src = __ffsll((unsigned long long)hit) - 1;
-                    const int excl = __shfl(incl - tiles, src, CK_WAVE);
-                    const int b = __shfl(begin, src, CK_WAVE);
-                    const int en = __shfl(end, src, CK_WAVE);
-                    found_e = e0 + src;
-                    found_start = b + (mt - excl) * BM;
-                    found_rows = min(BM, en - found_start);
-                }
-                base_tiles = __shfl(incl, CK_WAVE - 1, CK_WAVE);
-            }
+            expert_of_row_tile<BM>(offsets, E, lane, mt, mine, found_e, found_start, found_rows);
         }
         if (lane == 0) {
             sh_info[0] = found_e;
@@ -221,13 +265,8 @@ __device__ __forceinline__ void find_tile_split(const int64_t* __restrict__ offs
     if (threadIdx.x < CK_WAVE) {
         constexpr int XCDS = 8, GROUP_M = 8, CUS = 32;
         const int lane = lane_id();
-        int m_tiles = 0;
-        for (int e0 = 0; e0 < E; e0 += CK_WAVE) {
-            const int e = e0 + lane;
-            int tiles = 0;
-            if (e < E) tiles = ((int)offsets[e] - (e == 0 ? 0 : (int)offsets[e - 1]) + BM - 1) / BM;
-            m_tiles += wave_sum_i(tiles);
-        }
+        ExpertTiles et;
+        const int m_tiles = count_row_tiles<BM>(offsets, E, lane, et);
         const int total = m_tiles * n_tiles;
         const int per_xcd = (total + XCDS - 1) / XCDS;
         const int xcd = blockIdx.x % XCDS, pos = blockIdx.x / XCDS;
@@ -266,28 +305,7 @@ __device__ __forceinline__ void find_tile_split(const int64_t* __restrict__ offs
             const int in_group = L - group * group_span;
             const int mt = first_m + in_group % gm;
             nt = in_group / gm;
-            int base_tiles = 0;
-            for (int e0 = 0; e0 < E && found_e < 0; e0 += CK_WAVE) {
-                const int e = e0 + lane;
-                int begin = 0, end = 0;
-                if (e < E) {
-                    end = (int)offsets[e];
-                    begin = e == 0 ? 0 : (int)offsets[e - 1];
-                }
-                const int tiles = (end - begin + BM - 1) / BM;
-                const int incl = wave_inclusive_scan_i(tiles) + base_tiles;
-                const uint64_t hit = __ballot(e < E && incl > mt);
-                if (hit != 0) {
-                    const int src = __ffsll((unsigned long long)hit) - 1;
-                    const int excl = __shfl(incl - tiles, src, CK_WAVE);
-                    const int b = __shfl(begin, src, CK_WAVE);
-                    const int en = __shfl(end, src, CK_WAVE);
-                    found_e = e0 + src;
-                    found_start = b + (mt - excl) * BM;
-                    found_rows = min(BM, en - found_start);
-                }
-                base_tiles = __shfl(incl, CK_WAVE - 1, CK_WAVE);
-            }
+            expert_of_row_tile<BM>(offsets, E, lane, mt, et, found_e, found_start, found_rows);
         }
         if (lane == 0) {
             sh_info[0] = found_e;
