@@ -256,6 +256,22 @@ int ck_router_topk_softmax_backward(const void* d_weights, const float* weights_
                                     int dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * Router forward in one launch: the router's linear followed by the selection above
+ * replaces `self.gate(hidden_states)` (a bias-free linear, scattermoe/torch_implementation.py:122) together
+ * with the topk / softmax sequence of :123-132.
+ *   logits [tokens, E] = x [tokens, H] * gate_weight [E, H]^T, fp32 accumulation, rounded once to the storage
+ *   type and written (row stride logits_stride); selected / weights / weights_f32 as
+ *   ck_router_topk_softmax_forward gives them for these stored logits.
+ * bf16 and fp16 only (CK_ERR_DTYPE otherwise: the caller uses its linear and ck_router_topk_softmax_forward);
+ * H a multiple of 8, x and gate_weight 16-byte aligned with row strides that are multiples of 8 elements and
+ * unit column stride; E <= 128, k <= min(E, 64).  The backward is ck_router_topk_softmax_backward followed by the
+ * caller's two products with d_logits.
+ * ------------------------------------------------------------------------------------------- */
+int ck_router_forward(const void* x, int64_t x_stride, const void* gate_weight, int64_t gate_weight_stride,
+                      void* logits, int64_t logits_stride, void* weights, float* weights_f32, int64_t* selected,
+                      int64_t tokens, int64_t H, int64_t E, int64_t k, int dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
  * Per-expert bias of the grouped linears
  * replaces the bias term of F.linear(rows_e, W[e], bias[e]) in scattermoe/torch_implementation.py:35-43 (the
  * reference's Triton experts, triton_implementation/__init__.py:24-34, do not read their bias parameter).

@@ -8,6 +8,11 @@
 //                               rounded once to the storage type; the fp32 values are kept for the backward
 //   backward: d_v[t, j]       = w_j * (g_j - sum_i g_i w_i)     (softmax backward on the fp32 weights)
 //             d_logits[t, e]  = d_v[t, j] where e = selected[t, j], else 0  (every element of the row is written)
+// The forward also exists with the router's linear in front (logits = x W^T, torch_implementation.py:122): a
+// workgroup multiplies 16 tokens by all experts' rows with MFMAs, its four waves splitting the hidden dimension,
+// adds the four partial blocks up through LDS, rounds the logits once to the storage type, writes them, and selects
+// from the rounded values - as the stock sequence does, which selects from the stored logits.  x is read once; a
+// library GEMM with so few output columns reads it at a fraction of the memory bandwidth.
 #include <math.h>
 
 #include "ck_device.h"
@@ -22,20 +27,11 @@ __device__ __forceinline__ bool router_ahead(float a, int ai, float b, int bi) {
     return gt || (eq && ai < bi);
 }
 
+// Selection and softmax for one token by one wavefront: lane l holds the logits of experts l, l + 64, ... in v.
 template <typename T, int VPL>
-__global__ void __launch_bounds__(256)
-    router_fwd_kernel(const typename T::storage_t* __restrict__ logits, int64_t ld,
-                      typename T::storage_t* __restrict__ weights, float* __restrict__ weights_f32,
-                      int64_t* __restrict__ selected, int64_t tokens, int E, int k) {
-    const int64_t t = (int64_t)blockIdx.x * 4 + threadIdx.x / CK_WAVE;
-    if (t >= tokens) return;
-    const int lane = lane_id();
-    float v[VPL];
-#pragma unroll
-    for (int i = 0; i < VPL; ++i) {
-        const int e = i * CK_WAVE + lane;
-        v[i] = e < E ? T::up(logits[t * ld + e]) : 0.f;
-    }
+__device__ __forceinline__ void router_select_token(const float (&v)[VPL], int lane, int E, int k, int64_t t,
+                                                    typename T::storage_t* __restrict__ weights,
+                                                    float* __restrict__ weights_f32, int64_t* __restrict__ selected) {
     uint32_t taken = 0;  // bit i: v[i] is already among the selected
     float my_val = 0.f;  // lane j < k ends up with the j-th largest value and its position
     int my_idx = 0;
@@ -77,6 +73,123 @@ __global__ void __launch_bounds__(256)
 
 template <typename T, int VPL>
 __global__ void __launch_bounds__(256)
+    router_fwd_kernel(const typename T::storage_t* __restrict__ logits, int64_t ld,
+                      typename T::storage_t* __restrict__ weights, float* __restrict__ weights_f32,
+                      int64_t* __restrict__ selected, int64_t tokens, int E, int k) {
+    const int64_t t = (int64_t)blockIdx.x * 4 + threadIdx.x / CK_WAVE;
+    if (t >= tokens) return;
+    const int lane = lane_id();
+    float v[VPL];
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+        const int e = i * CK_WAVE + lane;
+        v[i] = e < E ? T::up(logits[t * ld + e]) : 0.f;
+    }
+    router_select_token<T, VPL>(v, lane, E, k, t, weights, weights_f32, selected);
+}
+
+// ---- the router's linear and the selection in one launch ---------------------------------------------------
+template <typename T>
+struct RouterMma;
+template <>
+struct RouterMma<BF16> {
+    typedef bf16x8_t frag_t;
+    static __device__ __forceinline__ f32x4_t mma(frag_t a, frag_t b, f32x4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    }
+};
+template <>
+struct RouterMma<F16> {
+    typedef f16x8_t frag_t;
+    static __device__ __forceinline__ f32x4_t mma(frag_t a, frag_t b, f32x4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    }
+};
+
+constexpr int kRouterTokens = 16;  // tokens per workgroup: one MFMA row tile
+
+// NT column tiles of 16 experts.  Operand fragments come straight from memory: lane l of a 16 x 16 x 32 MFMA supplies
+// the 8 consecutive hidden positions 8 * (l / 16) ... of row l % 16 of either operand - one 16-byte load each, and
+// the weight rows stay in L2.  Wave w takes the blocks of 32 hidden positions w, w + 4, ...; U of them are in flight.
+// The result lane l holds of tile nt is (token 4 * (l / 16) + r, expert 16 nt + l % 16), r = 0 .. 3.
+template <typename T, int NT>
+__global__ void __launch_bounds__(256)
+    router_linear_fwd_kernel(const typename T::storage_t* __restrict__ x, int64_t ldx,
+                             const typename T::storage_t* __restrict__ w, int64_t ldw,
+                             typename T::storage_t* __restrict__ logits, int64_t ld_logits,
+                             typename T::storage_t* __restrict__ weights, float* __restrict__ weights_f32,
+                             int64_t* __restrict__ selected, int64_t tokens, int H, int E, int k) {
+    typedef typename T::storage_t S;
+    typedef typename RouterMma<T>::frag_t frag_t;
+    constexpr int EP = NT * 16, VPL = (EP + CK_WAVE - 1) / CK_WAVE, U = NT <= 2 ? 4 : 2;
+    __shared__ float part[4][kRouterTokens][EP + 1];
+    const int wave = threadIdx.x / CK_WAVE, lane = lane_id();
+    const int row = lane % 16, kc = lane / 16;
+    const int64_t t0 = (int64_t)blockIdx.x * kRouterTokens;
+    const S* xrow = x + min(t0 + row, tokens - 1) * ldx + kc * 8;
+    const S* wrow[NT];
+    bool live[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const int n = nt * 16 + row;
+        live[nt] = n < E;
+        wrow[nt] = w + (int64_t)(live[nt] ? n : 0) * ldw + kc * 8;
+    }
+    f32x4_t acc[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) acc[nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    const frag_t zero = {};
+    const int k_last = H - 8 - kc * 8;  // (relative to the lane's first packet) the last packet of the row
+    for (int kb = wave; kb * 32 < H; kb += 4 * U) {
+        // All loads of a turn are issued before any is used, and none sits behind a branch: a packet past the end of
+        // the row (H is a multiple of 8, so it lies wholly inside or outside) or in a row past the last expert is
+        // read from a valid place instead and replaced by zeros afterwards.
+        frag_t a[U], b[U][NT];
+        bool in[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int k0 = (kb + 4 * u) * 32;
+            in[u] = k0 <= k_last;
+            const int kl = in[u] ? k0 : 0;
+            a[u] = nt_load(reinterpret_cast<const frag_t*>(xrow + kl));
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) b[u][nt] = *reinterpret_cast<const frag_t*>(wrow[nt] + kl);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            a[u] = in[u] ? a[u] : zero;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) acc[nt] = RouterMma<T>::mma(a[u], live[nt] ? b[u][nt] : zero, acc[nt]);
+        }
+    }
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) part[wave][4 * kc + r][nt * 16 + row] = acc[nt][r];
+    __syncthreads();
+    // wave w finishes tokens 4 w .. 4 w + 3: lane l holds experts l, l + 64
+    for (int i = 0; i < 4; ++i) {
+        const int tt = wave * 4 + i;
+        const int64_t t = t0 + tt;
+        if (t >= tokens) break;
+        float v[VPL];
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+            const int e = j * CK_WAVE + lane;
+            v[j] = 0.f;
+            if (e < E) {
+                const S rounded = T::down(((part[0][tt][e] + part[1][tt][e]) + part[2][tt][e]) + part[3][tt][e]);
+                logits[t * ld_logits + e] = rounded;
+                v[j] = T::up(rounded);
+            }
+        }
+        router_select_token<T, VPL>(v, lane, E, k, t, weights, weights_f32, selected);
+    }
+}
+
+
+template <typename T, int VPL>
+__global__ void __launch_bounds__(256)
     router_bwd_kernel(const typename T::storage_t* __restrict__ d_weights, const float* __restrict__ weights_f32,
                       const int64_t* __restrict__ selected, typename T::storage_t* __restrict__ d_logits, int64_t ld,
                       int64_t tokens, int E, int k) {
@@ -109,6 +222,7 @@ __global__ void __launch_bounds__(256)
 
 namespace {
 constexpr int64_t kMaxRouterExperts = 1024;  // 16 values per lane
+constexpr int64_t kMaxLinearExperts = 128;   // 8 MFMA column tiles
 }
 
 #define CK_ROUTER_LAUNCH(KERNEL, ...)                                                                              \
@@ -142,6 +256,48 @@ extern "C" int ck_router_topk_softmax_forward(const void* logits, int64_t logits
         CK_ROUTER_LAUNCH(router_fwd_kernel, (const S*)logits, logits_stride, (S*)weights, weights_f32, selected, tokens,
                          (int)E, (int)k);
     });
+    return ck_launch_status();
+}
+
+extern "C" int ck_router_forward(const void* x, int64_t x_stride, const void* gate_weight, int64_t gate_weight_stride,
+                                 void* logits, int64_t logits_stride, void* weights, float* weights_f32,
+                                 int64_t* selected, int64_t tokens, int64_t H, int64_t E, int64_t k, int dtype,
+                                 void* stream) {
+    if (dtype != CK_BF16 && dtype != CK_F16) return CK_ERR_DTYPE;
+    if (tokens < 0 || H <= 0 || H > 0x7fffffff - 1024 || (H & 7) || E <= 0 || E > kMaxLinearExperts || k <= 0 || k > E ||
+        k > CK_WAVE || x_stride < H || gate_weight_stride < H || (x_stride & 7) || (gate_weight_stride & 7) ||
+        logits_stride < E)
+        return CK_ERR_SHAPE;
+    if (tokens == 0) return CK_OK;
+    if (!x || !gate_weight || !logits || !weights || !weights_f32 || !selected) return CK_ERR_NULL;
+    if (!ck_aligned16(x) || !ck_aligned16(gate_weight) || !ck_aligned_elem(logits, dtype) || !ck_aligned_elem(weights, dtype))
+        return CK_ERR_ALIGN;
+    const int64_t grid = ck_ceil_div(tokens, ck::kRouterTokens);
+    if (grid > 0x7fffffff) return CK_ERR_SHAPE;
+    hipStream_t s = (hipStream_t)stream;
+    const int nt = (int)ck_ceil_div(E, 16);
+#define CK_ROUTER_LINEAR(TT, NT)                                                                                    \
+    hipLaunchKernelGGL((ck::router_linear_fwd_kernel<TT, NT>), dim3((unsigned)grid), dim3(256), 0, s,               \
+                       (const TT::storage_t*)x, x_stride, (const TT::storage_t*)gate_weight, gate_weight_stride,  \
+                       (TT::storage_t*)logits, logits_stride, (TT::storage_t*)weights, weights_f32, selected, tokens, \
+                       (int)H, (int)E, (int)k)
+#define CK_ROUTER_LINEAR_NT(TT)            \
+    do {                                   \
+        if (nt <= 1)                       \
+            CK_ROUTER_LINEAR(TT, 1);       \
+        else if (nt <= 2)                  \
+            CK_ROUTER_LINEAR(TT, 2);       \
+        else if (nt <= 4)                  \
+            CK_ROUTER_LINEAR(TT, 4);       \
+        else                               \
+            CK_ROUTER_LINEAR(TT, 8);       \
+    } while (0)
+    if (dtype == CK_BF16)
+        CK_ROUTER_LINEAR_NT(ck::BF16);
+    else
+        CK_ROUTER_LINEAR_NT(ck::F16);
+#undef CK_ROUTER_LINEAR_NT
+#undef CK_ROUTER_LINEAR
     return ck_launch_status();
 }
 

@@ -79,6 +79,7 @@ _SIGNATURES = {
     "ck_expert_bias_backward": (_i32, [_p, _i64, _p, _p, _i64, _i64, _i64, _i64, _i32, _p]),
     "ck_router_topk_softmax_forward": (_i32, [_p, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, _p]),
     "ck_router_topk_softmax_backward": (_i32, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i32, _p]),
+    "ck_router_forward": (_i32, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _i32, _p]),
     "ck_probe_mfma": (_i32, [_p, _i64, _i32, _p, _p]),
 }
 
@@ -537,6 +538,7 @@ def expert_bias_backward(dy, expert_offsets, d_bias) -> None:
 
 ROUTER_MAX_EXPERTS = 1024
 ROUTER_MAX_TOP_K = 64
+ROUTER_LINEAR_MAX_EXPERTS = 128  # the launch with the router's linear in front
 
 
 def router_topk_softmax_forward(logits, weights, weights_f32, selected) -> None:
@@ -556,6 +558,49 @@ def router_topk_softmax_forward(logits, weights, weights_f32, selected) -> None:
             lib.ck_router_topk_softmax_forward(_ptr(logits), logits.stride(0), _ptr(weights), _ptr(weights_f32),
                                                _ptr(selected), T, E, k, dtype_code(logits.dtype), L.stream),
             "ck_router_topk_softmax_forward",
+        )
+
+
+def router_forward_supported(x, gate_weight, top_k: int) -> bool:
+    """Whether ``router_forward`` takes operands of this type, shape and strides (otherwise: the linear, then
+    router_topk_softmax_forward).  Only properties a traced graph knows; the 16-byte alignment of the first elements
+    is the caller's to provide."""
+    return (
+        x.dim() == 2
+        and gate_weight.dim() == 2
+        and x.dtype in (torch.bfloat16, torch.float16)
+        and gate_weight.dtype == x.dtype
+        and gate_weight.size(0) <= ROUTER_LINEAR_MAX_EXPERTS
+        and top_k <= min(gate_weight.size(0), ROUTER_MAX_TOP_K)
+        and x.size(1) % 8 == 0
+        and x.stride(1) == 1 and gate_weight.stride(1) == 1
+        and x.stride(0) % 8 == 0 and gate_weight.stride(0) % 8 == 0
+    )
+
+
+def router_forward(x, gate_weight, logits, weights, weights_f32, selected) -> None:
+    """logits [T, E] = x [T, H] @ gate_weight [E, H]^T (rounded once), and the selection from the stored logits."""
+    lib = load_library()
+    T, H = x.shape
+    E = gate_weight.size(0)
+    k = selected.size(1)
+    if gate_weight.size(1) != H or gate_weight.dtype != x.dtype:
+        raise ValueError("router_forward: gate_weight must be [E, H] in x's dtype")
+    if x.stride(1) != 1 or gate_weight.stride(1) != 1:
+        raise ValueError("router_forward needs unit column stride for x and gate_weight")
+    if tuple(logits.shape) != (T, E) or logits.dtype != x.dtype or logits.stride(1) != 1:
+        raise ValueError("router_forward: logits must be [tokens, E] in x's dtype with unit column stride")
+    if weights.dtype != x.dtype or weights_f32.dtype != torch.float32 or selected.dtype != torch.int64:
+        raise ValueError("router_forward: weights in x's dtype, weights_f32 fp32, selected int64")
+    for out in (weights, weights_f32, selected):
+        if tuple(out.shape) != (T, k) or not out.is_contiguous():
+            raise ValueError("router_forward: weights, weights_f32 and selected must be dense [tokens, k]")
+    with _Launch(x, gate_weight, logits, weights, weights_f32, selected) as L:
+        _check(
+            lib.ck_router_forward(_ptr(x), x.stride(0), _ptr(gate_weight), gate_weight.stride(0), _ptr(logits),
+                                  logits.stride(0), _ptr(weights), _ptr(weights_f32), _ptr(selected), T, H, E, k,
+                                  dtype_code(x.dtype), L.stream),
+            "ck_router_forward",
         )
 
 

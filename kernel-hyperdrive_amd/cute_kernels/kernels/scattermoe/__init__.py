@@ -1,4 +1,4 @@
-from .moe_hip import Experts_HIP, Experts_Triton, MoE_HIP, MoE_Triton, moe_sort, router_topk_softmax
+from .moe_hip import Experts_HIP, Experts_Triton, MoE_HIP, MoE_Triton, moe_router, moe_sort, router_topk_softmax
 from .moe_torch import Experts_Torch, MoE_Torch
 from .ops import (
     group,

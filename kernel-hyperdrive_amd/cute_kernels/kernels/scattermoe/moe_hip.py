@@ -110,6 +110,85 @@ def router_topk_softmax(router_logits: torch.Tensor, top_k: int) -> tuple[torch.
     return _RouterTopKSoftmax.apply(router_logits, top_k)
 
 
+def _router_linear_forward_fake(x: torch.Tensor, gate_weight: torch.Tensor, top_k: int):
+    T, E = x.size(0), gate_weight.size(0)
+    return (
+        torch.empty(T, E, dtype=x.dtype, device=x.device),
+        torch.empty(T, top_k, dtype=x.dtype, device=x.device),
+        torch.empty(T, top_k, dtype=torch.float32, device=x.device),
+        torch.empty(T, top_k, dtype=torch.int64, device=x.device),
+    )
+
+
+@cute_op(f"{LIBRARY_NAME}::router_forward_hip", mutates_args={}, fake_func=_router_linear_forward_fake)
+def router_forward_hip(
+    x: torch.Tensor, gate_weight: torch.Tensor, top_k: int
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    T, E = x.size(0), gate_weight.size(0)
+    logits = torch.empty(T, E, dtype=x.dtype, device=x.device)
+    weights = torch.empty(T, top_k, dtype=x.dtype, device=x.device)
+    weights_f32 = torch.empty(T, top_k, dtype=torch.float32, device=x.device)
+    selected = torch.empty(T, top_k, dtype=torch.int64, device=x.device)
+    # rows are read as 16-byte packets: a view that starts in the middle of one is copied to a fresh allocation
+    if x.data_ptr() % 16 != 0:
+        x = x.clone()
+    if gate_weight.data_ptr() % 16 != 0:
+        gate_weight = gate_weight.clone()
+    _C.router_forward(x, gate_weight, logits, weights, weights_f32, selected)
+    return logits, weights, weights_f32, selected
+
+
+class _Router(torch.autograd.Function):
+    """Router linear, top-k and softmax as one forward launch.  Backward: the selection's backward launch gives
+    d_logits, the caller's own gradient of the logits (an auxiliary loss) is added, and the two products with
+    d_logits are library GEMMs as they are for ``F.linear``."""
+
+    @staticmethod
+    def forward(ctx, x, gate_weight, top_k):
+        logits, weights, weights_f32, selected = router_forward_hip(x, gate_weight, top_k)
+        ctx.save_for_backward(x, gate_weight, weights_f32, selected)
+        ctx.mark_non_differentiable(selected)
+        ctx.set_materialize_grads(False)
+        return logits, weights, selected
+
+    @staticmethod
+    def backward(ctx, d_logits, d_weights, _d_selected):
+        x, gate_weight, weights_f32, selected = ctx.saved_tensors
+        total = None
+        if d_weights is not None:
+            total = router_topk_softmax_backward_hip(d_weights, weights_f32, selected, gate_weight.size(0))
+        if d_logits is not None:
+            total = d_logits if total is None else total + d_logits
+        if total is None:
+            return None, None, None
+        d_x = total @ gate_weight if ctx.needs_input_grad[0] else None
+        d_gate_weight = total.t() @ x if ctx.needs_input_grad[1] else None
+        return d_x, d_gate_weight, None
+
+
+# Up to this many experts the launch with the linear in front is the faster one (8 experts, 8192 x 4096 tokens:
+# 25 us against 22 + 15 for the library GEMM and the selection; 64 experts, 16384 x 2048: 61 against 23 + 21 - a wave
+# of that launch selects for four tokens one after the other, and a selection is a chain of dependent shuffles).
+_FUSED_ROUTER_MAX_EXPERTS = 16
+
+
+def moe_router(
+    x: torch.Tensor, gate_weight: torch.Tensor, top_k: int, fused: bool | None = None
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``(router_logits [T, E], router_weights [T, k], selected_experts [T, k])`` from the tokens ``x [T, H]`` and the
+    router's weight ``[E, H]``: ``MoE_Torch._compute_routing_weights`` (torch_implementation.py:120-133) with a
+    bias-free gate.  One launch where ``_C.router_forward_supported`` holds (16-bit, E <= 128, H % 8 == 0, aligned
+    rows) and ``fused`` asks for it (``None``: where it is the faster way), else the linear followed by
+    ``router_topk_softmax``."""
+    if fused is None:
+        fused = gate_weight.size(0) <= _FUSED_ROUTER_MAX_EXPERTS
+    if fused and _C.router_forward_supported(x, gate_weight, top_k):
+        return _Router.apply(x, gate_weight, top_k)
+    router_logits = torch.nn.functional.linear(x, gate_weight)
+    router_weights, selected_experts = router_topk_softmax(router_logits, top_k)
+    return router_logits, router_weights, selected_experts
+
+
 class Experts_HIP(Experts_Torch):
     """The grouped linears on the HIP kernels.  ``add_bias=True`` applies the ``[E, out]`` bias as the plain-torch
     experts do (torch_implementation.py:35-43); the reference's ``Experts_Triton`` holds the same parameter and
@@ -146,8 +225,13 @@ class MoE_HIP(MoE_Torch):
     # GEMMs' epilogues (same values, two passes over the intermediate activations fewer).  False keeps the three
     # separate autograd nodes of the reference layer.
     fuse_swiglu = True
-    # Top-k, softmax and their backward as one launch each instead of the stock torch ops (False: inherited routing).
+    # The router's linear, top-k and softmax as one forward launch, the selection's backward as one launch, instead
+    # of the stock torch ops (False: inherited routing).
     fuse_router = True
+    # ... with the router's linear in the same forward launch.  Its logits are the fp32 sums rounded once, as a library
+    # GEMM's are, but summed in another order: a few differ in the last bit, which can turn a near-tie the other way.
+    # False keeps ``self.gate`` as a module call.
+    fuse_router_linear = True
 
     def _compute_routing_weights(self, hidden_states: torch.Tensor):
         if not (
@@ -156,6 +240,8 @@ class MoE_HIP(MoE_Torch):
             and self.top_k <= min(self.num_experts, _C.ROUTER_MAX_TOP_K)
         ):
             return super()._compute_routing_weights(hidden_states)
+        if self.fuse_router_linear and getattr(self.gate, "bias", None) is None:
+            return moe_router(hidden_states, self.gate.weight, self.top_k)
         router_logits = self.gate(hidden_states)  # [T, E]
         router_weights, selected_experts = router_topk_softmax(router_logits, self.top_k)
         return router_logits, router_weights, selected_experts

@@ -27,6 +27,9 @@ with and without biases as well):
   router_topk_softmax the routing of MoE_Torch (scattermoe/torch_implementation.py:121-132, 193-199); checked against
                       torch.topk + softmax on tie-free logits, a brute-force selection on tiny inputs with ties, and
                       the closed form of the softmax gradient in fp64
+  router_linear       the bias-free gate, x @ w_gate^T (scattermoe/torch_implementation.py:122); checked against a
+                      scalar triple loop, ``F.linear`` and the logits ``moe_forward`` returns in fp64, and against the
+                      exact sum rounded once for 16-bit storage
   expert_bias_*       the bias term of F.linear(rows_e, W[e], bias[e]) (scattermoe/torch_implementation.py:35-43);
                       checked against F.linear per expert and its autograd in fp64
   scatter2scatter, group_bwd_W, group
@@ -284,6 +287,13 @@ def expert_bias_backward(dy, expert_offsets, compute_dtype=torch.float32):
             out[e] = dy[start:end].to(compute_dtype).sum(0)
         start = end
     return out.to(dy.dtype)
+
+
+def router_linear(x: torch.Tensor, w_gate: torch.Tensor, compute_dtype=torch.float32) -> torch.Tensor:
+    """router_logits [T, E] = x [T, H] @ w_gate [E, H]^T of the bias-free gate
+    (scattermoe/torch_implementation.py:122, the ``nn.Linear`` of :110-112): products summed in ``compute_dtype``,
+    one rounding to x's dtype."""
+    return (x.to(compute_dtype) @ w_gate.to(compute_dtype).t()).to(x.dtype)
 
 
 def router_topk_softmax(router_logits: torch.Tensor, top_k: int, compute_dtype=torch.float32):

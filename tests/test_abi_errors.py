@@ -178,6 +178,19 @@ def test_grouped_gemm_argument_checks(lib):
     assert router_bwd(P, P, P, None, 8, 16, 8, 2, BF16, None) == NULL
     assert router_bwd(P, P, P, P, 8, 16, 8, 2, 9, None) == DTYPE
     assert router_bwd(P, P, P, P + 2, 8, 16, 8, 2, F32, None) == ALIGN
+    fused = lib.ck_router_forward
+    #          x  ldx w  ldw logits ld w  w32 sel T   H   E  k  dtype stream
+    assert fused(P, 64, P, 64, P, 8, P, P, P, 16, 64, 8, 2, F32, None) == DTYPE  # 16-bit storage only
+    assert fused(P, 64, P, 64, P, 8, P, P, P, 16, 60, 8, 2, BF16, None) == SHAPE  # H not a multiple of 8
+    assert fused(P, 64, P, 64, P, 8, P, P, P, 16, 64, 129, 2, BF16, None) == SHAPE  # more experts than the launch takes
+    assert fused(P, 64, P, 64, P, 8, P, P, P, 16, 64, 8, 9, BF16, None) == SHAPE  # k > E
+    assert fused(P, 32, P, 64, P, 8, P, P, P, 16, 64, 8, 2, BF16, None) == SHAPE  # row stride below the row length
+    assert fused(P, 68, P, 64, P, 8, P, P, P, 16, 64, 8, 2, BF16, None) == SHAPE  # rows not 16-byte aligned
+    assert fused(P, 64, P, 64, P, 4, P, P, P, 16, 64, 8, 2, BF16, None) == SHAPE  # logits stride below E
+    assert fused(P, 64, None, 64, P, 8, P, P, P, 16, 64, 8, 2, BF16, None) == NULL
+    assert fused(P, 64, P, 64, P, 8, P, P, None, 16, 64, 8, 2, BF16, None) == NULL
+    assert fused(P + 2, 64, P, 64, P, 8, P, P, P, 16, 64, 8, 2, BF16, None) == ALIGN
+    assert fused(P, 64, P, 64, P, 8, P, P, P, 0, 64, 8, 2, BF16, None) == OK  # no tokens
     assert lib.ck_probe_mfma(None, 10, 1, P, None) == NULL
     assert lib.ck_probe_mfma(P, 10, 0, P, None) == SHAPE
 

@@ -373,6 +373,60 @@ def test_router_matches_the_stock_ops_on_the_device(gpu, dtype):
         assert (weights != stock).float().mean().item() < 1e-3  # the two exp implementations round alike
 
 
+ROUTER_LINEAR_CASES = [
+    # T, H, E, k
+    (1000, 256, 8, 2),
+    (333, 1000, 64, 6),    # H = 31.25 blocks of 32: the last block is partly outside the row
+    (50, 72, 5, 5),        # fewer blocks than waves
+    (129, 512, 100, 3),    # 7 column tiles, two values per lane in the selection
+    (77, 64, 128, 64),     # the limits of the launch
+    (9, 8, 1, 1),
+    (4100, 2048, 64, 6),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,H,E,k", ROUTER_LINEAR_CASES)
+def test_router_linear_topk_softmax(gpu, dtype, T, H, E, k):
+    """Router linear + selection in one launch: the logits against the oracle's product, the selection and the
+    weights against the oracle's selection from the logits the launch stored (bit-exact positions), and the three
+    gradients against the oracle's backward through the same selection."""
+    from cute_kernels import _C
+    from cute_kernels.kernels.scattermoe import moe_router
+
+    announce("router linear", dtype, T, H, E, k)
+    x = randn((T, H), dtype, seed=84, scale=0.5)
+    w = randn((E, H), dtype, seed=85, scale=0.2)
+    # a view with a row stride wider than H, as a slice of a larger tensor would be
+    wide = torch.zeros(T, H + 8, dtype=dtype, device=gpu)
+    wide[:, :H] = x.to(gpu)
+    for source in (x.to(gpu), wide[:, :H]):
+        xg = source.detach().requires_grad_(True)
+        wg = w.to(gpu).requires_grad_(True)
+        assert _C.router_forward_supported(xg, wg, k)
+        logits, weights, selected = moe_router(xg, wg, k, fused=True)
+        assert_close(logits, O.router_linear(x, w), dtype, "router logits")
+        stored = logits.detach().cpu()
+        exp_w, exp_sel = O.router_topk_softmax(stored, k)
+        assert torch.equal(selected.cpu(), exp_sel), "positions: selected from the stored logits"
+        assert_close(weights, exp_w, dtype, "routing weights")
+        # gradients: d_logits = backward of the selection + the caller's own gradient of the logits
+        d_weights = randn((T, k), dtype, seed=86)
+        d_direct = randn((T, E), dtype, seed=87, scale=0.1)
+        ((weights * d_weights.to(gpu)).sum() + (logits * d_direct.to(gpu)).sum()).backward()
+        # (the device adds the two parts in the storage type)
+        d_logits = (O.router_topk_softmax_backward(d_weights, stored, exp_sel).float() + d_direct.float()).to(dtype).float()
+        assert_close_long_sums(xg.grad, (d_logits @ w.float()).to(dtype), dtype, "d_x")
+        assert_close_long_sums(wg.grad, (d_logits.t() @ x.float()).to(dtype), dtype, "d_gate_weight")
+    # unsupported operands take the linear followed by the selection
+    odd = x[:, : H - 1].to(gpu) if H > 8 else None
+    if odd is not None:
+        assert not _C.router_forward_supported(odd, w[:, : H - 1].to(gpu), k)
+        l2, w2, s2 = moe_router(odd, w[:, : H - 1].to(gpu).contiguous(), k)
+        assert_close(l2, O.router_linear(x[:, : H - 1], w[:, : H - 1]), dtype, "router logits (two launches)")
+        assert torch.equal(s2.cpu(), O.router_topk_softmax(l2.cpu(), k)[1])
+
+
 # ---- per-expert bias -------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("T,k,E,N,empty", [(16, 2, 4, 128, ()), (300, 3, 7, 200, (0, 6)), (257, 2, 5, 36, (2,)),
@@ -675,6 +729,9 @@ def test_moe_full_size_against_torch_layer(gpu, case):
     moe = build_moe(MoE_Triton, gpu, dtype, E, k, H, I, w_gate, w_fc, w_proj)
     ref = build_moe(MoE_Torch, gpu, dtype, E, k, H, I, w_gate, w_fc, w_proj)
     del w_fc, w_proj
+    # Both layers must route alike to be comparable: the logits of the launch with the router's linear in front can
+    # differ from the library GEMM's in the last bit, and a near-tie then goes to another expert (checked below).
+    moe.fuse_router_linear = False
 
     with torch.no_grad():
         _, _, selected = moe._compute_routing_weights(x)
@@ -709,6 +766,20 @@ def test_moe_full_size_against_torch_layer(gpu, case):
     empty = (load == 0).nonzero().flatten().tolist()
     for e in empty:
         assert not moe.c_fc.weight.grad[e].any() and not moe.c_proj.weight.grad[e].any(), "experts without tokens get zero grads"
+
+    # the router in one launch, at the same size: logits against the library GEMM's, and how often the last bit matters
+    from cute_kernels.kernels.scattermoe import moe_router
+
+    with torch.no_grad():
+        fused_logits, fused_weights, fused_selected = moe_router(x, moe.gate.weight, k, fused=True)
+        _, ref_weights, ref_selected = ref._compute_routing_weights(x)
+    assert_close(fused_logits, logits_r.detach(), dtype, "router logits at full size")
+    assert (fused_logits != logits_r).float().mean().item() < 0.1, "most logits agree to the last bit"
+    agree = (fused_selected.sort(-1).values == ref_selected.sort(-1).values).all(-1)
+    assert agree.float().mean().item() > 0.99, "the same experts for nearly all tokens"
+    exp_w, exp_sel = O.router_topk_softmax(fused_logits.cpu(), k)
+    assert torch.equal(fused_selected.cpu(), exp_sel)
+    assert_close(fused_weights, exp_w, dtype, "routing weights at full size")
 
 
 # ---- operands beyond 32-bit byte offsets: the grouped GEMM switches to 64-bit addressing ------------------------

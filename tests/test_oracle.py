@@ -354,6 +354,30 @@ def test_router_topk_softmax_against_topk_brute_force_and_closed_form():
     assert torch.allclose(d_logits.sum(-1), torch.zeros(37, dtype=F64), atol=1e-15)  # softmax gradients sum to zero
 
 
+def test_router_linear_against_brute_force_and_moe_forward():
+    g = torch.Generator().manual_seed(13)
+    x = torch.randn(7, 10, generator=g, dtype=F64)
+    w = torch.randn(4, 10, generator=g, dtype=F64)
+    logits = O.router_linear(x, w, compute_dtype=F64)
+    for t in range(7):
+        for e in range(4):
+            brute = sum(x[t, h].item() * w[e, h].item() for h in range(10))
+            assert abs(logits[t, e].item() - brute) < 1e-13
+    # a transposed weight or a swapped operand changes the shape or the values
+    assert logits.shape == (7, 4)
+    assert torch.allclose(logits, F.linear(x, w), rtol=1e-14, atol=1e-14)
+    # the layer's own logits are these (second return value of moe_forward)
+    w_fc = torch.randn(4, 12, 10, generator=g, dtype=F64)
+    w_proj = torch.randn(4, 10, 6, generator=g, dtype=F64)
+    _, layer_logits = O.moe_forward(x, w, w_fc, w_proj, 2)
+    assert torch.allclose(layer_logits, logits, rtol=1e-14, atol=1e-14)
+    # 16-bit storage: one rounding of the exact sum (inputs on a coarse grid make the fp32 sum exact)
+    xb = (torch.randint(-8, 9, (5, 16), generator=g).float() / 4).to(torch.bfloat16)
+    wb = (torch.randint(-8, 9, (3, 16), generator=g).float() / 4).to(torch.bfloat16)
+    exact = xb.double() @ wb.double().t()
+    assert torch.equal(O.router_linear(xb, wb), exact.to(torch.bfloat16))
+
+
 def test_residual_rmsnorm_against_autograd_of_the_composition():
     g = torch.Generator().manual_seed(12)
     B, H, eps = 9, 24, 1e-5
