@@ -110,10 +110,12 @@ constexpr int kRouterTokens = 16;  // tokens per workgroup: one MFMA row tile
 
 // NT column tiles of 16 experts.  Operand fragments come straight from memory: lane l of a 16 x 16 x 32 MFMA supplies
 // the 8 consecutive hidden positions 8 * (l / 16) ... of row l % 16 of either operand - one 16-byte load each, and
-// the weight rows stay in L2.  Wave w takes the blocks of 32 hidden positions w, w + 4, ...; U of them are in flight.
+// the weight rows stay in L2.  Wave w of NW takes the blocks of 32 hidden positions w, w + NW, ...; U of them are in
+// flight.  Many waves per workgroup keep both chains short: the blocks a wave walks through, and the tokens it then
+// selects for one after the other (16 / NW; a selection is a chain of dependent shuffles).
 // The result lane l holds of tile nt is (token 4 * (l / 16) + r, expert 16 nt + l % 16), r = 0 .. 3.
-template <typename T, int NT>
-__global__ void __launch_bounds__(256)
+template <typename T, int NT, int NW>
+__global__ void __launch_bounds__(NW * CK_WAVE)
     router_linear_fwd_kernel(const typename T::storage_t* __restrict__ x, int64_t ldx,
                              const typename T::storage_t* __restrict__ w, int64_t ldw,
                              typename T::storage_t* __restrict__ logits, int64_t ld_logits,
@@ -121,8 +123,10 @@ __global__ void __launch_bounds__(256)
                              int64_t* __restrict__ selected, int64_t tokens, int H, int E, int k) {
     typedef typename T::storage_t S;
     typedef typename RouterMma<T>::frag_t frag_t;
-    constexpr int EP = NT * 16, VPL = (EP + CK_WAVE - 1) / CK_WAVE, U = NT <= 2 ? 4 : 2;
-    __shared__ float part[4][kRouterTokens][EP + 1];
+    constexpr int EP = NT * 16, VPL = (EP + CK_WAVE - 1) / CK_WAVE, U = NT <= 1 ? 4 : NT <= 2 ? 2 : 1;
+    constexpr int TPW = kRouterTokens / NW;  // tokens a wave selects for
+    static_assert(kRouterTokens % NW == 0, "whole tokens per wave");
+    __shared__ float part[NW][kRouterTokens][EP + 1];
     const int wave = threadIdx.x / CK_WAVE, lane = lane_id();
     const int row = lane % 16, kc = lane / 16;
     const int64_t t0 = (int64_t)blockIdx.x * kRouterTokens;
@@ -140,7 +144,7 @@ __global__ void __launch_bounds__(256)
     for (int nt = 0; nt < NT; ++nt) acc[nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     const frag_t zero = {};
     const int k_last = H - 8 - kc * 8;  // (relative to the lane's first packet) the last packet of the row
-    for (int kb = wave; kb * 32 < H; kb += 4 * U) {
+    for (int kb = wave; kb * 32 < H; kb += NW * U) {
         // All loads of a turn are issued before any is used, and none sits behind a branch: a packet past the end of
         // the row (H is a multiple of 8, so it lies wholly inside or outside) or in a row past the last expert is
         // read from a valid place instead and replaced by zeros afterwards.
@@ -148,7 +152,7 @@ __global__ void __launch_bounds__(256)
         bool in[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int k0 = (kb + 4 * u) * 32;
+            const int k0 = (kb + NW * u) * 32;
             in[u] = k0 <= k_last;
             const int kl = in[u] ? k0 : 0;
             a[u] = nt_load(reinterpret_cast<const frag_t*>(xrow + kl));
@@ -167,9 +171,9 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
         for (int r = 0; r < 4; ++r) part[wave][4 * kc + r][nt * 16 + row] = acc[nt][r];
     __syncthreads();
-    // wave w finishes tokens 4 w .. 4 w + 3: lane l holds experts l, l + 64
-    for (int i = 0; i < 4; ++i) {
-        const int tt = wave * 4 + i;
+    // wave w finishes tokens TPW w ...: lane l holds experts l, l + 64
+    for (int i = 0; i < TPW; ++i) {
+        const int tt = wave * TPW + i;
         const int64_t t = t0 + tt;
         if (t >= tokens) break;
         float v[VPL];
@@ -178,7 +182,10 @@ __global__ void __launch_bounds__(256)
             const int e = j * CK_WAVE + lane;
             v[j] = 0.f;
             if (e < E) {
-                const S rounded = T::down(((part[0][tt][e] + part[1][tt][e]) + part[2][tt][e]) + part[3][tt][e]);
+                float sum = part[0][tt][e];
+#pragma unroll
+                for (int pw = 1; pw < NW; ++pw) sum += part[pw][tt][e];
+                const S rounded = T::down(sum);
                 logits[t * ld_logits + e] = rounded;
                 v[j] = T::up(rounded);
             }
@@ -277,7 +284,8 @@ extern "C" int ck_router_forward(const void* x, int64_t x_stride, const void* ga
     hipStream_t s = (hipStream_t)stream;
     const int nt = (int)ck_ceil_div(E, 16);
 #define CK_ROUTER_LINEAR(TT, NT)                                                                                    \
-    hipLaunchKernelGGL((ck::router_linear_fwd_kernel<TT, NT>), dim3((unsigned)grid), dim3(256), 0, s,               \
+    hipLaunchKernelGGL((ck::router_linear_fwd_kernel<TT, NT, NT <= 4 ? 16 : 8>), dim3((unsigned)grid),             \
+                       dim3((NT <= 4 ? 16 : 8) * CK_WAVE), 0, s,                                                   \
                        (const TT::storage_t*)x, x_stride, (const TT::storage_t*)gate_weight, gate_weight_stride,  \
                        (TT::storage_t*)logits, logits_stride, (TT::storage_t*)weights, weights_f32, selected, tokens, \
                        (int)H, (int)E, (int)k)

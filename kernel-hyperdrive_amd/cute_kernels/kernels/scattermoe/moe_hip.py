@@ -166,9 +166,9 @@ class _Router(torch.autograd.Function):
         return d_x, d_gate_weight, None
 
 
-# Up to this many experts the launch with the linear in front is the faster one (8 experts, 8192 x 4096 tokens:
-# 25 us against 22 + 15 for the library GEMM and the selection; 64 experts, 16384 x 2048: 61 against 23 + 21 - a wave
-# of that launch selects for four tokens one after the other, and a selection is a chain of dependent shuffles).
+# Up to this many experts the launch with the linear in front is used: level with the library GEMM + selection at 8
+# experts (22 us against 15 + 8 at 8192 x 4096 tokens, one launch fewer), slower at 64 (51 us against 22 + 21 at
+# 16384 x 2048: selecting 6 of 64 is a long chain of dependent shuffles per token).
 _FUSED_ROUTER_MAX_EXPERTS = 16
 
 
