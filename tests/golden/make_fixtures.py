@@ -152,6 +152,23 @@ def make_router(rng):
              weights=weights, d_logits=d_logits)
 
 
+def make_router_linear(rng):
+    """Logits of the bias-free gate as exact sums: every product is a multiple of 2^-12 below 2^3 and a sum of 40 of
+    them is exact in fp32 and fp64 alike, so an implementation that accumulates in fp32 must give the one rounding of
+    these values to its storage type, bit for bit."""
+    T, H, E = 12, 40, 6
+    x = dyadic(rng, (T, H), 0.25)
+    w = dyadic(rng, (E, H), 0.25)
+    logits = np.zeros((T, E))
+    for t in range(T):
+        for e in range(E):
+            acc = 0.0
+            for h in range(H):
+                acc += x[t, h] * w[e, h]
+            logits[t, e] = acc
+    np.savez(os.path.join(HERE, "router_linear.npz"), x=x, w=w, logits=logits)
+
+
 def make_residual_rmsnorm(rng):
     B, H, eps = 6, 48, 1e-5
     x = dyadic(rng, (B, H), 1.0)
@@ -215,6 +232,7 @@ def main():
     make_router(rng2)
     make_residual_rmsnorm(rng2)
     make_moe_bias(rng2)
+    make_router_linear(np.random.default_rng(20240609))
     for name in sorted(os.listdir(HERE)):
         if name.endswith(".npz"):
             print(name, os.path.getsize(os.path.join(HERE, name)), "bytes")

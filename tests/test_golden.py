@@ -25,7 +25,7 @@ def load(name):
 def test_fixture_inputs_are_exact_in_bfloat16():
     for name, keys in (("swiglu", ["gate", "up", "dy"]), ("rmsnorm", ["x", "w", "dy"]), ("embedding", ["table", "dy"]),
                        ("moe", ["x", "w_gate", "w_fc", "w_proj", "dy"]), ("router", ["logits", "d_weights"]),
-                       ("residual_rmsnorm", ["x", "r", "s", "w", "dy", "ds"]),
+                       ("residual_rmsnorm", ["x", "r", "s", "w", "dy", "ds"]), ("router_linear", ["x", "w"]),
                        ("moe_bias", ["x", "w_gate", "w_fc", "w_proj", "b_fc", "b_proj", "dy"])):
         f = load(name)
         for k in keys:
@@ -96,6 +96,14 @@ def test_oracle_router_golden():
     torch.testing.assert_close(d_logits, f["d_logits"], rtol=1e-12, atol=1e-13)
 
 
+def test_oracle_router_linear_golden():
+    f = load("router_linear")
+    assert torch.equal(O.router_linear(f["x"], f["w"], torch.float64), f["logits"])
+    # fp32 accumulation of these operands is exact: one rounding of the exact sums
+    for dtype in (torch.bfloat16, torch.float16):
+        assert torch.equal(O.router_linear(f["x"].to(dtype), f["w"].to(dtype)), f["logits"].to(dtype))
+
+
 def test_oracle_residual_rmsnorm_golden():
     f = load("residual_rmsnorm")
     eps = float(f["eps"])
@@ -128,6 +136,21 @@ def test_hip_router_golden(gpu, dtype):
     assert torch.equal(selected.cpu(), f["selected"]), "largest first, equal logits in the order of their positions"
     assert_close(weights.detach(), f["weights"].to(dtype), dtype, "weights")
     assert_close(logits.grad, f["d_logits"].to(dtype), dtype, "d_logits")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_hip_router_linear_golden(gpu, dtype):
+    from cute_kernels.kernels.scattermoe import moe_router
+
+    announce("golden router linear", dtype)
+    f = load("router_linear")
+    x, w = f["x"].to(dtype).to(gpu), f["w"].to(dtype).to(gpu)
+    logits, weights, selected = moe_router(x, w, 2, fused=True)
+    assert torch.equal(logits.cpu(), f["logits"].to(dtype)), "exact sums, rounded once"
+    exp_w, exp_sel = O.router_topk_softmax(logits.cpu(), 2)
+    assert torch.equal(selected.cpu(), exp_sel)
+    assert_close(weights, exp_w, dtype, "weights")
 
 
 @pytest.mark.gpu
