@@ -9,10 +9,9 @@
 //   backward: d_v[t, j]       = w_j * (g_j - sum_i g_i w_i)     (softmax backward on the fp32 weights)
 //             d_logits[t, e]  = d_v[t, j] where e = selected[t, j], else 0  (every element of the row is written)
 // The forward also exists with the router's linear in front (logits = x W^T, torch_implementation.py:122): a
-// workgroup multiplies 16 tokens by all experts' rows with MFMAs, its four waves splitting the hidden dimension,
-// adds the four partial blocks up through LDS, rounds the logits once to the storage type, writes them, and selects
-// from the rounded values - as the stock sequence does, which selects from the stored logits.  x is read once; a
-// library GEMM with so few output columns reads it at a fraction of the memory bandwidth.
+// workgroup multiplies 16 tokens by all experts' rows with MFMAs, its waves splitting the hidden dimension, adds
+// the partial blocks up through LDS in a fixed order, rounds the logits once to the storage type, writes them, and
+// selects from the rounded values - as the stock sequence does, which selects from the stored logits.
 #include <math.h>
 
 #include "ck_device.h"
@@ -193,7 +192,6 @@ __global__ void __launch_bounds__(NW * CK_WAVE)
         router_select_token<T, VPL>(v, lane, E, k, t, weights, weights_f32, selected);
     }
 }
-
 
 template <typename T, int VPL>
 __global__ void __launch_bounds__(256)
