@@ -272,6 +272,21 @@ int ck_router_forward(const void* x, int64_t x_stride, const void* gate_weight, 
                       int64_t tokens, int64_t H, int64_t E, int64_t k, int dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * Gradient of the router's weight: d_weight [E, H] = d_logits^T x
+ * replaces the weight gradient autograd derives for `self.gate(hidden_states)`
+ * (scattermoe/torch_implementation.py:122; an [E, tokens] x [tokens, H] product with few outputs).
+ *   d_logits_t [E, tokens]: d_logits transposed, dense; x [tokens, H] with row stride x_stride.
+ *   The tokens are cut into pieces whose products are kept in fp32 in the workspace
+ *   (ck_router_weight_grad_workspace_size bytes, 16-byte aligned) and added up in a fixed order: one rounding.
+ * bf16 and fp16 only (CK_ERR_DTYPE otherwise); tokens and H multiples of 8, E <= 128, d_logits_t and x 16-byte
+ * aligned, x_stride a multiple of 8.
+ * ------------------------------------------------------------------------------------------- */
+int64_t ck_router_weight_grad_workspace_size(int64_t tokens, int64_t H, int64_t E);
+int ck_router_weight_grad(const void* d_logits_t, const void* x, int64_t x_stride, void* d_weight,
+                          int64_t d_weight_stride, void* workspace, int64_t workspace_bytes, int64_t tokens, int64_t H,
+                          int64_t E, int dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
  * Per-expert bias of the grouped linears
  * replaces the bias term of F.linear(rows_e, W[e], bias[e]) in scattermoe/torch_implementation.py:35-43 (the
  * reference's Triton experts, triton_implementation/__init__.py:24-34, do not read their bias parameter).

@@ -223,6 +223,123 @@ __global__ void __launch_bounds__(256)
     }
 }
 
+
+// ---- gradient of the router's weight -----------------------------------------------------------------------
+// d_weight[e, h] = sum_t d_logits[t, e] * x[t, h]: few outputs, a sum over every token.  The tokens are cut into
+// pieces; workgroup (column group, piece) multiplies its piece for 256 columns and writes an fp32 partial block, and
+// a second launch adds the pieces up in their order and rounds once.  d_logits comes transposed ([E, T], a small
+// tensor), so the MFMA's row operand is one 16-byte load per lane; x is contracted along its rows, so each wave
+// copies 32 tokens x 64 columns to its own LDS region with 16-byte accesses and picks the column operand from there
+// element by element.  Lane l holds (expert 16 nt + 4 (l / 16) + r, column 16 ht + l % 16) of tile (nt, ht).
+constexpr int kWgPieceTokens = 32;   // tokens per step
+constexpr int kWgWaveCols = 64;      // columns per wave
+constexpr int kWgCols = 4 * kWgWaveCols;
+constexpr int kWgRowPad = kWgWaveCols + 8;  // LDS row length in elements (16-byte aligned rows)
+
+template <typename T, int NT>
+__global__ void __launch_bounds__(256)
+    router_weight_grad_kernel(const typename T::storage_t* __restrict__ dlt, const typename T::storage_t* __restrict__ x,
+                              int64_t ldx, float* __restrict__ partial, int tokens, int H, int E, int piece_tokens) {
+    typedef typename T::storage_t S;
+    typedef typename RouterMma<T>::frag_t frag_t;
+    __shared__ __attribute__((aligned(16))) S tile[4][kWgPieceTokens][kWgRowPad];
+    const int wave = threadIdx.x / CK_WAVE, lane = lane_id();
+    const int row = lane % 16, g = lane / 16;
+    const int h0 = blockIdx.x * kWgCols + wave * kWgWaveCols;
+    const int piece = blockIdx.y;
+    const int t_begin = piece * piece_tokens, t_end = min(tokens, t_begin + piece_tokens);
+    f32x4_t acc[NT][4];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int ht = 0; ht < 4; ++ht) acc[nt][ht] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    const frag_t zero = {};
+    // the lane's part in copying the x tile: token lane / 8 + 8 i of the step, columns 8 (lane % 8) ... of the wave's 64
+    const int ct = lane / 8, cc = (lane % 8) * 8;
+    const int col = min(h0 + cc, H - 8);  // columns past H are read from a valid place and never stored
+    if (h0 < H) {
+        for (int t0 = t_begin; t0 < t_end; t0 += kWgPieceTokens) {
+            frag_t xin[4], a[NT];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int t = t0 + ct + 8 * i;
+                xin[i] = nt_load(reinterpret_cast<const frag_t*>(x + (int64_t)min(t, tokens - 1) * ldx + col));
+            }
+            const int ta = t0 + 8 * g;  // tokens are a multiple of 8: the packet lies inside the row or outside
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const int e = nt * 16 + row;
+                a[nt] = *reinterpret_cast<const frag_t*>(dlt + (int64_t)min(e, E - 1) * tokens + min(ta, tokens - 8));
+                if (e >= E || ta >= t_end) a[nt] = zero;
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int t = t0 + ct + 8 * i;
+                *reinterpret_cast<frag_t*>(&tile[wave][ct + 8 * i][cc]) = t < t_end ? xin[i] : zero;
+            }
+            __builtin_amdgcn_s_waitcnt(0xC07F);  // the wave's own LDS writes (lgkmcnt 0)
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int ht = 0; ht < 4; ++ht) {
+                union {
+                    S e[8];
+                    frag_t f;
+                } b;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) b.e[j] = tile[wave][8 * g + j][ht * 16 + row];
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) acc[nt][ht] = RouterMma<T>::mma(a[nt], b.f, acc[nt][ht]);
+            }
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+            __builtin_amdgcn_wave_barrier();
+        }
+    }
+    float* out = partial + (int64_t)piece * E * H;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int ht = 0; ht < 4; ++ht)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int e = nt * 16 + 4 * g + r, h = h0 + ht * 16 + row;
+                if (e < E && h < H) out[(int64_t)e * H + h] = acc[nt][ht][r];
+            }
+}
+
+// d_weight[e, h] = sum over the pieces of partial[piece][e][h], four columns per lane, in a fixed order (four running
+// sums over the pieces p % 4, so that four loads are under way); one rounding
+template <typename T>
+__global__ void __launch_bounds__(256)
+    router_weight_grad_sum_kernel(const float* __restrict__ partial, typename T::storage_t* __restrict__ dw, int64_t ld,
+                                  int pieces, int H, int E) {
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;  // H is a multiple of 8: the four share a row
+    const int64_t n = (int64_t)E * H;
+    if (i >= n) return;
+    f32x4_t sum[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) sum[u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    int p = 0;
+    for (; p + 4 <= pieces; p += 4) {
+        f32x4_t v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const f32x4_t*>(partial + (int64_t)(p + u) * n + i);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) sum[u] += v[u];
+    }
+    for (; p < pieces; ++p) sum[p % 4] += *reinterpret_cast<const f32x4_t*>(partial + (int64_t)p * n + i);
+    const f32x4_t total = (sum[0] + sum[1]) + (sum[2] + sum[3]);
+    VPack<T, 4> out;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) out.v[r] = T::down(total[r]);
+    typename T::storage_t* dst = dw + (i / H) * ld + i % H;
+    if ((reinterpret_cast<uintptr_t>(dst) & 7u) == 0) {
+        *reinterpret_cast<VPack<T, 4>*>(dst) = out;
+    } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) dst[r] = out.v[r];
+    }
+}
+
 }  // namespace ck
 
 namespace {
@@ -323,5 +440,69 @@ extern "C" int ck_router_topk_softmax_backward(const void* d_weights, const floa
         CK_ROUTER_LAUNCH(router_bwd_kernel, (const S*)d_weights, weights_f32, selected, (S*)d_logits, d_logits_stride,
                          tokens, (int)E, (int)k);
     });
+    return ck_launch_status();
+}
+
+namespace {
+// pieces of the token range for ck_router_weight_grad: about two workgroups per CU, pieces of whole 32-token steps
+void weight_grad_pieces(int64_t tokens, int64_t H, int64_t* pieces, int64_t* piece_tokens) {
+    const int64_t groups = ck_ceil_div(H, ck::kWgCols);
+    int64_t want = ck_ceil_div(512, groups);
+    const int64_t steps = ck_ceil_div(tokens, ck::kWgPieceTokens);
+    if (want > steps) want = steps;
+    if (want < 1) want = 1;
+    *piece_tokens = ck_ceil_div(steps, want) * ck::kWgPieceTokens;
+    *pieces = ck_ceil_div(tokens, *piece_tokens);
+}
+}  // namespace
+
+extern "C" int64_t ck_router_weight_grad_workspace_size(int64_t tokens, int64_t H, int64_t E) {
+    if (tokens <= 0 || H <= 0 || E <= 0) return 0;
+    int64_t pieces, piece_tokens;
+    weight_grad_pieces(tokens, H, &pieces, &piece_tokens);
+    return pieces * E * H * (int64_t)sizeof(float);
+}
+
+extern "C" int ck_router_weight_grad(const void* d_logits_t, const void* x, int64_t x_stride, void* d_weight,
+                                     int64_t d_weight_stride, void* workspace, int64_t workspace_bytes, int64_t tokens,
+                                     int64_t H, int64_t E, int dtype, void* stream) {
+    if (dtype != CK_BF16 && dtype != CK_F16) return CK_ERR_DTYPE;
+    if (tokens <= 0 || tokens > 0x7fffffff - 1024 || (tokens & 7) || H <= 0 || H > 0x7fffffff - 1024 || (H & 7) || E <= 0 ||
+        E > kMaxLinearExperts || x_stride < H || (x_stride & 7) || d_weight_stride < H)
+        return CK_ERR_SHAPE;
+    if (!d_logits_t || !x || !d_weight || !workspace) return CK_ERR_NULL;
+    if (!ck_aligned16(d_logits_t) || !ck_aligned16(x) || !ck_aligned_elem(d_weight, dtype)) return CK_ERR_ALIGN;
+    if ((reinterpret_cast<uintptr_t>(workspace) & 15u) || workspace_bytes < ck_router_weight_grad_workspace_size(tokens, H, E))
+        return CK_ERR_WORKSPACE;
+    int64_t pieces, piece_tokens;
+    weight_grad_pieces(tokens, H, &pieces, &piece_tokens);
+    if (pieces > 65535) return CK_ERR_SHAPE;
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid((unsigned)ck_ceil_div(H, ck::kWgCols), (unsigned)pieces);
+    const int nt = (int)ck_ceil_div(E, 16);
+#define CK_WEIGHT_GRAD(TT, NT)                                                                                       \
+    hipLaunchKernelGGL((ck::router_weight_grad_kernel<TT, NT>), grid, dim3(256), 0, s, (const TT::storage_t*)d_logits_t, \
+                       (const TT::storage_t*)x, x_stride, (float*)workspace, (int)tokens, (int)H, (int)E,           \
+                       (int)piece_tokens)
+#define CK_WEIGHT_GRAD_NT(TT)                                                                                   \
+    do {                                                                                                        \
+        if (nt <= 1)                                                                                            \
+            CK_WEIGHT_GRAD(TT, 1);                                                                              \
+        else if (nt <= 2)                                                                                       \
+            CK_WEIGHT_GRAD(TT, 2);                                                                              \
+        else if (nt <= 4)                                                                                       \
+            CK_WEIGHT_GRAD(TT, 4);                                                                              \
+        else                                                                                                    \
+            CK_WEIGHT_GRAD(TT, 8);                                                                              \
+        hipLaunchKernelGGL((ck::router_weight_grad_sum_kernel<TT>), dim3((unsigned)ck_ceil_div(E * H, 1024)),   \
+                           dim3(256), 0, s, (const float*)workspace, (TT::storage_t*)d_weight, d_weight_stride, \
+                           (int)pieces, (int)H, (int)E);                                                        \
+    } while (0)
+    if (dtype == CK_BF16)
+        CK_WEIGHT_GRAD_NT(ck::BF16);
+    else
+        CK_WEIGHT_GRAD_NT(ck::F16);
+#undef CK_WEIGHT_GRAD_NT
+#undef CK_WEIGHT_GRAD
     return ck_launch_status();
 }

@@ -80,6 +80,8 @@ _SIGNATURES = {
     "ck_router_topk_softmax_forward": (_i32, [_p, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, _p]),
     "ck_router_topk_softmax_backward": (_i32, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i32, _p]),
     "ck_router_forward": (_i32, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _i32, _p]),
+    "ck_router_weight_grad_workspace_size": (_i64, [_i64, _i64, _i64]),
+    "ck_router_weight_grad": (_i32, [_p, _p, _i64, _p, _i64, _p, _i64, _i64, _i64, _i64, _i32, _p]),
     "ck_probe_mfma": (_i32, [_p, _i64, _i32, _p, _p]),
 }
 
@@ -601,6 +603,42 @@ def router_forward(x, gate_weight, logits, weights, weights_f32, selected) -> No
                                   logits.stride(0), _ptr(weights), _ptr(weights_f32), _ptr(selected), T, H, E, k,
                                   dtype_code(x.dtype), L.stream),
             "ck_router_forward",
+        )
+
+
+def router_weight_grad_supported(d_logits, x) -> bool:
+    """Whether ``router_weight_grad`` takes operands of this type, shape and strides."""
+    return (
+        x.dim() == 2
+        and d_logits.dim() == 2
+        and x.dtype in (torch.bfloat16, torch.float16)
+        and d_logits.dtype == x.dtype
+        and 0 < d_logits.size(1) <= ROUTER_LINEAR_MAX_EXPERTS
+        and x.size(0) > 0 and x.size(0) % 8 == 0
+        and x.size(1) % 8 == 0
+        and x.stride(1) == 1 and x.stride(0) % 8 == 0
+    )
+
+
+def router_weight_grad_workspace_size(tokens: int, H: int, E: int) -> int:
+    return int(load_library().ck_router_weight_grad_workspace_size(tokens, H, E))
+
+
+def router_weight_grad(d_logits_t, x, d_weight, workspace) -> None:
+    """d_weight [E, H] = d_logits_t [E, T] @ x [T, H], fp32 partial sums over pieces of the tokens, one rounding."""
+    lib = load_library()
+    E, T = d_logits_t.shape
+    H = x.size(1)
+    if x.size(0) != T or d_logits_t.dtype != x.dtype or d_weight.dtype != x.dtype:
+        raise ValueError("router_weight_grad: d_logits_t [E, T], x [T, H] and d_weight [E, H] of one dtype")
+    if not d_logits_t.is_contiguous() or x.stride(1) != 1 or d_weight.stride(1) != 1 or tuple(d_weight.shape) != (E, H):
+        raise ValueError("router_weight_grad: dense d_logits_t, unit column stride for x and d_weight [E, H]")
+    with _Launch(d_logits_t, x, d_weight, workspace) as L:
+        _check(
+            lib.ck_router_weight_grad(_ptr(d_logits_t), _ptr(x), x.stride(0), _ptr(d_weight), d_weight.stride(0),
+                                      _ptr(workspace), workspace.numel() * workspace.element_size(), T, H, E,
+                                      dtype_code(x.dtype), L.stream),
+            "ck_router_weight_grad",
         )
 
 

@@ -138,10 +138,51 @@ def router_forward_hip(
     return logits, weights, weights_f32, selected
 
 
+def _router_weight_grad_fake(d_logits: torch.Tensor, x: torch.Tensor):
+    return torch.empty(d_logits.size(1), x.size(1), dtype=x.dtype, device=x.device)
+
+
+@cute_op(f"{LIBRARY_NAME}::router_weight_grad_hip", mutates_args={}, fake_func=_router_weight_grad_fake)
+def router_weight_grad_hip(d_logits: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+    T, E = d_logits.shape
+    H = x.size(1)
+    d_logits_t = d_logits.t().contiguous()
+    if x.data_ptr() % 16 != 0:
+        x = x.clone()
+    d_weight = torch.empty(E, H, dtype=x.dtype, device=x.device)
+    workspace = torch.empty(_C.router_weight_grad_workspace_size(T, H, E), dtype=torch.uint8, device=x.device)
+    _C.router_weight_grad(d_logits_t, x, d_weight, workspace)
+    return d_weight
+
+
+def _gate_weight_grad(d_logits: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+    """``d_logits^T @ x`` -> [E, H]: a sum over all tokens with few outputs, which a library GEMM runs on a handful
+    of CUs; the HIP launch cuts the tokens into pieces with fp32 partial sums."""
+    if _C.router_weight_grad_supported(d_logits, x):
+        return router_weight_grad_hip(d_logits, x)
+    return d_logits.t() @ x
+
+
+class _GateLinear(torch.autograd.Function):
+    """``F.linear(x, gate_weight)`` with the weight's gradient through ``_gate_weight_grad``."""
+
+    @staticmethod
+    def forward(ctx, x, gate_weight):
+        ctx.save_for_backward(x, gate_weight)
+        return torch.nn.functional.linear(x, gate_weight)
+
+    @staticmethod
+    def backward(ctx, d_logits):
+        x, gate_weight = ctx.saved_tensors
+        d_x = d_logits @ gate_weight if ctx.needs_input_grad[0] else None
+        d_gate_weight = _gate_weight_grad(d_logits, x) if ctx.needs_input_grad[1] else None
+        return d_x, d_gate_weight
+
+
 class _Router(torch.autograd.Function):
     """Router linear, top-k and softmax as one forward launch.  Backward: the selection's backward launch gives
-    d_logits, the caller's own gradient of the logits (an auxiliary loss) is added, and the two products with
-    d_logits are library GEMMs as they are for ``F.linear``."""
+    d_logits, the caller's own gradient of the logits (an auxiliary loss) is added; d_x is a library GEMM as it is for
+    ``F.linear``, the weight's gradient goes through ``_gate_weight_grad``."""
 
     @staticmethod
     def forward(ctx, x, gate_weight, top_k):
@@ -162,7 +203,7 @@ class _Router(torch.autograd.Function):
         if total is None:
             return None, None, None
         d_x = total @ gate_weight if ctx.needs_input_grad[0] else None
-        d_gate_weight = total.t() @ x if ctx.needs_input_grad[1] else None
+        d_gate_weight = _gate_weight_grad(total, x) if ctx.needs_input_grad[1] else None
         return d_x, d_gate_weight, None
 
 
@@ -184,7 +225,10 @@ def moe_router(
         fused = gate_weight.size(0) <= _FUSED_ROUTER_MAX_EXPERTS
     if fused and _C.router_forward_supported(x, gate_weight, top_k):
         return _Router.apply(x, gate_weight, top_k)
-    router_logits = torch.nn.functional.linear(x, gate_weight)
+    if x.dim() == 2 and x.dtype in (torch.bfloat16, torch.float16) and gate_weight.dtype == x.dtype:
+        router_logits = _GateLinear.apply(x, gate_weight)
+    else:
+        router_logits = torch.nn.functional.linear(x, gate_weight)
     router_weights, selected_experts = router_topk_softmax(router_logits, top_k)
     return router_logits, router_weights, selected_experts
 

@@ -29,7 +29,8 @@ with and without biases as well):
                       the closed form of the softmax gradient in fp64
   router_linear       the bias-free gate, x @ w_gate^T (scattermoe/torch_implementation.py:122); checked against a
                       scalar triple loop, ``F.linear`` and the logits ``moe_forward`` returns in fp64, and against the
-                      exact sum rounded once for 16-bit storage
+                      exact sum rounded once for 16-bit storage; router_linear_backward against autograd of
+                      ``F.linear`` in fp64
   expert_bias_*       the bias term of F.linear(rows_e, W[e], bias[e]) (scattermoe/torch_implementation.py:35-43);
                       checked against F.linear per expert and its autograd in fp64
   scatter2scatter, group_bwd_W, group
@@ -294,6 +295,15 @@ def router_linear(x: torch.Tensor, w_gate: torch.Tensor, compute_dtype=torch.flo
     (scattermoe/torch_implementation.py:122, the ``nn.Linear`` of :110-112): products summed in ``compute_dtype``,
     one rounding to x's dtype."""
     return (x.to(compute_dtype) @ w_gate.to(compute_dtype).t()).to(x.dtype)
+
+
+def router_linear_backward(d_logits: torch.Tensor, x: torch.Tensor, w_gate: torch.Tensor, compute_dtype=torch.float32):
+    """(d_x [T, H], d_w_gate [E, H]) of ``router_linear``: d_logits @ w_gate and d_logits^T @ x, each summed in
+    ``compute_dtype`` and rounded once - what autograd derives for the ``nn.Linear`` of
+    scattermoe/torch_implementation.py:122."""
+    d_x = (d_logits.to(compute_dtype) @ w_gate.to(compute_dtype)).to(x.dtype)
+    d_w = (d_logits.to(compute_dtype).t() @ x.to(compute_dtype)).to(w_gate.dtype)
+    return d_x, d_w
 
 
 def router_topk_softmax(router_logits: torch.Tensor, top_k: int, compute_dtype=torch.float32):

@@ -191,6 +191,21 @@ def test_grouped_gemm_argument_checks(lib):
     assert fused(P, 64, P, 64, P, 8, P, P, None, 16, 64, 8, 2, BF16, None) == NULL
     assert fused(P + 2, 64, P, 64, P, 8, P, P, P, 16, 64, 8, 2, BF16, None) == ALIGN
     assert fused(P, 64, P, 64, P, 8, P, P, P, 0, 64, 8, 2, BF16, None) == OK  # no tokens
+    wgrad = lib.ck_router_weight_grad
+    big = 1 << 30
+    #          dlt x  ldx dw ld  ws  bytes T   H   E  dtype stream
+    assert wgrad(P, P, 64, P, 64, P, big, 16, 64, 8, F32, None) == DTYPE  # 16-bit storage only
+    assert wgrad(P, P, 64, P, 64, P, big, 12, 64, 8, BF16, None) == SHAPE  # tokens not a multiple of 8
+    assert wgrad(P, P, 64, P, 64, P, big, 16, 60, 8, BF16, None) == SHAPE  # H not a multiple of 8
+    assert wgrad(P, P, 64, P, 64, P, big, 16, 64, 129, BF16, None) == SHAPE  # more experts than the launch takes
+    assert wgrad(P, P, 32, P, 64, P, big, 16, 64, 8, BF16, None) == SHAPE  # row stride below the row length
+    assert wgrad(P, P, 64, P, 32, P, big, 16, 64, 8, BF16, None) == SHAPE
+    assert wgrad(None, P, 64, P, 64, P, big, 16, 64, 8, BF16, None) == NULL
+    assert wgrad(P, P, 64, P, 64, None, big, 16, 64, 8, BF16, None) == NULL
+    assert wgrad(P, P + 2, 64, P, 64, P, big, 16, 64, 8, BF16, None) == ALIGN
+    assert wgrad(P, P, 64, P, 64, P, 16, 16, 64, 8, BF16, None) == WORKSPACE  # workspace too small
+    assert lib.ck_router_weight_grad_workspace_size(16, 64, 8) == 8 * 64 * 4  # one piece
+    assert lib.ck_router_weight_grad_workspace_size(0, 64, 8) == 0
     assert lib.ck_probe_mfma(None, 10, 1, P, None) == NULL
     assert lib.ck_probe_mfma(P, 10, 0, P, None) == SHAPE
 

@@ -427,6 +427,33 @@ def test_router_linear_topk_softmax(gpu, dtype, T, H, E, k):
         assert torch.equal(s2.cpu(), O.router_topk_softmax(l2.cpu(), k)[1])
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,H,E", [(8, 8, 1), (1000, 200, 5), (4104, 1000, 64), (16384, 2048, 64), (8192, 4096, 8),
+                                   (40, 264, 128), (3000, 72, 100)])
+def test_router_weight_grad(gpu, dtype, T, H, E):
+    """d_logits^T x with the tokens cut into pieces: against the oracle's product (fp32 sums, one rounding), through a
+    view of x with a wider row stride as well."""
+    from cute_kernels import _C
+    from cute_kernels.kernels.scattermoe.moe_hip import _gate_weight_grad
+
+    announce("router weight grad", dtype, T, H, E)
+    x = randn((T, H), dtype, seed=88, scale=0.5)
+    d_logits = randn((T, E), dtype, seed=89, scale=0.5)
+    w = torch.zeros(E, H, dtype=dtype)
+    _, expected = O.router_linear_backward(d_logits, x, w)
+    wide = torch.zeros(T, H + 16, dtype=dtype, device=gpu)
+    wide[:, :H] = x.to(gpu)
+    for source in (x.to(gpu), wide[:, :H]):
+        assert _C.router_weight_grad_supported(d_logits.to(gpu), source)
+        got = _gate_weight_grad(d_logits.to(gpu), source)
+        assert got.shape == (E, H)
+        assert_close(got, expected, dtype, "d_gate_weight")
+    # operands the launch does not take go to the library product
+    assert not _C.router_weight_grad_supported(d_logits[:-1].to(gpu), x[:-1].to(gpu))
+    assert_close(_gate_weight_grad(d_logits[:-1].to(gpu), x[:-1].to(gpu)),
+                 O.router_linear_backward(d_logits[:-1], x[:-1], w)[1], dtype, "d_gate_weight (library product)")
+
+
 # ---- per-expert bias -------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("T,k,E,N,empty", [(16, 2, 4, 128, ()), (300, 3, 7, 200, (0, 6)), (257, 2, 5, 36, (2,)),

@@ -378,6 +378,17 @@ def test_router_linear_against_brute_force_and_moe_forward():
     assert torch.equal(O.router_linear(xb, wb), exact.to(torch.bfloat16))
 
 
+def test_router_linear_backward_against_autograd():
+    g = torch.Generator().manual_seed(14)
+    x = torch.randn(9, 6, generator=g, dtype=F64, requires_grad=True)
+    w = torch.randn(4, 6, generator=g, dtype=F64, requires_grad=True)
+    d_logits = torch.randn(9, 4, generator=g, dtype=F64)
+    F.linear(x, w).backward(d_logits)
+    d_x, d_w = O.router_linear_backward(d_logits, x.detach(), w.detach(), compute_dtype=F64)
+    assert d_x.shape == (9, 6) and d_w.shape == (4, 6)
+    assert torch.allclose(d_x, x.grad, rtol=1e-13, atol=1e-14) and torch.allclose(d_w, w.grad, rtol=1e-13, atol=1e-14)
+
+
 def test_residual_rmsnorm_against_autograd_of_the_composition():
     g = torch.Generator().manual_seed(12)
     B, H, eps = 9, 24, 1e-5
