@@ -155,18 +155,23 @@ def make_router(rng):
 def make_router_linear(rng):
     """Logits of the bias-free gate as exact sums: every product is a multiple of 2^-12 below 2^3 and a sum of 40 of
     them is exact in fp32 and fp64 alike, so an implementation that accumulates in fp32 must give the one rounding of
-    these values to its storage type, bit for bit."""
-    T, H, E = 12, 40, 6
+    these values to its storage type, bit for bit.  The same holds for the two gradients (sums of 6 and 16 products)."""
+    T, H, E = 16, 40, 6
     x = dyadic(rng, (T, H), 0.25)
     w = dyadic(rng, (E, H), 0.25)
+    d_logits = dyadic(rng, (T, E), 0.25)
     logits = np.zeros((T, E))
+    d_x = np.zeros((T, H))
+    d_w = np.zeros((E, H))
     for t in range(T):
         for e in range(E):
             acc = 0.0
             for h in range(H):
                 acc += x[t, h] * w[e, h]
+                d_x[t, h] += d_logits[t, e] * w[e, h]
+                d_w[e, h] += d_logits[t, e] * x[t, h]
             logits[t, e] = acc
-    np.savez(os.path.join(HERE, "router_linear.npz"), x=x, w=w, logits=logits)
+    np.savez(os.path.join(HERE, "router_linear.npz"), x=x, w=w, logits=logits, d_logits=d_logits, d_x=d_x, d_w=d_w)
 
 
 def make_residual_rmsnorm(rng):

@@ -25,7 +25,7 @@ def load(name):
 def test_fixture_inputs_are_exact_in_bfloat16():
     for name, keys in (("swiglu", ["gate", "up", "dy"]), ("rmsnorm", ["x", "w", "dy"]), ("embedding", ["table", "dy"]),
                        ("moe", ["x", "w_gate", "w_fc", "w_proj", "dy"]), ("router", ["logits", "d_weights"]),
-                       ("residual_rmsnorm", ["x", "r", "s", "w", "dy", "ds"]), ("router_linear", ["x", "w"]),
+                       ("residual_rmsnorm", ["x", "r", "s", "w", "dy", "ds"]), ("router_linear", ["x", "w", "d_logits"]),
                        ("moe_bias", ["x", "w_gate", "w_fc", "w_proj", "b_fc", "b_proj", "dy"])):
         f = load(name)
         for k in keys:
@@ -102,6 +102,8 @@ def test_oracle_router_linear_golden():
     # fp32 accumulation of these operands is exact: one rounding of the exact sums
     for dtype in (torch.bfloat16, torch.float16):
         assert torch.equal(O.router_linear(f["x"].to(dtype), f["w"].to(dtype)), f["logits"].to(dtype))
+    d_x, d_w = O.router_linear_backward(f["d_logits"], f["x"], f["w"], torch.float64)
+    assert torch.equal(d_x, f["d_x"]) and torch.equal(d_w, f["d_w"])
 
 
 def test_oracle_residual_rmsnorm_golden():
@@ -151,6 +153,16 @@ def test_hip_router_linear_golden(gpu, dtype):
     exp_w, exp_sel = O.router_topk_softmax(logits.cpu(), 2)
     assert torch.equal(selected.cpu(), exp_sel)
     assert_close(weights, exp_w, dtype, "weights")
+    # the gate's gradients for a given d_logits: exact sums again
+    from cute_kernels import _C
+    from cute_kernels.kernels.scattermoe.moe_hip import _GateLinear
+
+    xg, wg = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    d_logits = f["d_logits"].to(dtype).to(gpu)
+    assert _C.router_weight_grad_supported(d_logits, xg)
+    _GateLinear.apply(xg, wg).backward(d_logits)
+    assert torch.equal(wg.grad.cpu(), f["d_w"].to(dtype)), "d_w: exact sums, rounded once"
+    assert torch.equal(xg.grad.cpu(), f["d_x"].to(dtype)), "d_x: exact sums, rounded once"
 
 
 @pytest.mark.gpu
