@@ -116,13 +116,14 @@ def test_compiled_contiguous_count(gpu):
     assert torch.equal(out.cpu().long(), x.bincount(minlength=72))
 
 
+@pytest.mark.parametrize("E", [8, 24])  # the router as one forward launch / library linear with its own weight gradient
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_compiled_moe(gpu, dtype):
+def test_compiled_moe(gpu, dtype, E):
     from cute_kernels import MoE_Triton
     from test_gpu_moe import build_moe
 
-    announce("compiled moe", dtype)
-    T, H, I, E, k = 256, 256, 128, 8, 2
+    announce("compiled moe", dtype, E)
+    T, H, I, k = 256, 256, 128, 2
     x, w_gate, w_fc, w_proj, dy = O.moe_inputs(T, H, I, E, dtype, seed=81)
     moe = build_moe(MoE_Triton, gpu, dtype, E, k, H, I, w_gate, w_fc, w_proj)
     compiled = torch.compile(moe, fullgraph=True)
@@ -136,6 +137,7 @@ def test_compiled_moe(gpu, dtype):
     assert_close(xg.grad, expected["dx"], dtype, "dx")
     assert_close(moe.c_fc.weight.grad, expected["dw_fc"], dtype, "dw_fc")
     assert_close(moe.c_proj.weight.grad, expected["dw_proj"], dtype, "dw_proj")
+    assert_close(moe.gate.weight.grad, expected["dw_gate"], dtype, "dw_gate")
 
 
 class _Block(torch.nn.Module):
