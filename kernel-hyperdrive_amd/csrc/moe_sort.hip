@@ -119,11 +119,12 @@ __global__ void __launch_bounds__(kSortThreads)
 }
 
 // ---- the same sort spread over the GPU -----------------------------------------------------------
-// One workgroup sorts 16K ids in ~30 us but needs ~200 us for 100K: from kGridSortFrom ids on (and up to
-// 2^kGridSortMaxBits experts, one radix pass) the three kernels of ck_grid_sort.h take over.  Ids become the
+// One workgroup sorts 16K ids in ~37 us (the three launches below: 15) and needs ~200 us for 100K: from
+// kGridSortFrom ids on (and up to 2^kGridSortMaxBits experts, one radix pass) the three kernels of
+// ck_grid_sort.h take over.  Ids become the
 // keys, positions the values; the scatter kernel also derives the expert offsets from the scanned histogram
 // (the exclusive offset of bin e + 1 for the first wave = number of ids <= e).
-constexpr int64_t kGridSortFrom = 32768;
+constexpr int64_t kGridSortFrom = 16384;
 
 template <bool I32>
 struct ExpertIdLoader {

@@ -26,7 +26,7 @@ def test_contiguous_count(gpu, dtype, n, size):
 
 @pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
 @pytest.mark.parametrize("M,E", [(0, 8), (1, 1), (2, 8), (64, 2), (1000, 6), (16384, 8), (98304, 64), (5000, 72), (3000, 300), (70000, 1000),
-                                 (32768, 8), (32769, 3), (100000, 300), (40000, 512), (50000, 1), (131071, 65)])
+                                 (16383, 8), (16385, 5), (32768, 8), (32769, 3), (100000, 300), (40000, 512), (50000, 1), (131071, 65)])
 def test_moe_sort(gpu, dtype, M, E):
     from cute_kernels.kernels.scattermoe import moe_sort
 
