@@ -31,7 +31,9 @@ typedef enum {
     CK_ERR_NULL = 3,      /* required pointer is NULL */
     CK_ERR_WORKSPACE = 4, /* workspace smaller than the *_workspace_size query */
     CK_ERR_LAUNCH = 5,    /* hipGetLastError() reported a launch failure */
-    CK_ERR_ALIGN = 6      /* pointer not aligned to the element size */
+    CK_ERR_ALIGN = 6,     /* pointer not aligned to the element size */
+    CK_ERR_SCRATCH = 7,   /* problem too large for the library's built-in scratch buffer (ck_moe_sort_noalloc) */
+    CK_ERR_RUNTIME = 8    /* a HIP runtime query (current device, symbol address) failed */
 } ck_status;
 
 /* Human-readable text for a ck_status (host pointer to a static string). */
@@ -137,6 +139,19 @@ int64_t ck_moe_sort_workspace_size(int64_t M, int64_t E);
 int ck_moe_sort(const void* expert_ids, int ids_are_i32, int64_t* sorted_expert_idxs,
                 int64_t* sorted_scattered_idxs, int64_t* expert_offsets, void* workspace,
                 int64_t workspace_bytes, int64_t M, int64_t E, void* stream);
+
+/* ck_moe_sort for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference, which takes every buffer from torch's
+ * allocator.  Same arguments and results as ck_moe_sort, minus the workspace: that lives in a device array of
+ * CK_MOE_SORT_NOALLOC_SCRATCH_BYTES inside the library, one copy per GPU, held until the process ends.  The call
+ * makes no hipMalloc / hipFree and no allocating library call; the first call on a device looks the array's
+ * address up once.  (M, E) whose ck_moe_sort_workspace_size exceeds the array gives CK_ERR_SCRATCH and launches
+ * nothing (the limit is far away: 98304 ids of 64 experts need 48 KiB, a million ids of 512 experts 4 MiB).
+ * All calls on one GPU share the array: calls that overlap there (different streams or threads) race; calls
+ * ordered on one stream do not.  Nothing in the array has to be cleared between calls. */
+#define CK_MOE_SORT_NOALLOC_SCRATCH_BYTES (4 * 1024 * 1024)
+int ck_moe_sort_noalloc(const void* expert_ids, int ids_are_i32, int64_t* sorted_expert_idxs,
+                        int64_t* sorted_scattered_idxs, int64_t* expert_offsets, int64_t M, int64_t E, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Grouped GEMM with row gather / scatter ("scatter2scatter")

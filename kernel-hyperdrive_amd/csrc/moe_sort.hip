@@ -6,6 +6,8 @@
 //       (cute_kernels/kernels/scattermoe/triton_implementation/__init__.py:80-81), with ties kept in
 //       input order (stable), which torch's default sort does not promise
 //   - ck_offsets_from_sorted : cumsum(bincount) recovered from already-sorted ids.
+#include <mutex>
+
 #include "ck_block_sort.h"
 #include "ck_grid_sort.h"
 
@@ -230,15 +232,10 @@ extern "C" int64_t ck_moe_sort_workspace_size(int64_t M, int64_t E) {
     return ck::ck_sort_passes(ck::ck_key_bits(E)) > 1 ? 4 * M * (int64_t)sizeof(uint32_t) : 0;
 }
 
-extern "C" int ck_moe_sort(const void* expert_ids, int ids_are_i32, int64_t* sorted_expert_idxs,
-                           int64_t* sorted_scattered_idxs, int64_t* expert_offsets, void* workspace,
-                           int64_t workspace_bytes, int64_t M, int64_t E, void* stream) {
-    if (M < 0 || E <= 0 || M > 0x7fffffff || E > 0x7fffffff) return CK_ERR_SHAPE;
-    if (!expert_offsets) return CK_ERR_NULL;
-    if (M > 0 && (!expert_ids || !sorted_expert_idxs || !sorted_scattered_idxs)) return CK_ERR_NULL;
-    const int64_t need = ck_moe_sort_workspace_size(M, E);
-    if (need > 0 && (!workspace || workspace_bytes < need)) return CK_ERR_WORKSPACE;
-    hipStream_t s = (hipStream_t)stream;
+// The launches of ck_moe_sort; `workspace` holds ck_moe_sort_workspace_size(M, E) bytes (checked by the callers).
+static int moe_sort_launch(const void* expert_ids, int ids_are_i32, int64_t* sorted_expert_idxs,
+                           int64_t* sorted_scattered_idxs, int64_t* expert_offsets, void* workspace, int64_t M,
+                           int64_t E, hipStream_t s) {
     const int key_bits = ck::ck_key_bits(E);
     if (use_grid_sort(M, E)) {
         if (reinterpret_cast<uintptr_t>(workspace) & 3u) return CK_ERR_WORKSPACE;
@@ -273,6 +270,67 @@ extern "C" int ck_moe_sort(const void* expert_ids, int ids_are_i32, int64_t* sor
                            sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, (uint32_t*)workspace, (int)M,
                            (int)E, key_bits);
     return ck_launch_status();
+}
+
+static int moe_sort_check(const void* expert_ids, const int64_t* sorted_expert_idxs,
+                          const int64_t* sorted_scattered_idxs, const int64_t* expert_offsets, int64_t M, int64_t E) {
+    if (M < 0 || E <= 0 || M > 0x7fffffff || E > 0x7fffffff) return CK_ERR_SHAPE;
+    if (!expert_offsets) return CK_ERR_NULL;
+    if (M > 0 && (!expert_ids || !sorted_expert_idxs || !sorted_scattered_idxs)) return CK_ERR_NULL;
+    return CK_OK;
+}
+
+extern "C" int ck_moe_sort(const void* expert_ids, int ids_are_i32, int64_t* sorted_expert_idxs,
+                           int64_t* sorted_scattered_idxs, int64_t* expert_offsets, void* workspace,
+                           int64_t workspace_bytes, int64_t M, int64_t E, void* stream) {
+    const int bad = moe_sort_check(expert_ids, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, M, E);
+    if (bad) return bad;
+    const int64_t need = ck_moe_sort_workspace_size(M, E);
+    if (need > 0 && (!workspace || workspace_bytes < need)) return CK_ERR_WORKSPACE;
+    return moe_sort_launch(expert_ids, ids_are_i32, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets,
+                           workspace, M, E, (hipStream_t)stream);
+}
+
+// ---- the same sort for callers that cannot allocate -----------------------------------------------
+// The workspace of ck_moe_sort (the grid-wide sort's [bins][waves] histogram, or the key / value ping-pong
+// arrays of a multi-pass single-workgroup sort) lives in this file-scope device array instead of a buffer the
+// caller brings.  Every GPU the library runs on holds its own copy until the process ends.  In host code the
+// array's name is only a handle for hipGetSymbolAddress: the kernels get the address that call returns for
+// the current device, kept per device below.  Nothing in it has to start at zero (the histogram kernel writes
+// every entry the scan reads, a radix pass writes every pair the next one reads), so no clearing is needed;
+// two calls that overlap on one GPU (different streams) would share it and race.
+static __device__ __align__(256) unsigned char scratch[CK_MOE_SORT_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+int scratch_for_current_device(void** out) {
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return CK_ERR_RUNTIME;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[device]) {
+        void* ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return CK_ERR_RUNTIME;
+        g_scratch_ptr[device] = ptr;
+    }
+    *out = g_scratch_ptr[device];
+    return CK_OK;
+}
+}  // namespace
+
+extern "C" int ck_moe_sort_noalloc(const void* expert_ids, int ids_are_i32, int64_t* sorted_expert_idxs,
+                                   int64_t* sorted_scattered_idxs, int64_t* expert_offsets, int64_t M, int64_t E,
+                                   void* stream) {
+    const int bad = moe_sort_check(expert_ids, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, M, E);
+    if (bad) return bad;
+    if (ck_moe_sort_workspace_size(M, E) > (int64_t)CK_MOE_SORT_NOALLOC_SCRATCH_BYTES) return CK_ERR_SCRATCH;
+    void* ptr = nullptr;
+    const int status = scratch_for_current_device(&ptr);
+    if (status) return status;
+    return moe_sort_launch(expert_ids, ids_are_i32, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, ptr, M,
+                           E, (hipStream_t)stream);
 }
 
 extern "C" int ck_offsets_from_sorted(const int64_t* sorted_expert_idxs, int64_t* expert_offsets, int64_t M, int64_t E,

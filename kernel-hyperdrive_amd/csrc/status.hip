@@ -10,8 +10,10 @@ extern "C" const char* ck_status_string(int status) {
         case CK_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
         case CK_ERR_LAUNCH: return "kernel launch failed";
         case CK_ERR_ALIGN: return "pointer not aligned to its element size";
+        case CK_ERR_SCRATCH: return "problem too large for the library's built-in scratch buffer";
+        case CK_ERR_RUNTIME: return "HIP runtime query failed";
         default: return "unknown status";
     }
 }
 
-extern "C" int ck_abi_version(void) { return 1; }
+extern "C" int ck_abi_version(void) { return 2; }

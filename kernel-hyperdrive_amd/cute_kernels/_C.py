@@ -19,7 +19,7 @@ import torch
 _LIB_PATH = os.environ.get("CUTE_HIP_LIBRARY") or os.path.join(
     os.path.dirname(os.path.abspath(__file__)), "lib", "libcute_hip.so"
 )
-_ABI_VERSION = 1
+_ABI_VERSION = 2
 
 _lib = None
 _lock = threading.Lock()
@@ -52,6 +52,7 @@ _SIGNATURES = {
     "ck_contiguous_count": (_i32, [_p, _i32, _p, _i64, _i64, _p]),
     "ck_moe_sort_workspace_size": (_i64, [_i64, _i64]),
     "ck_moe_sort": (_i32, [_p, _i32, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
+    "ck_moe_sort_noalloc": (_i32, [_p, _i32, _p, _p, _p, _i64, _i64, _p]),
     "ck_scatter2scatter": (
         _i32,
         [_p, _i64, _p, _i64, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _p],
@@ -376,6 +377,22 @@ def moe_sort(expert_ids, sorted_expert_idxs, sorted_scattered_idxs, expert_offse
                             0 if workspace is None else workspace.numel() * workspace.element_size(),
                             expert_ids.numel(), E, L.stream),
             "ck_moe_sort",
+        )
+
+
+MOE_SORT_NOALLOC_SCRATCH_BYTES = 4 * 1024 * 1024
+
+
+def moe_sort_noalloc(expert_ids, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, E: int) -> None:
+    """``moe_sort`` with the workspace inside the library (a fixed device array per GPU): for callers that must
+    not allocate.  Calls that overlap on one GPU share that array and race."""
+    lib = load_library()
+    with _Launch(expert_ids, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets) as L:
+        _check(
+            lib.ck_moe_sort_noalloc(_ptr(expert_ids), _ids_are_i32(expert_ids), _ptr(sorted_expert_idxs),
+                                    _ptr(sorted_scattered_idxs), _ptr(expert_offsets), expert_ids.numel(), E,
+                                    L.stream),
+            "ck_moe_sort_noalloc",
         )
 
 

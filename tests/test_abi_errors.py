@@ -9,7 +9,7 @@ import ctypes
 
 import pytest
 
-OK, DTYPE, SHAPE, NULL, WORKSPACE, LAUNCH, ALIGN = range(7)
+OK, DTYPE, SHAPE, NULL, WORKSPACE, LAUNCH, ALIGN, SCRATCH, RUNTIME = range(9)
 F32, F16, BF16 = 0, 1, 2
 P = 0x10000  # a well-aligned non-null "device pointer"; no call below gets as far as using it
 
@@ -22,8 +22,8 @@ def lib():
 
 
 def test_status_strings(lib):
-    texts = [lib.ck_status_string(i) for i in range(7)]
-    assert texts[0] == b"ok" and len(set(texts)) == 7
+    texts = [lib.ck_status_string(i) for i in range(9)]
+    assert texts[0] == b"ok" and len(set(texts)) == 9
     assert lib.ck_status_string(99)  # unknown codes still give a string
 
 
@@ -92,6 +92,13 @@ def test_routing_argument_checks(lib):
     need = lib.ck_moe_sort_workspace_size(1000, 1000)
     assert need > 0
     assert lib.ck_moe_sort(P, 0, P, P, P, P, need - 1, 1000, 1000, None) == WORKSPACE
+    # the variant with the workspace inside the library: same argument checks, and a size limit instead of a workspace
+    assert lib.ck_moe_sort_noalloc(P, 0, P, P, P, 10, 0, None) == SHAPE
+    assert lib.ck_moe_sort_noalloc(P, 0, P, P, None, 10, 8, None) == NULL
+    limit = 4 * 1024 * 1024
+    assert lib.ck_moe_sort_workspace_size(1 << 20, 512) == limit  # a million ids of 512 experts just fit
+    assert lib.ck_moe_sort_workspace_size((1 << 20) + 1, 512) > limit
+    assert lib.ck_moe_sort_noalloc(P, 0, P, P, P, (1 << 20) + 1, 512, None) == SCRATCH
     assert lib.ck_offsets_from_sorted(None, P, 4, 8, None) == NULL
     assert lib.ck_offsets_from_sorted(P, P, 4, 0, None) == SHAPE
 

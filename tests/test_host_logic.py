@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"{name} is declared in include/cute_hip.h but not exported"
     assert sorted(_C.EXPORTED_SYMBOLS) == declared, "the ctypes binding and the header must list the same functions"
-    assert lib.ck_abi_version() == 1
+    assert lib.ck_abi_version() == 2
     assert lib.ck_status_string(0) == b"ok"
     assert b"workspace" in lib.ck_status_string(4)
 
