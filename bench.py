@@ -9,7 +9,9 @@ timed region.  Prints ONE JSON line:
                activation and gate mixing are inside the timed region but not in the flop count
   roofline     the grouped GEMM (6 launches per step: forward, dX and dW of c_fc and c_proj), timed inside the
                timed region with GPU events on the launch stream, against the 2.5 PFLOP/s dense bf16 MFMA peak
-  cpu_baseline the oracle's torch restatement of the reference layer on the host cores, on a bounded sample
+  cpu_baseline the oracle's torch restatement of the reference layer on the host cores, on a bounded sample of the
+               same workload (T=512 of the 8192 tokens), plus BASELINE configs[0] exactly (T=1024, H=512, I=1024,
+               fp32, 3 warm-up and 10 timed runs, median) under "c1"
   extras       HBM GB/s of SwiGLU, RMSNorm and embedding at their BASELINE shapes (buffers rotated so that the
                256 MB last-level cache cannot serve them), and the step of the fine-grained skewed MoE
                configuration (configs[4]: T=16384 H=2048 I=1408 E=64 top-6, Zipf(1.2) expert popularity)
@@ -30,11 +32,22 @@ import torch  # noqa: E402
 
 BF16_MFMA_PEAK_TFLOPS = 2500.0
 HBM_PEAK_GBS = 8000.0
-# HBM-side bytes per grouped-GEMM launch at the Mixtral shape, from two rocprofv3 --pmc runs of this file
+# HBM-side bytes per grouped-GEMM launch at the Mixtral shape come from two rocprofv3 --pmc runs of this file
 # (FETCH_SIZE, then WRITE_SIZE, each scaled by what the same counter reads for the 1 GiB copies of
-# --copy-calibration): 38.2 GB read + 5.6 GB written per step over 6 products.  Summary:
-# profiles/grouped_gemm_hbm_traffic_moe_mixtral_bf16.txt
-GEMM_HBM_BYTES_PER_LAUNCH = 7.29e9
+# --copy-calibration); the committed summary of those runs ends with a line "roofline.traffic = <bytes>".
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "grouped_gemm_hbm_traffic_moe_mixtral_bf16.txt")
+
+
+def gemm_hbm_bytes_per_launch():
+    """The figure of the committed counter summary (None when the summary is missing or has no such line)."""
+    import re
+
+    try:
+        with open(TRAFFIC_SUMMARY) as f:
+            found = re.findall(r"^roofline\.traffic\s*=\s*([0-9.eE+]+)", f.read(), flags=re.M)
+    except OSError:
+        return None
+    return float(found[-1]) if found else None
 
 
 def parse_args():
@@ -46,7 +59,6 @@ def parse_args():
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     p.add_argument("--only-extras", action="store_true", help="only the HBM-bound ops (for profiling them)")
     p.add_argument("--tokens", type=int, default=8192, help="T of the MoE workload (default: the BASELINE shape)")
-    p.add_argument("--no-ceiling", action="store_true", help="skip the sustained-MFMA-rate probe")
     p.add_argument("--copy-calibration", action="store_true",
                    help="also run three 1 GiB device copies before the steps (a kernel of known HBM traffic, to scale "
                         "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -116,7 +128,8 @@ def bench_moe(device, args):
         "peak": BF16_MFMA_PEAK_TFLOPS,
         "unit": "TFLOP/s",
         "frac": round(achieved / BF16_MFMA_PEAK_TFLOPS, 4),
-        "traffic": GEMM_HBM_BYTES_PER_LAUNCH if (T, H, I, E, k) == (8192, 4096, 14336, 8, 2) else None,
+        "traffic": gemm_hbm_bytes_per_launch() if (T, H, I, E, k) == (8192, 4096, 14336, 8, 2) else None,
+        "traffic_source": "profiles/grouped_gemm_hbm_traffic_moe_mixtral_bf16.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)",
         "launches_per_step": launches // args.steps,
         "avg_launch_ms": round(gemm_ms / max(launches, 1), 4),
         "gemm_ms_per_step": round(gemm_ms / args.steps, 3),
@@ -132,35 +145,6 @@ def bench_moe(device, args):
     del moe, x, dy
     torch.cuda.empty_cache()
     return result, roofline, config
-
-
-def mfma_ceiling(device):
-    """TFLOP/s of back-to-back bf16 MFMAs on register operands: all-zero data, then random data (which draws
-    more power and so runs at a lower clock).  The second figure bounds any bf16 GEMM on real data here."""
-    from cute_kernels import _C
-
-    out = {}
-    sink = torch.zeros(1, device=device, dtype=torch.float32)
-    blocks, iters = 256, 20000
-    flop = blocks * 8 * iters * 32 * 32768.0
-    g = torch.Generator(device=device).manual_seed(0)
-    for label in ("zeros", "random"):
-        if label == "zeros":
-            ops = torch.zeros(24 * 512 * 8, device=device, dtype=torch.bfloat16)
-        else:
-            ops = torch.randn(24 * 512 * 8, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
-        best = None
-        for _ in range(3):
-            start = torch.cuda.Event(enable_timing=True)
-            end = torch.cuda.Event(enable_timing=True)
-            start.record()
-            _C.probe_mfma(ops, iters, blocks, sink)
-            end.record()
-            torch.cuda.synchronize()
-            ms = start.elapsed_time(end)
-            best = ms if best is None else min(best, ms)
-        out[label] = round(flop / (best * 1e-3) / 1e12, 1)
-    return out
 
 
 def copy_calibration(device):
@@ -294,9 +278,12 @@ def bench_extras(device):
     dys = [torch.randn(8, 4096, H, device=device, dtype=dtype) for _ in range(2)]
     for label, ids in (("uniform", torch.randint(0, V, (8, 4096), generator=torch.Generator().manual_seed(0))),
                        ("zipf", zipf_ids((8, 4096), V, 1.1, seed=0))):
+        # distinct table rows: a row that several ids select is read from HBM once and from the caches after that
+        distinct = int(torch.unique(ids).numel())
         ids = ids.to(device)
         ms = _time_rotating(lambda i: EM._forward(input_ids=ids, weight=table, kernel_backend=hip, BLOCK_SIZE_B=4, BLOCK_SIZE_H=512), 1)
-        out[f"embedding_fwd_{label}"] = gbs(2 * n * H * 2 + 8 * n, ms)
+        out[f"embedding_fwd_{label}"] = gbs((distinct + n) * H * 2 + 8 * n, ms)
+        out[f"embedding_fwd_{label}"]["distinct_rows"] = distinct
         ms = _time_rotating(lambda i: EM._backward(input_ids=ids, weight=table, output_grad=dys[i % 2], kernel_backend=hip,
                                                    BLOCK_SIZE_B=4, BLOCK_SIZE_H=512), 2, iters=10)
         out[f"embedding_bwd_{label}"] = gbs(n * H * 2 + V * H * 2 + 8 * n, ms)
@@ -308,36 +295,60 @@ def bench_extras(device):
 
 
 # ---- CPU baseline -----------------------------------------------------------------------------------------
-def bench_cpu():
-    """The oracle's restatement of the reference torch layer, fp32, on the host cores: the Mixtral shape with
-    T=512 of the 8192 tokens (same H, I, E, k).  About 1.1e12 flop per step."""
+def _cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def _cpu_moe(T, H, I, E, k, warmup, runs, budget_s):
+    """Median seconds of the oracle's fp32 layer forward + backward on the host, and the number of timed runs."""
     from oracle import cute_oracle as O
 
-    threads = min(os.cpu_count() or 1, 16)
-    torch.set_num_threads(threads)
-    T, H, I, E, k = 512, 4096, 14336, 8, 2
     g = torch.Generator().manual_seed(0)
     x = torch.randn(T, H, generator=g)
     w_gate = torch.randn(E, H, generator=g) * 0.02
     w_fc = torch.empty(E, 2 * I, H).normal_(0, 0.02, generator=g)
     w_proj = torch.empty(E, H, I).normal_(0, 0.02, generator=g)
     dy = torch.randn(T, H, generator=g)
-    flop = 18.0 * T * k * H * I
-    O.moe_forward_backward(x, w_gate, w_fc, w_proj, dy, k)  # warm-up
+    for _ in range(warmup):
+        O.moe_forward_backward(x, w_gate, w_fc, w_proj, dy, k)
     times = []
     t_start = time.perf_counter()
-    while len(times) < 5 and time.perf_counter() - t_start < 20.0:
+    while len(times) < runs and (time.perf_counter() - t_start < budget_s or not times):
         t0 = time.perf_counter()
         O.moe_forward_backward(x, w_gate, w_fc, w_proj, dy, k)
         times.append(time.perf_counter() - t0)
-    best = sorted(times)[len(times) // 2]
+    return sorted(times)[len(times) // 2], len(times)
+
+
+def bench_cpu():
+    """The oracle's restatement of the reference torch layer, fp32, on the host cores.  `value`: the Mixtral shape
+    with T=512 of the 8192 tokens (same H, I, E, k; about 1.1e12 flop per step).  `c1`: BASELINE configs[0] as
+    stated (T=1024, H=512, I=1024, E=8, top-2; 3 warm-up and 10 timed runs, median).  Threads: the CPU share of a
+    one-GPU box (OMP_NUM_THREADS as exported there, 16), not os.cpu_count(), which counts every core of the host."""
+    threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16") or 16))
+    torch.set_num_threads(threads)
+    T, H, I, E, k = 512, 4096, 14336, 8, 2
+    best, runs = _cpu_moe(T, H, I, E, k, warmup=1, runs=5, budget_s=20.0)
+    flop = 18.0 * T * k * H * I
+    c1_t, c1_runs = _cpu_moe(1024, 512, 1024, 8, 2, warmup=3, runs=10, budget_s=30.0)
+    c1_flop = 18.0 * 1024 * 2 * 512 * 1024
     return {
         "value": round(flop / best / 1e12, 4),
         "unit": "TFLOP/s",
         "cores": threads,
         "kind": "port",
         "sample": f"Mixtral shape with T={T} of 8192 tokens (H={H} I={I} E={E} top-{k}), fp32 fwd+bwd, "
-                  f"median of {len(times)} runs, {best * 1e3:.0f} ms each; torch {torch.__version__}",
+                  f"median of {runs} runs, {best * 1e3:.0f} ms each; torch {torch.__version__}",
+        "c1": {"value": round(c1_flop / c1_t / 1e12, 4), "unit": "TFLOP/s", "ms": round(c1_t * 1e3, 2), "runs": c1_runs,
+               "warmup": 3, "config": "BASELINE configs[0]: T=1024 H=512 I=1024 E=8 top-2, fp32 fwd+bwd, median"},
+        "host": {"cpu_model": _cpu_model(), "os_cpu_count": os.cpu_count(), "torch_threads": torch.get_num_threads()},
     }
 
 
@@ -373,8 +384,6 @@ def main():
         "frac_of_mfma_peak": result["frac_of_mfma_peak"],
         "roofline": roofline,
     }
-    if not args.no_ceiling:
-        line["sustained_mfma_tflops"] = mfma_ceiling(device)
     if not args.no_extras:
         line["extras"] = bench_extras(device)
     if not args.no_cpu:

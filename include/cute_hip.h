@@ -318,15 +318,6 @@ int ck_expert_bias_forward(void* y, int64_t y_stride, const void* bias, int64_t 
 int ck_expert_bias_backward(const void* dy, int64_t dy_stride, const int64_t* expert_offsets, void* d_bias,
                             int64_t d_bias_stride, int64_t num_rows, int64_t N, int64_t E, int dtype, void* stream);
 
-/* ---------------------------------------------------------------------------------------------
- * Measurement aid with no counterpart in the reference: back-to-back v_mfma_f32_32x32x16_bf16 on operands
- * held in registers (the register footprint of the grouped GEMM's inner loop, no LDS or memory traffic), to
- * read off the rate the matrix cores sustain on given data under the part's power limit.
- *   operands : 24 * 512 * 16 bytes of bf16 values (device), sink: one float (device)
- *   work     : blocks * 8 waves * iters * 32 MFMAs of 32768 flop; the caller times the launch
- * ------------------------------------------------------------------------------------------- */
-int ck_probe_mfma(const void* operands, int64_t iters, int blocks, float* sink, void* stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -77,6 +77,7 @@ struct GemmParams {
 };
 
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
 // Expert tile lookup: row tile `mt` (counted over all experts, each expert's rows cut into BM-row tiles)
 // -> expert, first row, valid rows.  Executed by the first wave; result broadcast through LDS.
@@ -651,6 +652,18 @@ __device__ __forceinline__ uint64_t opaque_s64(uint64_t v) {  // same for a wave
     return v;
 }
 
+// two fp32 values rounded to the storage type (round to nearest even) and packed into one dword, first value low
+template <typename T>
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+    typedef typename T::storage_t S2 __attribute__((ext_vector_type(2)));
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t f = {a, b};
+    const S2 h = __builtin_convertvector(f, S2);
+    uint32_t w;
+    __builtin_memcpy(&w, &h, 4);
+    return w;
+}
+
 // MODE 0: one workgroup per tile.  MODE 1: tiles dealt by find_tile_split; a workgroup with a piece of a tile writes its
 // fp32 accumulators to p.partials instead of running the epilogue.  MODE 2: the launch that follows MODE 1 - one
 // workgroup per split tile adds the pieces up and runs the epilogue.
@@ -1106,10 +1119,10 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
         for (int j = 0; j < TN; ++j) {
             const int row = wm * RW + (i % TH) * 16 + lane % 16;  // inside this half of the tile
             const int col = (j / TNH) * (BN / 2) + wn * CW + (j % TNH) * 16 + 4 * (lane / 16);
-            VPack<T, 4> four;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) four.v[r] = T::down(acc[i][j][r]);
-            *reinterpret_cast<VPack<T, 4>*>(Ch + row * C_LD + col) = four;
+            u32x2_t four;
+            four.x = pack2<T>(acc[i][j][0], acc[i][j][1]);
+            four.y = pack2<T>(acc[i][j][2], acc[i][j][3]);
+            *reinterpret_cast<u32x2_t*>(Ch + row * C_LD + col) = four;
         }
     }
     S* Cbase = reinterpret_cast<S*>(p.C) + (GROUP_K ? (int64_t)expert * p.c_stride_e : 0);

@@ -153,7 +153,7 @@ __global__ void __launch_bounds__(NW * CK_WAVE)
         for (int u = 0; u < U; ++u) {
             const int k0 = (kb + NW * u) * 32;
             in[u] = k0 <= k_last;
-            const int kl = in[u] ? k0 : 0;
+            const int kl = in[u] ? k0 : -kc * 8;  // the row's first packet (xrow / wrow point kc packets into the row)
             a[u] = nt_load(reinterpret_cast<const frag_t*>(xrow + kl));
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) b[u][nt] = *reinterpret_cast<const frag_t*>(wrow[nt] + kl);

@@ -83,7 +83,6 @@ _SIGNATURES = {
     "ck_router_forward": (_i32, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _i32, _p]),
     "ck_router_weight_grad_workspace_size": (_i64, [_i64, _i64, _i64]),
     "ck_router_weight_grad": (_i32, [_p, _p, _i64, _p, _i64, _p, _i64, _i64, _i64, _i64, _i32, _p]),
-    "ck_probe_mfma": (_i32, [_p, _i64, _i32, _p, _p]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
@@ -211,6 +210,28 @@ def _ids_are_i32(ids: torch.Tensor) -> int:
     raise ValueError(f"index tensor must be int32 or int64, got {ids.dtype}")
 
 
+def _index_i64(t: torch.Tensor, name: str) -> torch.Tensor:
+    """An index tensor as the kernels read it: int64, dense.  The reference's Triton kernels take any integer type
+    (they load through typed pointers); the native entry points read int64, so other integer types are converted
+    here and anything else is refused - read as int64, an int32 tensor would be twice as long as it is."""
+    if t.dtype == torch.int64:
+        return t if t.is_contiguous() else t.contiguous()
+    if t.dtype in (torch.int32, torch.int16, torch.int8, torch.uint8):
+        return t.to(torch.int64).contiguous()
+    raise ValueError(f"{name} must be an integer tensor, got {t.dtype}")
+
+
+def _index_i64_out(t: torch.Tensor, name: str) -> None:
+    if t.dtype != torch.int64 or not t.is_contiguous():
+        raise ValueError(f"{name} is written as dense int64; got {t.dtype}, strides {tuple(t.stride())}")
+
+
+def _same_dtype(ref: torch.Tensor, what: str, **others: torch.Tensor) -> None:
+    for name, t in others.items():
+        if t is not None and t.dtype != ref.dtype:
+            raise ValueError(f"{what}: {name} is {t.dtype}, expected {ref.dtype} like the first operand")
+
+
 # ---- one Python function per C entry point ----------------------------------------------------------
 # All tensors must be contiguous unless a stride is passed explicitly.
 
@@ -280,6 +301,7 @@ def swiglu_unchunked_backward(x, output_grad, x_grad, block_size: int) -> None:
 
 def rmsnorm_forward(x, weight, output, rstd, eps: float) -> None:
     lib = load_library()
+    _same_dtype(x, "rmsnorm_forward", weight=weight, output=output)
     H = x.size(-1)
     B = x.numel() // H if H > 0 else 0
     with _Launch(x, weight, output, rstd) as L:
@@ -316,6 +338,7 @@ def rmsnorm_backward_workspace_size(B: int, H: int, device: torch.device) -> int
 
 def rmsnorm_backward(x, weight, output_grad, rstd, x_grad, weight_grad, workspace, eps: float) -> None:
     lib = load_library()
+    _same_dtype(x, "rmsnorm_backward", weight=weight, output_grad=output_grad, x_grad=x_grad, weight_grad=weight_grad)
     H = x.size(-1)
     B = x.numel() // H if H > 0 else 0
     with _Launch(x, weight, output_grad, rstd, x_grad, weight_grad, workspace) as L:
@@ -357,6 +380,10 @@ def embedding_backward(input_ids, output_grad, weight_grad, workspace) -> None:
 
 def contiguous_count(x, output, size: int) -> None:
     lib = load_library()
+    if output.dtype != torch.int32 or not output.is_contiguous() or output.numel() != size:
+        raise ValueError("contiguous_count writes a dense int32 tensor of `size` counts")
+    if not x.is_contiguous():
+        x = x.contiguous()
     with _Launch(x, output) as L:
         _check(
             lib.ck_contiguous_count(_ptr(x), _ids_are_i32(x), _ptr(output), x.numel(), size, L.stream),
@@ -370,6 +397,15 @@ def moe_sort_workspace_size(M: int, E: int) -> int:
 
 def moe_sort(expert_ids, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, workspace, E: int) -> None:
     lib = load_library()
+    if not expert_ids.is_contiguous():
+        expert_ids = expert_ids.contiguous()
+    for name, t in (("sorted_expert_idxs", sorted_expert_idxs), ("sorted_scattered_idxs", sorted_scattered_idxs),
+                    ("expert_offsets", expert_offsets)):
+        _index_i64_out(t, name)
+    if sorted_expert_idxs.numel() != expert_ids.numel() or sorted_scattered_idxs.numel() != expert_ids.numel():
+        raise ValueError("moe_sort: one sorted id and one position per expert id")
+    if expert_offsets.numel() != E:
+        raise ValueError("moe_sort: one offset per expert")
     with _Launch(expert_ids, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, workspace) as L:
         _check(
             lib.ck_moe_sort(_ptr(expert_ids), _ids_are_i32(expert_ids), _ptr(sorted_expert_idxs),
@@ -387,6 +423,15 @@ def moe_sort_noalloc(expert_ids, sorted_expert_idxs, sorted_scattered_idxs, expe
     """``moe_sort`` with the workspace inside the library (a fixed device array per GPU): for callers that must
     not allocate.  Calls that overlap on one GPU share that array and race."""
     lib = load_library()
+    if not expert_ids.is_contiguous():
+        expert_ids = expert_ids.contiguous()
+    for name, t in (("sorted_expert_idxs", sorted_expert_idxs), ("sorted_scattered_idxs", sorted_scattered_idxs),
+                    ("expert_offsets", expert_offsets)):
+        _index_i64_out(t, name)
+    if sorted_expert_idxs.numel() != expert_ids.numel() or sorted_scattered_idxs.numel() != expert_ids.numel():
+        raise ValueError("moe_sort: one sorted id and one position per expert id")
+    if expert_offsets.numel() != E:
+        raise ValueError("moe_sort: one offset per expert")
     with _Launch(expert_ids, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets) as L:
         _check(
             lib.ck_moe_sort_noalloc(_ptr(expert_ids), _ids_are_i32(expert_ids), _ptr(sorted_expert_idxs),
@@ -398,6 +443,8 @@ def moe_sort_noalloc(expert_ids, sorted_expert_idxs, sorted_scattered_idxs, expe
 
 def offsets_from_sorted(sorted_expert_idxs, expert_offsets) -> None:
     lib = load_library()
+    sorted_expert_idxs = _index_i64(sorted_expert_idxs, "sorted_expert_idxs")
+    _index_i64_out(expert_offsets, "expert_offsets")
     with _Launch(sorted_expert_idxs, expert_offsets) as L:
         _check(
             lib.ck_offsets_from_sorted(_ptr(sorted_expert_idxs), _ptr(expert_offsets), sorted_expert_idxs.numel(),
@@ -418,6 +465,12 @@ def scatter2scatter(X, W, sorted_scattered_idxs, expert_offsets, out, fan_out: i
     lib = load_library()
     if X.stride(1) != 1 or out.stride(1) != 1:
         raise ValueError("scatter2scatter needs unit column stride for X and out")
+    _same_dtype(X, "scatter2scatter", W=W, out=out)
+    if sorted_scattered_idxs is not None:
+        sorted_scattered_idxs = _index_i64(sorted_scattered_idxs, "sorted_scattered_idxs")
+    expert_offsets = _index_i64(expert_offsets, "expert_offsets")
+    if expert_offsets.numel() != W.size(0):
+        raise ValueError("scatter2scatter: one expert offset per expert of W")
     flop = 2.0 * out.size(0) * X.size(1) * out.size(1)
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     with _Launch(X, W, sorted_scattered_idxs, expert_offsets, out, workspace) as L, _Timed("scatter2scatter", flop):
@@ -437,6 +490,12 @@ def scatter2scatter_glu(X, W, sorted_scattered_idxs, expert_offsets, h, act, fan
         raise ValueError("scatter2scatter_glu needs unit column stride for X, h and act")
     if h.size(1) != 2 * act.size(1) or h.size(0) != act.size(0):
         raise ValueError("scatter2scatter_glu: h must be [slots, 2I] and act [slots, I]")
+    _same_dtype(X, "scatter2scatter_glu", W=W, h=h, act=act)
+    if sorted_scattered_idxs is not None:
+        sorted_scattered_idxs = _index_i64(sorted_scattered_idxs, "sorted_scattered_idxs")
+    expert_offsets = _index_i64(expert_offsets, "expert_offsets")
+    if expert_offsets.numel() != W.size(0):
+        raise ValueError("scatter2scatter_glu: one expert offset per expert of W")
     flop = 2.0 * h.size(0) * X.size(1) * h.size(1)
     with _Launch(X, W, sorted_scattered_idxs, expert_offsets, h, act) as L, _Timed("scatter2scatter", flop):
         _check(
@@ -455,6 +514,10 @@ def scatter2scatter_glu_bwd(DY, W, expert_offsets, h, d_h) -> None:
         raise ValueError("scatter2scatter_glu_bwd needs unit column stride for DY, h and d_h")
     if h.shape != d_h.shape or h.size(1) != 2 * W.size(2) or h.size(0) != DY.size(0):
         raise ValueError("scatter2scatter_glu_bwd: h and d_h must be [slots, 2I] for W [E, K, I]")
+    _same_dtype(DY, "scatter2scatter_glu_bwd", W=W, h=h, d_h=d_h)
+    expert_offsets = _index_i64(expert_offsets, "expert_offsets")
+    if expert_offsets.numel() != W.size(0):
+        raise ValueError("scatter2scatter_glu_bwd: one expert offset per expert of W")
     flop = 2.0 * DY.size(0) * DY.size(1) * W.size(2)
     with _Launch(DY, W, expert_offsets, h, d_h) as L, _Timed("scatter2scatter", flop):
         _check(
@@ -469,6 +532,10 @@ def group_bwd_W(DY, X, expert_offsets, DW, E: int) -> None:
     lib = load_library()
     if X.stride(1) != 1 or DY.stride(1) != 1:
         raise ValueError("group_bwd_W needs unit column stride for X and DY")
+    _same_dtype(X, "group_bwd_W", DY=DY, DW=DW)
+    expert_offsets = _index_i64(expert_offsets, "expert_offsets")
+    if expert_offsets.numel() != E or DW.size(0) != E:
+        raise ValueError("group_bwd_W: one expert offset and one DW block per expert")
     flop = 2.0 * X.size(0) * X.size(1) * DY.size(1)
     with _Launch(DY, X, expert_offsets, DW) as L, _Timed("group_bwd_W", flop):
         _check(
@@ -483,6 +550,10 @@ def group(A, idx, coeff, out, fan_out: int) -> None:
     lib = load_library()
     if A.stride(1) != 1 or out.stride(1) != 1:
         raise ValueError("group needs unit column stride for A and out")
+    _same_dtype(A, "group", coeff=coeff, out=out)
+    idx = _index_i64(idx, "the row index")
+    if coeff is not None and not coeff.is_contiguous():
+        coeff = coeff.contiguous()
     with _Launch(A, idx, coeff, out) as L:
         _check(
             lib.ck_group(_ptr(A), A.stride(0), _ptr(idx), _ptr(coeff), _ptr(out), out.stride(0), idx.numel(),
@@ -495,6 +566,7 @@ def moe_combine_forward(expanded, gates, out) -> None:
     """expanded [T, k, H], gates [T, k] (or None: plain sum over the k slots), out [T, H]; all dense."""
     lib = load_library()
     T, k, H = expanded.shape
+    _same_dtype(expanded, "moe_combine_forward", gates=gates, out=out)
     with _Launch(expanded, gates, out) as L:
         _check(
             lib.ck_moe_combine_forward(_ptr(expanded), _ptr(gates), _ptr(out), T, k, H, dtype_code(expanded.dtype),
@@ -507,6 +579,7 @@ def moe_combine_backward_gates(expanded, grad_out, d_gates) -> None:
     """expanded [T, k, H], grad_out [T, H], d_gates [T, k]; all dense."""
     lib = load_library()
     T, k, H = expanded.shape
+    _same_dtype(expanded, "moe_combine_backward_gates", grad_out=grad_out, d_gates=d_gates)
     with _Launch(expanded, grad_out, d_gates) as L:
         _check(
             lib.ck_moe_combine_backward_gates(_ptr(expanded), _ptr(grad_out), _ptr(d_gates), T, k, H,
@@ -677,13 +750,3 @@ def router_topk_softmax_backward(d_weights, weights_f32, selected, d_logits) -> 
                                                 d_logits.stride(0), T, E, k, dtype_code(d_logits.dtype), L.stream),
             "ck_router_topk_softmax_backward",
         )
-
-
-def probe_mfma(operands, iters: int, blocks: int, sink) -> None:
-    """Measurement aid: `blocks` workgroups of 8 waves issue `iters` * 32 MFMAs each on `operands` (uint8/any
-    tensor of at least 24 * 512 * 16 bytes, device); `sink` is a one-element float32 device tensor."""
-    lib = load_library()
-    if operands.numel() * operands.element_size() < 24 * 512 * 16:
-        raise ValueError("operands must hold at least 24 * 512 * 16 bytes")
-    with _Launch(operands, sink) as L:
-        _check(lib.ck_probe_mfma(_ptr(operands), iters, blocks, _ptr(sink), L.stream), "ck_probe_mfma")

@@ -19,7 +19,7 @@ CSRC_DIR = os.path.normpath(os.path.join(PACKAGE_DIR, "..", "csrc"))
 LIB_DIR = os.path.join(PACKAGE_DIR, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libcute_hip.so")
 
-SOURCES = ["status.hip", "add.hip", "swiglu.hip", "rmsnorm.hip", "embedding.hip", "moe_sort.hip", "moe_combine.hip", "expert_bias.hip", "router.hip", "grouped_gemm.hip", "probe.hip"]
+SOURCES = ["status.hip", "add.hip", "swiglu.hip", "rmsnorm.hip", "embedding.hip", "moe_sort.hip", "moe_combine.hip", "expert_bias.hip", "router.hip", "grouped_gemm.hip"]
 
 # -packed-fp32-ops off: the packed fp32 VALU forms are not wanted in any kernel of this library
 HIPCC_FLAGS = [

@@ -213,8 +213,6 @@ def test_grouped_gemm_argument_checks(lib):
     assert wgrad(P, P, 64, P, 64, P, 16, 16, 64, 8, BF16, None) == WORKSPACE  # workspace too small
     assert lib.ck_router_weight_grad_workspace_size(16, 64, 8) == 8 * 64 * 4  # one piece
     assert lib.ck_router_weight_grad_workspace_size(0, 64, 8) == 0
-    assert lib.ck_probe_mfma(None, 10, 1, P, None) == NULL
-    assert lib.ck_probe_mfma(P, 10, 0, P, None) == SHAPE
 
 
 def test_binding_turns_a_status_into_an_exception():
@@ -223,3 +221,46 @@ def test_binding_turns_a_status_into_an_exception():
     with pytest.raises(RuntimeError, match="ck_swiglu_forward"):
         _C._check(SHAPE, "ck_swiglu_forward")
     _C._check(OK, "anything")
+
+
+def test_binding_checks_index_and_operand_types_before_any_launch():
+    """The Python binding reads index tensors as int64 and every floating-point operand in the first operand's
+    type: other integer types are converted, anything else is refused before the library is called (CPU tensors
+    here: a call that got past the checks would fail on them, with another error)."""
+    import torch
+
+    from cute_kernels import _C
+
+    i32 = torch.tensor([3, 1, 2], dtype=torch.int32)
+    assert _C._index_i64(i32, "idx").dtype == torch.int64 and _C._index_i64(i32, "idx").tolist() == [3, 1, 2]
+    strided = torch.arange(8)[::2]
+    assert _C._index_i64(strided, "idx").is_contiguous()
+    with pytest.raises(ValueError, match="integer"):
+        _C._index_i64(torch.zeros(3), "idx")
+
+    X = torch.zeros(4, 8, dtype=torch.bfloat16)
+    W32 = torch.zeros(2, 8, 16, dtype=torch.float32)
+    W = W32.bfloat16()
+    out = torch.zeros(4, 16, dtype=torch.bfloat16)
+    idx = torch.arange(4)
+    off = torch.tensor([2, 4])
+    with pytest.raises(ValueError, match="W is torch.float32"):
+        _C.scatter2scatter(X, W32, idx, off, out, 1, True, True)
+    with pytest.raises(ValueError, match="integer"):
+        _C.scatter2scatter(X, W, idx.float(), off, out, 1, True, True)
+    with pytest.raises(ValueError, match="one expert offset per expert"):
+        _C.scatter2scatter(X, W, idx, torch.tensor([4]), out, 1, True, True)
+    with pytest.raises(ValueError, match="DW is torch.float32"):
+        _C.group_bwd_W(out, X, off, torch.zeros(2, 8, 16), 2)
+    with pytest.raises(ValueError, match="out is torch.float16"):
+        _C.group(X, idx, None, torch.zeros(4, 8, dtype=torch.float16), 1)
+    with pytest.raises(ValueError, match="dense int64"):
+        _C.offsets_from_sorted(idx, torch.zeros(2, dtype=torch.int32))
+    with pytest.raises(ValueError, match="dense int64"):
+        _C.moe_sort(idx, torch.zeros(4, dtype=torch.int32), torch.zeros(4, dtype=torch.int64),
+                    torch.zeros(2, dtype=torch.int64), None, 2)
+    with pytest.raises(ValueError, match="weight is torch.float32"):
+        _C.rmsnorm_forward(X, torch.ones(8), torch.empty_like(X), None, 1e-5)
+    # operands that pass the checks get as far as the device check
+    with pytest.raises(RuntimeError, match="GPU tensors"):
+        _C.scatter2scatter(X, W, idx.int(), off.int(), out, 1, True, True)

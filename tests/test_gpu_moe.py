@@ -242,7 +242,12 @@ def test_scatter2scatter_glu(gpu, dtype, shape):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("dw_layout", ["k_contiguous", "n_contiguous"])
 @pytest.mark.parametrize("shape", [(16, 2, 4, 64, 128, ()), (100, 2, 4, 72, 136, (1,)), (300, 3, 7, 200, 40, (0, 6)),
-                                   (900, 2, 3, 256, 384, ()), (50, 2, 5, 30, 20, ())])
+                                   (900, 2, 3, 256, 384, ()), (50, 2, 5, 30, 20, ()),
+                                   # output dimensions that are not multiples of the tile, more experts than a
+                                   # wavefront has lanes, experts with fewer rows than one contraction step and
+                                   # without any, more tiles than compute units
+                                   (700, 3, 70, 264, 520, (5, 69)), (40, 2, 9, 256, 256, (0, 1, 2)),
+                                   (2500, 2, 4, 1288, 2056, (2,))])
 def test_group_bwd_W(gpu, dtype, dw_layout, shape):
     from cute_kernels.kernels.scattermoe import group_bwd_W
 
