@@ -73,23 +73,28 @@ int ck_swiglu_unchunked_backward(const void* x, const void* output_grad, void* x
  *   backward : weight_grad ([H], dtype of x) is written when weight != NULL; it is reduced without
  *              atomics through `workspace` (ck_rmsnorm_backward_workspace_size bytes).
  * H must be <= 65536 (the reference's MAX_TRITON_BLOCK_SIZE limit, rmsnorm/forward.py:31-32).
+ * block_size_b is the reference's tunable BLOCK_SIZE_B (rows per program, kernels_forward.py:63-107,
+ * kernels_backward.py:177-228), here the launch variant for rows that one wavefront holds (up to 512 packets of 16
+ * bytes: 4096 16-bit elements): forward 1, 2, 4 = rows a wave requests at once before it ends, 8 or more = waves that
+ * walk rows with the next row in flight; backward 1 = two workgroups per compute unit without a row in flight,
+ * 2 or more = one workgroup per compute unit with.  0 = the library's default.  Every variant gives the same values.
  * ------------------------------------------------------------------------------------------- */
 int ck_rmsnorm_forward(const void* x, const void* weight, void* output, float* rstd, int64_t B, int64_t H,
-                       float eps, int dtype, void* stream);
+                       float eps, int dtype, int block_size_b, void* stream);
 
 /* Residual addition and RMSNorm in one pass (no counterpart in the reference, whose transformer blocks would run
  * x + residual through add_tensor (kernels/add/add_tensor/__init__.py) and then rmsnorm (kernels/rmsnorm/__init__.py)):
  *   residual_out = x + residual  (fp32 sum, rounded to the storage type),  output = rmsnorm(residual_out) as above.
  * Same values as ck_add_tensor_forward followed by ck_rmsnorm_forward, with one read of the sum less.  All tensors
- * are dense [B, H]; rstd as in ck_rmsnorm_forward.  The gradient of the pair is ck_rmsnorm_backward on residual_out
- * plus whatever gradient reaches residual_out (ck_add_tensor_forward). */
+ * are dense [B, H]; rstd and block_size_b as in ck_rmsnorm_forward.  The gradient of the pair is ck_rmsnorm_backward on
+ * residual_out plus whatever gradient reaches residual_out (ck_add_tensor_forward). */
 int ck_residual_rmsnorm_forward(const void* x, const void* residual, const void* weight, void* output,
                                 void* residual_out, float* rstd, int64_t B, int64_t H, float eps, int dtype,
-                                void* stream);
+                                int block_size_b, void* stream);
 int64_t ck_rmsnorm_backward_workspace_size(int64_t B, int64_t H);
 int ck_rmsnorm_backward(const void* x, const void* weight, const void* output_grad, const float* rstd,
                         void* x_grad, void* weight_grad, void* workspace, int64_t workspace_bytes,
-                        int64_t B, int64_t H, float eps, int dtype, void* stream);
+                        int64_t B, int64_t H, float eps, int dtype, int block_size_b, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Embedding gather / scatter-add

@@ -9,6 +9,9 @@
 //   rows column-wise with shuffles.  No atomics anywhere, so dweight is deterministic for a given team count.
 // Generic path (any H, any element alignment): one 256-lane team per row re-reading the row from cache,
 //   and a column kernel for the dweight partials.
+#include <map>
+#include <mutex>
+
 #include "ck_device.h"
 
 namespace ck {
@@ -50,13 +53,16 @@ __device__ __forceinline__ void forget(P& p) {
 
 // RES: the row that is normalised is x + res, rounded to the storage type and written to res_out as well (the
 // residual stream of a transformer block: one pass instead of an addition followed by a normalisation).
-template <typename T, int TPR, bool RES = false>
+// NP: packets per lane when the row is exactly NP * TPR packets long (no lane ever idles, so no packet sits behind a
+// branch and the loads of a row are issued back to back); 0: any row length, every packet predicated.
+template <typename T, int TPR, bool RES = false, int NP = 0>
 __global__ void CK_RMS_BOUNDS(TPR)
     rmsnorm_fwd_kernel(const typename T::storage_t* __restrict__ x, const typename T::storage_t* __restrict__ w,
                        typename T::storage_t* __restrict__ y, float* __restrict__ rstd_out, int64_t B, int H,
                        float eps, const typename T::storage_t* __restrict__ res = nullptr,
                        typename T::storage_t* __restrict__ res_out = nullptr) {
     typedef VPack<T, T::kVec> P;
+    constexpr int N = NP != 0 ? NP : kMaxPacks;
     __shared__ float red[16];
     const int teams_per_block = blockDim.x / TPR;
     const int team = blockIdx.x * teams_per_block + threadIdx.x / TPR;
@@ -69,14 +75,26 @@ __global__ void CK_RMS_BOUNDS(TPR)
     // With TPR > 64 the block is one team, so the trip count is uniform across the barriers in team_sum.
     P cur[kMaxPacks], nxt[kMaxPacks];
     P rcur[RES ? kMaxPacks : 1], rnxt[RES ? kMaxPacks : 1];
+    // the weight stays in registers (packed) for all rows of the team: fetched per row it is as many requests to
+    // the L1 / L2 path as the row itself (measured: 55 instead of 49 us at 16384 rows of 4096)
+    // (where the registers allow: the 1024-lane team has 128 per lane, and the 256-lane team with a residual needs them)
+    constexpr bool HOIST_W = TPR == 64 || (TPR == 256 && !RES);
+    P wreg[HOIST_W ? kMaxPacks : 1];
+    if (HOIST_W && w != nullptr) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const int p = t + i * TPR;
+            if (NP != 0 || p < packs) wreg[i] = reinterpret_cast<const P*>(w)[p];
+        }
+    }
     int64_t row = team;
     if (row < B) {
         const P* xr = reinterpret_cast<const P*>(x + row * H);
         const P* rr = RES ? reinterpret_cast<const P*>(res + row * H) : nullptr;
 #pragma unroll
-        for (int i = 0; i < kMaxPacks; ++i) {
+        for (int i = 0; i < N; ++i) {
             const int p = t + i * TPR;
-            if (p < packs) {
+            if (NP != 0 || p < packs) {
                 cur[i] = nt_load(xr + p);
                 if (RES) rcur[i] = nt_load(rr + p);
             }
@@ -88,9 +106,9 @@ __global__ void CK_RMS_BOUNDS(TPR)
             const P* xr = reinterpret_cast<const P*>(x + next_row * H);
             const P* rr = RES ? reinterpret_cast<const P*>(res + next_row * H) : nullptr;
 #pragma unroll
-            for (int i = 0; i < kMaxPacks; ++i) {
+            for (int i = 0; i < N; ++i) {
                 const int p = t + i * TPR;
-                if (p < packs) {
+                if (NP != 0 || p < packs) {
                     nxt[i] = nt_load(xr + p);
                     if (RES) rnxt[i] = nt_load(rr + p);
                 }
@@ -101,9 +119,9 @@ __global__ void CK_RMS_BOUNDS(TPR)
             // is normalised, exactly as an addition kernel followed by the normalisation would have it
             P* so = reinterpret_cast<P*>(res_out + row * H);
 #pragma unroll
-            for (int i = 0; i < kMaxPacks; ++i) {
+            for (int i = 0; i < N; ++i) {
                 const int p = t + i * TPR;
-                if (p < packs) {
+                if (NP != 0 || p < packs) {
 #pragma unroll
                     for (int j = 0; j < T::kVec; ++j) cur[i].v[j] = T::down(T::up(cur[i].v[j]) + T::up(rcur[i].v[j]));
                     nt_store(cur[i], so + p);
@@ -112,14 +130,24 @@ __global__ void CK_RMS_BOUNDS(TPR)
         }
         float ss = 0.f;
 #pragma unroll
-        for (int i = 0; i < kMaxPacks; ++i) {
+        for (int i = 0; i < N; ++i) {
             const int p = t + i * TPR;
-            if (p < packs) {
+            if (NP != 0 || p < packs) {
 #pragma unroll
                 for (int j = 0; j < T::kVec; ++j) {
                     const float f = T::up(cur[i].v[j]);
                     ss += f * f;
                 }
+            }
+            __builtin_amdgcn_sched_barrier(0);  // one packet at a time: the widened values do not pile up
+        }
+        if (sizeof(typename T::storage_t) == 2) {
+            // 16-bit rows: only the packed form lives across the reduction (the widened copies would double the
+            // registers and halve the waves per SIMD)
+#pragma unroll
+            for (int i = 0; i < N; ++i) {
+                forget(cur[i]);
+                if (HOIST_W) forget(wreg[i]);
             }
         }
         ss = team_sum<TPR>(ss, red);
@@ -128,12 +156,12 @@ __global__ void CK_RMS_BOUNDS(TPR)
 
         P* yr = reinterpret_cast<P*>(y + row * H);
 #pragma unroll
-        for (int i = 0; i < kMaxPacks; ++i) {
+        for (int i = 0; i < N; ++i) {
             const int p = t + i * TPR;
-            if (p < packs) {
+            if (NP != 0 || p < packs) {
                 P o;
                 if (w != nullptr) {
-                    const P wv = reinterpret_cast<const P*>(w)[p];
+                    const P wv = HOIST_W ? wreg[HOIST_W ? i : 0] : reinterpret_cast<const P*>(w)[p];
 #pragma unroll
                     for (int j = 0; j < T::kVec; ++j) o.v[j] = T::down(T::up(cur[i].v[j]) * rstd * T::up(wv.v[j]));
                 } else {
@@ -142,24 +170,129 @@ __global__ void CK_RMS_BOUNDS(TPR)
                 }
                 nt_store(o, yr + p);
             }
+            __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
-        for (int i = 0; i < kMaxPacks; ++i) {
+        for (int i = 0; i < N; ++i) {
             cur[i] = nxt[i];
             if (RES) rcur[i] = rnxt[i];
         }
     }
 }
 
+// Rows of up to 64 * kMaxPacks packets, forward, without the walk over rows: one wave takes RPW consecutive rows,
+// requests all of them at once, reduces and writes them, and ends.  Few registers (the rows in their packed form), so
+// many waves per SIMD are resident and their requests overlap each other's reductions - the persistent kernel above
+// holds two rows per wave in 134 registers, three waves per SIMD, and its fourth workgroup per compute unit only
+// starts when another has ended.  RPW > 1 reads the weight once for RPW rows.
+template <typename T, int RPW, bool RES = false, int NP = 0>
+__global__ void __launch_bounds__(256)
+    rmsnorm_fwd_rows_kernel(const typename T::storage_t* __restrict__ x, const typename T::storage_t* __restrict__ w,
+                            typename T::storage_t* __restrict__ y, float* __restrict__ rstd_out, int64_t B, int H,
+                            float eps, const typename T::storage_t* __restrict__ res = nullptr,
+                            typename T::storage_t* __restrict__ res_out = nullptr) {
+    typedef VPack<T, T::kVec> P;
+    constexpr int N = NP != 0 ? NP : kMaxPacks;
+    const int lane = lane_id();
+    const int packs = H / T::kVec;
+    const float inv_h = 1.0f / (float)H;
+    const int64_t row0 = ((int64_t)blockIdx.x * (blockDim.x / CK_WAVE) + threadIdx.x / CK_WAVE) * RPW;
+    if (row0 >= B) return;
+    P v[RPW][kMaxPacks], r[RES ? RPW : 1][RES ? kMaxPacks : 1];
+#pragma unroll
+    for (int q = 0; q < RPW; ++q) {
+        if (row0 + q < B) {
+            const P* xr = reinterpret_cast<const P*>(x + (row0 + q) * H);
+            const P* rr = RES ? reinterpret_cast<const P*>(res + (row0 + q) * H) : nullptr;
+#pragma unroll
+            for (int i = 0; i < N; ++i) {
+                const int p = lane + i * CK_WAVE;
+                if (NP != 0 || p < packs) {
+                    v[q][i] = nt_load(xr + p);
+                    if (RES) r[q][i] = nt_load(rr + p);
+                }
+            }
+        }
+    }
+    P wv[kMaxPacks];
+    if (w != nullptr) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const int p = lane + i * CK_WAVE;
+            if (NP != 0 || p < packs) wv[i] = reinterpret_cast<const P*>(w)[p];
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < RPW; ++q) {
+        const int64_t row = row0 + q;
+        if (row >= B) break;
+        if (RES) {
+            // the sum is rounded to the storage type first: that value is both the new residual and the row that is
+            // normalised, exactly as an addition kernel followed by the normalisation would have it
+            P* so = reinterpret_cast<P*>(res_out + row * H);
+#pragma unroll
+            for (int i = 0; i < N; ++i) {
+                const int p = lane + i * CK_WAVE;
+                if (NP != 0 || p < packs) {
+#pragma unroll
+                    for (int j = 0; j < T::kVec; ++j) v[q][i].v[j] = T::down(T::up(v[q][i].v[j]) + T::up(r[q][i].v[j]));
+                    nt_store(v[q][i], so + p);
+                }
+            }
+        }
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const int p = lane + i * CK_WAVE;
+            if (NP != 0 || p < packs) {
+#pragma unroll
+                for (int j = 0; j < T::kVec; ++j) {
+                    const float f = T::up(v[q][i].v[j]);
+                    ss += f * f;
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);  // one packet at a time: the widened values do not pile up
+        }
+        if (sizeof(typename T::storage_t) == 2) {
+#pragma unroll
+            for (int i = 0; i < N; ++i) {
+                forget(v[q][i]);
+                forget(wv[i]);
+            }
+        }
+        ss = wave_sum(ss);
+        const float rstd = rsqrtf(ss * inv_h + eps);
+        if (rstd_out != nullptr && lane == 0) rstd_out[row] = rstd;
+        P* yr = reinterpret_cast<P*>(y + row * H);
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const int p = lane + i * CK_WAVE;
+            if (NP != 0 || p < packs) {
+                P o;
+                if (w != nullptr) {
+#pragma unroll
+                    for (int j = 0; j < T::kVec; ++j) o.v[j] = T::down(T::up(v[q][i].v[j]) * rstd * T::up(wv[i].v[j]));
+                } else {
+#pragma unroll
+                    for (int j = 0; j < T::kVec; ++j) o.v[j] = T::down(T::up(v[q][i].v[j]) * rstd);
+                }
+                nt_store(o, yr + p);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+}
+
 // Backward: one wave per SIMD with the whole register file (packed current row and next row of x and dy, packed
 // weight, 64 fp32 dweight accumulators); the next row's loads are in flight while the current row is reduced.
-template <typename T, int TPR, bool HAS_W>
-__global__ void __launch_bounds__(TPR > 256 ? TPR : 256)
-    rmsnorm_bwd_kernel(const typename T::storage_t* __restrict__ x, const typename T::storage_t* __restrict__ w,
-                       const typename T::storage_t* __restrict__ dy, const float* __restrict__ rstd_in,
-                       typename T::storage_t* __restrict__ dx, float* __restrict__ dw_partial, int64_t B, int H,
-                       float eps) {
+template <typename T, int TPR, bool HAS_W, bool PREFETCH, int NP>
+__device__ __forceinline__ void rmsnorm_bwd_body(const typename T::storage_t* __restrict__ x,
+                                                 const typename T::storage_t* __restrict__ w,
+                                                 const typename T::storage_t* __restrict__ dy,
+                                                 const float* __restrict__ rstd_in, typename T::storage_t* __restrict__ dx,
+                                                 float* __restrict__ dw_partial, int64_t B, int H, float eps) {
     typedef VPack<T, T::kVec> P;
+    constexpr int N = NP != 0 ? NP : kMaxPacks;
     __shared__ float red[16];
     const int teams_per_block = blockDim.x / TPR;
     const int team = blockIdx.x * teams_per_block + threadIdx.x / TPR;
@@ -172,39 +305,43 @@ __global__ void __launch_bounds__(TPR > 256 ? TPR : 256)
     float dw[kMaxPacks][T::kVec];
     if (HAS_W) {
 #pragma unroll
-        for (int i = 0; i < kMaxPacks; ++i) {
+        for (int i = 0; i < N; ++i) {
             const int p = t + i * TPR;
-            if (p < packs) wv[i] = reinterpret_cast<const P*>(w)[p];
+            if (NP != 0 || p < packs) wv[i] = reinterpret_cast<const P*>(w)[p];
 #pragma unroll
             for (int j = 0; j < T::kVec; ++j) dw[i][j] = 0.f;
         }
     }
 
     // rows are dealt round-robin; with TPR > 64 the block is one team so the trip count is block-uniform
-    constexpr bool PREFETCH = TPR <= 256;  // the 1024-lane variant has 128 registers per lane: no room
-    P xv[kMaxPacks], gv[kMaxPacks], xn[kMaxPacks], gn[kMaxPacks];
+    P xv[kMaxPacks], gv[kMaxPacks], xn[PREFETCH ? kMaxPacks : 1], gn[PREFETCH ? kMaxPacks : 1];
     if (PREFETCH && team < B) {
         const P* xr = reinterpret_cast<const P*>(x + (int64_t)team * H);
         const P* gr = reinterpret_cast<const P*>(dy + (int64_t)team * H);
 #pragma unroll
-        for (int i = 0; i < kMaxPacks; ++i) {
+        for (int i = 0; i < N; ++i) {
             const int p = t + i * TPR;
-            if (p < packs) {
+            if (NP != 0 || p < packs) {
                 xv[i] = nt_load(xr + p);
                 gv[i] = nt_load(gr + p);
             }
         }
     }
     for (int64_t row = team; row < B; row += num_teams) {
+        // 1/rms of this row, requested BEFORE the next row's packets: loads complete in the order they were issued,
+        // so a value requested behind them would not arrive before they all have - the wait for it would be a wait
+        // for the whole row that is meant to stay in flight during this row's arithmetic
+        float rstd_given = 0.f;
+        if (rstd_in != nullptr) rstd_given = rstd_in[row];
         if (PREFETCH) {
             const int64_t next_row = row + num_teams;
             if (next_row < B) {
                 const P* xr = reinterpret_cast<const P*>(x + next_row * H);
                 const P* gr = reinterpret_cast<const P*>(dy + next_row * H);
 #pragma unroll
-                for (int i = 0; i < kMaxPacks; ++i) {
+                for (int i = 0; i < N; ++i) {
                     const int p = t + i * TPR;
-                    if (p < packs) {
+                    if (NP != 0 || p < packs) {
                         xn[i] = nt_load(xr + p);
                         gn[i] = nt_load(gr + p);
                     }
@@ -214,9 +351,9 @@ __global__ void __launch_bounds__(TPR > 256 ? TPR : 256)
             const P* xr = reinterpret_cast<const P*>(x + row * H);
             const P* gr = reinterpret_cast<const P*>(dy + row * H);
 #pragma unroll
-            for (int i = 0; i < kMaxPacks; ++i) {
+            for (int i = 0; i < N; ++i) {
                 const int p = t + i * TPR;
-                if (p < packs) {
+                if (NP != 0 || p < packs) {
                     xv[i] = nt_load(xr + p);
                     gv[i] = nt_load(gr + p);
                 }
@@ -224,9 +361,9 @@ __global__ void __launch_bounds__(TPR > 256 ? TPR : 256)
         }
         float ss = 0.f, dot = 0.f;
 #pragma unroll
-        for (int i = 0; i < kMaxPacks; ++i) {
+        for (int i = 0; i < N; ++i) {
             const int p = t + i * TPR;
-            if (p < packs) {
+            if (NP != 0 || p < packs) {
 #pragma unroll
                 for (int j = 0; j < T::kVec; ++j) {
                     const float xf = T::up(xv[i].v[j]);
@@ -241,7 +378,7 @@ __global__ void __launch_bounds__(TPR > 256 ? TPR : 256)
         if (sizeof(typename T::storage_t) == 2) {
             // 16-bit rows: keep only the packed form across the reductions
 #pragma unroll
-            for (int i = 0; i < kMaxPacks; ++i) {
+            for (int i = 0; i < N; ++i) {
                 forget(xv[i]);
                 forget(gv[i]);
                 if (HAS_W) forget(wv[i]);
@@ -249,7 +386,7 @@ __global__ void __launch_bounds__(TPR > 256 ? TPR : 256)
         }
         float rstd;
         if (rstd_in != nullptr) {
-            rstd = rstd_in[row];
+            rstd = rstd_given;
         } else {
             ss = team_sum<TPR>(ss, red);
             rstd = rsqrtf(ss * inv_h + eps);
@@ -259,9 +396,9 @@ __global__ void __launch_bounds__(TPR > 256 ? TPR : 256)
 
         P* dr = reinterpret_cast<P*>(dx + row * H);
 #pragma unroll
-        for (int i = 0; i < kMaxPacks; ++i) {
+        for (int i = 0; i < N; ++i) {
             const int p = t + i * TPR;
-            if (p < packs) {
+            if (NP != 0 || p < packs) {
                 P o;
 #pragma unroll
                 for (int j = 0; j < T::kVec; ++j) {
@@ -281,7 +418,7 @@ __global__ void __launch_bounds__(TPR > 256 ? TPR : 256)
         }
         if (PREFETCH) {
 #pragma unroll
-            for (int i = 0; i < kMaxPacks; ++i) {
+            for (int i = 0; i < N; ++i) {
                 xv[i] = xn[i];
                 gv[i] = gn[i];
             }
@@ -296,9 +433,9 @@ __global__ void __launch_bounds__(TPR > 256 ? TPR : 256)
         __shared__ float comb[kTeams > 1 ? kTeams * kCols : 4];
         float* out = kTeams > 1 ? comb + (threadIdx.x / TPR) * kCols : dw_partial + (int64_t)team * H;
 #pragma unroll
-        for (int i = 0; i < kMaxPacks; ++i) {
+        for (int i = 0; i < N; ++i) {
             const int p = t + i * TPR;
-            if (p < packs) {
+            if (NP != 0 || p < packs) {
 #pragma unroll
                 for (int j = 0; j < T::kVec; j += 4) {
                     float4 v = make_float4(dw[i][j], dw[i][j + 1], dw[i][j + 2], dw[i][j + 3]);
@@ -323,6 +460,29 @@ __global__ void __launch_bounds__(TPR > 256 ? TPR : 256)
             }
         }
     }
+}
+
+// The next row of x and dy in flight while the current one is reduced: 288 registers with a weight at a row length
+// of 4096, i.e. one wave per SIMD and one workgroup per compute unit (the 1024-lane variant has 128 registers per
+// lane and no room for it).
+template <typename T, int TPR, bool HAS_W, int NP = 0>
+__global__ void __launch_bounds__(TPR > 256 ? TPR : 256)
+    rmsnorm_bwd_kernel(const typename T::storage_t* __restrict__ x, const typename T::storage_t* __restrict__ w,
+                       const typename T::storage_t* __restrict__ dy, const float* __restrict__ rstd_in,
+                       typename T::storage_t* __restrict__ dx, float* __restrict__ dw_partial, int64_t B, int H,
+                       float eps) {
+    rmsnorm_bwd_body<T, TPR, HAS_W, TPR <= 256, NP>(x, w, dy, rstd_in, dx, dw_partial, B, H, eps);
+}
+
+// One wave per row without the row in flight: fits two waves per SIMD, so two workgroups per compute unit walk the
+// rows and one wave's loads overlap the other's reductions and stores.
+template <typename T, bool HAS_W, int NP = 0>
+__global__ void __launch_bounds__(256, 2)
+    rmsnorm_bwd_two_kernel(const typename T::storage_t* __restrict__ x, const typename T::storage_t* __restrict__ w,
+                           const typename T::storage_t* __restrict__ dy, const float* __restrict__ rstd_in,
+                           typename T::storage_t* __restrict__ dx, float* __restrict__ dw_partial, int64_t B, int H,
+                           float eps) {
+    rmsnorm_bwd_body<T, 64, HAS_W, false, NP>(x, w, dy, rstd_in, dx, dw_partial, B, H, eps);
 }
 
 // dweight[j] = sum over `parts` partial rows of partial[r][j].  One wave per block owns 16 columns:
@@ -475,6 +635,12 @@ __global__ void __launch_bounds__(256)
 
 // ---- host side ------------------------------------------------------------------------------
 constexpr int kReduceSplits = 16;  // row splits of the first dweight reduction pass
+#ifndef CK_RMSNORM_FWD_DEFAULT_ROWS
+#define CK_RMSNORM_FWD_DEFAULT_ROWS 1
+#endif
+#ifndef CK_RMSNORM_BWD_DEFAULT_VARIANT
+#define CK_RMSNORM_BWD_DEFAULT_VARIANT 2
+#endif
 
 static int cu_count() {
     static int cached[64] = {0};
@@ -486,6 +652,21 @@ static int cu_count() {
         cached[dev] = n;
     }
     return cached[dev];
+}
+
+// Workgroups of `kernel` that one compute unit holds at once (registers, LDS): a persistent launch with more than
+// that leaves the surplus waiting for a slot while the others already finish their rows.  Looked up once per kernel.
+static int resident_blocks(const void* kernel, int block) {
+    static std::mutex mutex;
+    static std::map<const void*, int> known;
+    std::lock_guard<std::mutex> lock(mutex);
+    auto it = known.find(kernel);
+    if (it != known.end()) return it->second;
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, block, 0) != hipSuccess || n < 1) n = 1;
+    if (n > 8) n = 8;
+    known[kernel] = n;
+    return n;
 }
 
 // threads per row on the fast path, 0 when the row does not fit the register budget
@@ -500,18 +681,89 @@ static int fast_tpr(int64_t H, int dtype) {
 }
 
 // teams of the persistent backward kernel (an upper bound of the number of fp32 partial rows)
-static int bwd_teams(int64_t B, int tpr) {
+static int bwd_teams(int64_t B, int tpr, int per_cu = 1) {
     const int block = tpr > 256 ? tpr : 256;
     const int teams_per_block = block / tpr;
-    int64_t blocks = (int64_t)cu_count();  // one workgroup per CU: the kernel uses the whole register file
+    int64_t blocks = (int64_t)cu_count() * per_cu;  // per_cu = 1: the kernel uses the whole register file
     const int64_t need = ck_ceil_div(B, teams_per_block);
     if (blocks > need) blocks = need;
     if (blocks < 1) blocks = 1;
     return (int)(blocks * teams_per_block);
 }
 
+// Launch variants of the one-wave-per-row kernels, selected by `block_size_b` (the reference's BLOCK_SIZE_B: rows per
+// program): forward 1, 2, 4 = rows a wave requests at once and then ends (rmsnorm_fwd_rows_kernel), 8 or more = waves
+// that walk rows with the next one in flight (rmsnorm_fwd_kernel); backward 1 = two workgroups per compute unit
+// without a row in flight, 2 or more = one with.  0 = the default.  Rows wider than a wave's registers have one variant.
+constexpr int kFwdDefaultRows = CK_RMSNORM_FWD_DEFAULT_ROWS, kBwdDefaultVariant = CK_RMSNORM_BWD_DEFAULT_VARIANT;
+
+// packets per lane when a row is exactly that many packets per lane of a TPR-lane team (2, 4 or 8), else 0
+static int exact_packs(int64_t H, int dtype, int tpr) {
+    const int vec = dtype == CK_F32 ? 4 : 8;
+    const int64_t packs = H / vec;
+    for (int np : {8, 4, 2})
+        if (packs == (int64_t)np * tpr) return np;
+    return 0;
+}
+
+struct FwdArgs {
+    const void *x, *residual, *weight;
+    void *output, *residual_out;
+    float* rstd;
+    int64_t B;
+    int H;
+    float eps;
+};
+
+template <typename T, int RPW, bool RES, int NP>
+static void launch_fwd_rows_np(hipStream_t s, const FwdArgs& a) {
+    typedef typename T::storage_t S;
+    const int64_t grid = ck_ceil_div(a.B, 4 * RPW);
+    hipLaunchKernelGGL((ck::rmsnorm_fwd_rows_kernel<T, RPW, RES, NP>), dim3((unsigned)grid), dim3(256), 0, s, (const S*)a.x,
+                       (const S*)a.weight, (S*)a.output, a.rstd, a.B, a.H, a.eps, (const S*)a.residual, (S*)a.residual_out);
+}
+template <typename T, int RPW, bool RES>
+static void launch_fwd_rows(hipStream_t s, const FwdArgs& a, int np) {
+    if (np == 8) launch_fwd_rows_np<T, RPW, RES, 8>(s, a);
+    else if (np == 4) launch_fwd_rows_np<T, RPW, RES, 4>(s, a);
+    else launch_fwd_rows_np<T, RPW, RES, 0>(s, a);
+}
+
+// waves (or wider teams) that walk rows with the next row in flight: as many workgroups as are resident at once
+template <typename T, int TPR, bool RES, int NP>
+static void launch_fwd_walk_np(hipStream_t s, const FwdArgs& a) {
+    typedef typename T::storage_t S;
+    constexpr int block = TPR > 256 ? TPR : 256;
+    const void* kernel = (const void*)ck::rmsnorm_fwd_kernel<T, TPR, RES, NP>;
+    int64_t grid = (int64_t)cu_count() * resident_blocks(kernel, block);
+    const int64_t need = ck_ceil_div(a.B, block / TPR);
+    if (grid > need) grid = need;
+    hipLaunchKernelGGL((ck::rmsnorm_fwd_kernel<T, TPR, RES, NP>), dim3((unsigned)grid), dim3(block), 0, s, (const S*)a.x,
+                       (const S*)a.weight, (S*)a.output, a.rstd, a.B, a.H, a.eps, (const S*)a.residual, (S*)a.residual_out);
+}
+template <typename T, int TPR, bool RES>
+static void launch_fwd_walk(hipStream_t s, const FwdArgs& a, int np) {
+    if (np == 8) launch_fwd_walk_np<T, TPR, RES, 8>(s, a);
+    else if (np == 4) launch_fwd_walk_np<T, TPR, RES, 4>(s, a);
+    else if (np == 2) launch_fwd_walk_np<T, TPR, RES, 2>(s, a);
+    else launch_fwd_walk_np<T, TPR, RES, 0>(s, a);
+}
+
+// the fast paths of both forward entry points (tpr = 64, 256; 1024 without a residual)
+template <typename T, bool RES>
+static void launch_fwd_fast(hipStream_t s, const FwdArgs& a, int tpr, int dtype, int block_size_b) {
+    const int np = exact_packs(a.H, dtype, tpr);
+    const int rows = block_size_b == 0 ? kFwdDefaultRows : block_size_b;
+    if (tpr == 64 && rows == 1) launch_fwd_rows<T, 1, RES>(s, a, np);
+    else if (tpr == 64 && rows < 8) launch_fwd_rows<T, 2, RES>(s, a, np);
+    else if (tpr == 64) launch_fwd_walk<T, 64, RES>(s, a, np);
+    else if (tpr == 256) launch_fwd_walk<T, 256, RES>(s, a, np);
+    else launch_fwd_walk_np<T, 1024, false, 0>(s, a);
+}
+
 extern "C" int ck_rmsnorm_forward(const void* x, const void* weight, void* output, float* rstd, int64_t B, int64_t H,
-                                  float eps, int dtype, void* stream) {
+                                  float eps, int dtype, int block_size_b, void* stream) {
+    if (block_size_b < 0) return CK_ERR_SHAPE;
     if (B < 0 || H < 0 || H > 65536) return CK_ERR_SHAPE;
     if (B == 0 || H == 0) return CK_OK;
     if (!x || !output) return CK_ERR_NULL;
@@ -520,24 +772,11 @@ extern "C" int ck_rmsnorm_forward(const void* x, const void* weight, void* outpu
     hipStream_t s = (hipStream_t)stream;
     const bool aligned = ck_aligned16(x) && ck_aligned16(output) && (!weight || ck_aligned16(weight));
     const int tpr = aligned ? fast_tpr(H, dtype) : 0;
+    const FwdArgs a = {x, nullptr, weight, output, nullptr, rstd, B, (int)H, eps};
     CK_DISPATCH_DTYPE(dtype, {
         typedef typename T::storage_t S;
-        if (tpr == 64) {
-            // persistent: a few workgroups per CU, each wave walking rows with the next row in flight
-            int64_t grid = (int64_t)cu_count() * 4;
-            if (grid > ck_ceil_div(B, 4)) grid = ck_ceil_div(B, 4);
-            hipLaunchKernelGGL((ck::rmsnorm_fwd_kernel<T, 64>), dim3((unsigned)grid), dim3(256), 0, s, (const S*)x,
-                               (const S*)weight, (S*)output, rstd, B, (int)H, eps);
-        } else if (tpr == 256) {
-            int64_t grid = (int64_t)cu_count() * 4;
-            if (grid > B) grid = B;
-            hipLaunchKernelGGL((ck::rmsnorm_fwd_kernel<T, 256>), dim3((unsigned)grid), dim3(256), 0, s, (const S*)x,
-                               (const S*)weight, (S*)output, rstd, B, (int)H, eps);
-        } else if (tpr == 1024) {
-            int64_t grid = (int64_t)cu_count() * 2;
-            if (grid > B) grid = B;
-            hipLaunchKernelGGL((ck::rmsnorm_fwd_kernel<T, 1024>), dim3((unsigned)grid), dim3(1024), 0, s, (const S*)x,
-                               (const S*)weight, (S*)output, rstd, B, (int)H, eps);
+        if (tpr != 0) {
+            launch_fwd_fast<T, false>(s, a, tpr, dtype, block_size_b);
         } else {
             const int64_t grid = B < 65536 ? B : 65536;
             hipLaunchKernelGGL((ck::rmsnorm_fwd_generic_kernel<T>), dim3((unsigned)grid), dim3(256), 0, s, (const S*)x,
@@ -549,7 +788,8 @@ extern "C" int ck_rmsnorm_forward(const void* x, const void* weight, void* outpu
 
 extern "C" int ck_residual_rmsnorm_forward(const void* x, const void* residual, const void* weight, void* output,
                                            void* residual_out, float* rstd, int64_t B, int64_t H, float eps, int dtype,
-                                           void* stream) {
+                                           int block_size_b, void* stream) {
+    if (block_size_b < 0) return CK_ERR_SHAPE;
     if (B < 0 || H < 0 || H > 65536) return CK_ERR_SHAPE;
     if (B == 0 || H == 0) return CK_OK;
     if (!x || !residual || !output || !residual_out) return CK_ERR_NULL;
@@ -564,22 +804,10 @@ extern "C" int ck_residual_rmsnorm_forward(const void* x, const void* residual, 
         // rows outside the register budget of the one-pass kernel (or unaligned): the sum, then the normalisation
         const int st = ck_add_tensor_forward(x, residual, residual_out, B * H, dtype, 256, stream);
         if (st != CK_OK) return st;
-        return ck_rmsnorm_forward(residual_out, weight, output, rstd, B, H, eps, dtype, stream);
+        return ck_rmsnorm_forward(residual_out, weight, output, rstd, B, H, eps, dtype, block_size_b, stream);
     }
-    CK_DISPATCH_DTYPE(dtype, {
-        typedef typename T::storage_t S;
-        if (tpr == 64) {
-            int64_t grid = (int64_t)cu_count() * 4;
-            if (grid > ck_ceil_div(B, 4)) grid = ck_ceil_div(B, 4);
-            hipLaunchKernelGGL((ck::rmsnorm_fwd_kernel<T, 64, true>), dim3((unsigned)grid), dim3(256), 0, s, (const S*)x,
-                               (const S*)weight, (S*)output, rstd, B, (int)H, eps, (const S*)residual, (S*)residual_out);
-        } else {
-            int64_t grid = (int64_t)cu_count() * 4;
-            if (grid > B) grid = B;
-            hipLaunchKernelGGL((ck::rmsnorm_fwd_kernel<T, 256, true>), dim3((unsigned)grid), dim3(256), 0, s, (const S*)x,
-                               (const S*)weight, (S*)output, rstd, B, (int)H, eps, (const S*)residual, (S*)residual_out);
-        }
-    });
+    const FwdArgs a = {x, residual, weight, output, residual_out, rstd, B, (int)H, eps};
+    CK_DISPATCH_DTYPE(dtype, { launch_fwd_fast<T, true>(s, a, tpr, dtype, block_size_b); });
     return ck_launch_status();
 }
 
@@ -591,7 +819,7 @@ extern "C" int64_t ck_rmsnorm_backward_workspace_size(int64_t B, int64_t H) {
     if (B <= 0 || H <= 0) return 0;
     int64_t teams = 1;
     for (int tpr : {64, 256, 1024}) {
-        const int64_t t = bwd_teams(B, tpr);
+        const int64_t t = bwd_teams(B, tpr, tpr == 64 ? 2 : 1);
         if (t > teams) teams = t;
     }
     const int64_t fast = (teams + kReduceSplits) * H * 4;
@@ -599,22 +827,47 @@ extern "C" int64_t ck_rmsnorm_backward_workspace_size(int64_t B, int64_t H) {
     return fast > generic ? fast : generic;
 }
 
-template <typename T, int TPR>
-static void launch_bwd(unsigned grid, int block, hipStream_t s, const void* x, const void* weight, const void* dy,
-                       const float* rstd, void* dx, float* ws, int64_t B, int H, float eps) {
+struct BwdArgs {
+    const void *x, *weight, *dy;
+    const float* rstd;
+    void* dx;
+    float* ws;
+    int64_t B;
+    int H;
+    float eps;
+};
+
+template <typename T, int TPR, int NP>
+static void launch_bwd_np(unsigned grid, int block, hipStream_t s, const BwdArgs& a) {
     typedef typename T::storage_t S;
-    if (weight)
-        hipLaunchKernelGGL((ck::rmsnorm_bwd_kernel<T, TPR, true>), dim3(grid), dim3(block), 0, s, (const S*)x,
-                           (const S*)weight, (const S*)dy, rstd, (S*)dx, ws, B, H, eps);
+    if (a.weight)
+        hipLaunchKernelGGL((ck::rmsnorm_bwd_kernel<T, TPR, true, NP>), dim3(grid), dim3(block), 0, s, (const S*)a.x,
+                           (const S*)a.weight, (const S*)a.dy, a.rstd, (S*)a.dx, a.ws, a.B, a.H, a.eps);
     else
-        hipLaunchKernelGGL((ck::rmsnorm_bwd_kernel<T, TPR, false>), dim3(grid), dim3(block), 0, s, (const S*)x,
-                           (const S*)weight, (const S*)dy, rstd, (S*)dx, ws, B, H, eps);
+        hipLaunchKernelGGL((ck::rmsnorm_bwd_kernel<T, TPR, false, NP>), dim3(grid), dim3(block), 0, s, (const S*)a.x,
+                           (const S*)a.weight, (const S*)a.dy, a.rstd, (S*)a.dx, a.ws, a.B, a.H, a.eps);
+}
+template <typename T, int TPR>
+static void launch_bwd(unsigned grid, int block, hipStream_t s, const BwdArgs& a, int np) {
+    if (np == 8) launch_bwd_np<T, TPR, 8>(grid, block, s, a);
+    else if (np == 4) launch_bwd_np<T, TPR, 4>(grid, block, s, a);
+    else launch_bwd_np<T, TPR, 0>(grid, block, s, a);
+}
+template <typename T, int NP>
+static void launch_bwd_two_np(unsigned grid, hipStream_t s, const BwdArgs& a) {
+    typedef typename T::storage_t S;
+    if (a.weight)
+        hipLaunchKernelGGL((ck::rmsnorm_bwd_two_kernel<T, true, NP>), dim3(grid), dim3(256), 0, s, (const S*)a.x,
+                           (const S*)a.weight, (const S*)a.dy, a.rstd, (S*)a.dx, a.ws, a.B, a.H, a.eps);
+    else
+        hipLaunchKernelGGL((ck::rmsnorm_bwd_two_kernel<T, false, NP>), dim3(grid), dim3(256), 0, s, (const S*)a.x,
+                           (const S*)a.weight, (const S*)a.dy, a.rstd, (S*)a.dx, a.ws, a.B, a.H, a.eps);
 }
 
 extern "C" int ck_rmsnorm_backward(const void* x, const void* weight, const void* output_grad, const float* rstd,
                                    void* x_grad, void* weight_grad, void* workspace, int64_t workspace_bytes, int64_t B,
-                                   int64_t H, float eps, int dtype, void* stream) {
-    if (B < 0 || H < 0 || H > 65536) return CK_ERR_SHAPE;
+                                   int64_t H, float eps, int dtype, int block_size_b, void* stream) {
+    if (B < 0 || H < 0 || H > 65536 || block_size_b < 0) return CK_ERR_SHAPE;
     if (dtype != CK_F32 && dtype != CK_F16 && dtype != CK_BF16) return CK_ERR_DTYPE;
     hipStream_t s = (hipStream_t)stream;
     if (B == 0 || H == 0) {
@@ -642,12 +895,19 @@ extern "C" int ck_rmsnorm_backward(const void* x, const void* weight, const void
     CK_DISPATCH_DTYPE(dtype, {
         typedef typename T::storage_t S;
         if (tpr != 0) {
-            const int teams = bwd_teams(B, tpr);
+            const bool two = tpr == 64 && (block_size_b == 0 ? kBwdDefaultVariant : block_size_b) == 1;
+            const int teams = bwd_teams(B, tpr, two ? 2 : 1);
             const int block = tpr > 256 ? tpr : 256;
             const unsigned grid = (unsigned)(teams / (block / tpr));
-            if (tpr == 64) launch_bwd<T, 64>(grid, block, s, x, weight, output_grad, rstd, x_grad, ws, B, (int)H, eps);
-            else if (tpr == 256) launch_bwd<T, 256>(grid, block, s, x, weight, output_grad, rstd, x_grad, ws, B, (int)H, eps);
-            else launch_bwd<T, 1024>(grid, block, s, x, weight, output_grad, rstd, x_grad, ws, B, (int)H, eps);
+            const BwdArgs a = {x, weight, output_grad, rstd, x_grad, ws, B, (int)H, eps};
+            const int np = tpr == 1024 ? 0 : exact_packs(H, dtype, tpr);
+            if (two) {
+                // (the branch-free forms of this variant need more than the 256 registers two waves per SIMD leave)
+                if (np == 4) launch_bwd_two_np<T, 4>(grid, s, a);
+                else launch_bwd_two_np<T, 0>(grid, s, a);
+            } else if (tpr == 64) launch_bwd<T, 64>(grid, block, s, a, np);
+            else if (tpr == 256) launch_bwd<T, 256>(grid, block, s, a, np);
+            else launch_bwd_np<T, 1024, 0>(grid, block, s, a);
             if (weight) {
                 // one partial row per workgroup -> (kReduceSplits rows, fp32, behind the partial rows ->) dweight
                 const int rows = (int)grid;

@@ -42,10 +42,10 @@ _SIGNATURES = {
     "ck_swiglu_backward": (_i32, [_p, _p, _p, _p, _p, _i64, _i32, _i32, _p]),
     "ck_swiglu_unchunked_forward": (_i32, [_p, _p, _i64, _i64, _i32, _i32, _p]),
     "ck_swiglu_unchunked_backward": (_i32, [_p, _p, _p, _i64, _i64, _i32, _i32, _p]),
-    "ck_rmsnorm_forward": (_i32, [_p, _p, _p, _p, _i64, _i64, _f32, _i32, _p]),
-    "ck_residual_rmsnorm_forward": (_i32, [_p, _p, _p, _p, _p, _p, _i64, _i64, _f32, _i32, _p]),
+    "ck_rmsnorm_forward": (_i32, [_p, _p, _p, _p, _i64, _i64, _f32, _i32, _i32, _p]),
+    "ck_residual_rmsnorm_forward": (_i32, [_p, _p, _p, _p, _p, _p, _i64, _i64, _f32, _i32, _i32, _p]),
     "ck_rmsnorm_backward_workspace_size": (_i64, [_i64, _i64]),
-    "ck_rmsnorm_backward": (_i32, [_p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _f32, _i32, _p]),
+    "ck_rmsnorm_backward": (_i32, [_p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _f32, _i32, _i32, _p]),
     "ck_embedding_forward": (_i32, [_p, _i32, _p, _p, _i64, _i64, _i64, _i32, _p]),
     "ck_embedding_backward_workspace_size": (_i64, [_i64, _i64, _i64]),
     "ck_embedding_backward": (_i32, [_p, _i32, _p, _p, _p, _i64, _i64, _i64, _i64, _i32, _p]),
@@ -299,7 +299,7 @@ def swiglu_unchunked_backward(x, output_grad, x_grad, block_size: int) -> None:
         )
 
 
-def rmsnorm_forward(x, weight, output, rstd, eps: float) -> None:
+def rmsnorm_forward(x, weight, output, rstd, eps: float, block_size_b: int = 0) -> None:
     lib = load_library()
     _same_dtype(x, "rmsnorm_forward", weight=weight, output=output)
     H = x.size(-1)
@@ -307,12 +307,12 @@ def rmsnorm_forward(x, weight, output, rstd, eps: float) -> None:
     with _Launch(x, weight, output, rstd) as L:
         _check(
             lib.ck_rmsnorm_forward(_ptr(x), _ptr(weight), _ptr(output), _ptr(rstd), B, H, eps, dtype_code(x.dtype),
-                                   L.stream),
+                                   block_size_b, L.stream),
             "ck_rmsnorm_forward",
         )
 
 
-def residual_rmsnorm_forward(x, residual, weight, output, residual_out, rstd, eps: float) -> None:
+def residual_rmsnorm_forward(x, residual, weight, output, residual_out, rstd, eps: float, block_size_b: int = 0) -> None:
     """residual_out = x + residual, output = rmsnorm(residual_out); all dense and of one shape and dtype."""
     lib = load_library()
     H = x.size(-1)
@@ -325,7 +325,7 @@ def residual_rmsnorm_forward(x, residual, weight, output, residual_out, rstd, ep
     with _Launch(x, residual, weight, output, residual_out, rstd) as L:
         _check(
             lib.ck_residual_rmsnorm_forward(_ptr(x), _ptr(residual), _ptr(weight), _ptr(output), _ptr(residual_out),
-                                            _ptr(rstd), B, H, eps, dtype_code(x.dtype), L.stream),
+                                            _ptr(rstd), B, H, eps, dtype_code(x.dtype), block_size_b, L.stream),
             "ck_residual_rmsnorm_forward",
         )
 
@@ -336,7 +336,8 @@ def rmsnorm_backward_workspace_size(B: int, H: int, device: torch.device) -> int
         return lib.ck_rmsnorm_backward_workspace_size(B, H)
 
 
-def rmsnorm_backward(x, weight, output_grad, rstd, x_grad, weight_grad, workspace, eps: float) -> None:
+def rmsnorm_backward(x, weight, output_grad, rstd, x_grad, weight_grad, workspace, eps: float,
+                     block_size_b: int = 0) -> None:
     lib = load_library()
     _same_dtype(x, "rmsnorm_backward", weight=weight, output_grad=output_grad, x_grad=x_grad, weight_grad=weight_grad)
     H = x.size(-1)
@@ -346,7 +347,7 @@ def rmsnorm_backward(x, weight, output_grad, rstd, x_grad, weight_grad, workspac
             lib.ck_rmsnorm_backward(_ptr(x), _ptr(weight), _ptr(output_grad), _ptr(rstd), _ptr(x_grad),
                                     _ptr(weight_grad), _ptr(workspace),
                                     0 if workspace is None else workspace.numel() * workspace.element_size(), B, H,
-                                    eps, dtype_code(x.dtype), L.stream),
+                                    eps, dtype_code(x.dtype), block_size_b, L.stream),
             "ck_rmsnorm_backward",
         )
 

@@ -2,8 +2,12 @@
 
 Public function and autograd signature follow cute_kernels/kernels/rmsnorm/__init__.py:11-106 (1-D input,
 ``eps=None`` -> ``torch.finfo(dtype).eps``, optional weight, ``memory_efficient`` recomputation of 1/rms).
-The HIP kernels choose their own row tiling from the row length, so the BLOCK_SIZE_B / BLOCK_SIZE_H
-arguments of the reference are accepted for call compatibility and do not change the launch.
+BLOCK_SIZE_B (the reference's rows per program, tuned per dtype, row length and presence of a weight,
+kernels_forward.py:63-107 and kernels_backward.py:177-228) selects the launch variant of the kernels for rows that
+one wavefront holds: forward 1, 2, 4 rows requested at once by a wave that then ends, 8 waves that walk rows with
+the next one in flight; backward 1 two workgroups per compute unit, 2 one workgroup with the next row in flight.
+Every variant gives the same values; the tuner picks per (dtype, row length, weight).  BLOCK_SIZE_H is accepted for
+call compatibility: a row is always held whole.
 """
 
 import torch
@@ -11,7 +15,7 @@ import torch.nn.functional as F
 
 from .. import _C
 from ..constants import LIBRARY_NAME, MAX_ROW_LENGTH
-from ..cutotune import CutoTuneConfig, CutoTuneParameter, cutotune
+from ..cutotune import CutoTuneConfig, CutoTuneParameter, cutotune, get_cartesian_product_cutotune_configs
 from ..enums import KernelBackend
 from ..utils import cute_op, ensure_contiguous
 from ._common import check_backend
@@ -28,8 +32,9 @@ def rmsnorm_forward_hip(
     output: torch.Tensor,
     eps: float,
     rmsnorm_denominator: torch.Tensor | None,
+    BLOCK_SIZE_B: int = 0,
 ) -> None:
-    _C.rmsnorm_forward(x, weight, output, rmsnorm_denominator, eps)
+    _C.rmsnorm_forward(x, weight, output, rmsnorm_denominator, eps, BLOCK_SIZE_B)
 
 
 @cute_op(f"{LIBRARY_NAME}::rmsnorm_backward_hip", mutates_args={"x_grad", "weight_grad"})
@@ -41,6 +46,7 @@ def rmsnorm_backward_hip(
     x_grad: torch.Tensor,
     weight_grad: torch.Tensor | None,
     eps: float,
+    BLOCK_SIZE_B: int = 0,
 ) -> None:
     workspace = None
     if weight is not None:
@@ -49,15 +55,61 @@ def rmsnorm_backward_hip(
         num_rows = x.numel() // hidden_size if hidden_size > 0 else 0
         nbytes = _C.rmsnorm_backward_workspace_size(num_rows, hidden_size, x.device)
         workspace = torch.empty(max(nbytes, 16), device=x.device, dtype=torch.uint8)
-    _C.rmsnorm_backward(x, weight, output_grad, rmsnorm_denominator, x_grad, weight_grad, workspace, eps)
+    _C.rmsnorm_backward(x, weight, output_grad, rmsnorm_denominator, x_grad, weight_grad, workspace, eps, BLOCK_SIZE_B)
 
 
+# launch variants (see the module docstring)
+FORWARD_ROWS = [1, 2, 4, 8]
+BACKWARD_VARIANTS = [1, 2]
+# the reference's cache keys: dtype, row length, presence of a weight (kernels_forward.py:63-76)
+_TRIGGERS = {"x.dtype", "x.size(-1)"}
+_FUNCTIONAL_TRIGGERS = {"has_weight": lambda **kwargs: kwargs["weight"] is not None}
 _ONLY_CONFIG = CutoTuneConfig({"kernel_backend": KernelBackend.hip})
 
 
 def _check_row_length(hidden_size: int) -> None:
     if hidden_size > MAX_ROW_LENGTH:
         raise ValueError(f"hidden size ({hidden_size}) is larger than the longest supported row ({MAX_ROW_LENGTH})")
+
+
+# The reference tunes in two layers: the dispatcher picks the backend, the backend's launcher its BLOCK_SIZE_B
+# (forward.py:10-46 around kernels_forward.py:63-107).  Same here, so a caller may fix either without the other.
+@cutotune(
+    configs=get_cartesian_product_cutotune_configs(BLOCK_SIZE_B=FORWARD_ROWS),
+    default_config=CutoTuneConfig({"BLOCK_SIZE_B": 1}),
+    triggers=_TRIGGERS,
+    functional_triggers=_FUNCTIONAL_TRIGGERS,
+)
+def rmsnorm_forward_launch(
+    x: torch.Tensor,
+    weight: torch.Tensor | None,
+    output: torch.Tensor,
+    eps: float,
+    rmsnorm_denominator: torch.Tensor | None,
+    BLOCK_SIZE_B: int,
+) -> None:
+    rmsnorm_forward_hip(x=x, weight=weight, output=output, eps=eps, rmsnorm_denominator=rmsnorm_denominator,
+                        BLOCK_SIZE_B=BLOCK_SIZE_B)
+
+
+@cutotune(
+    configs=get_cartesian_product_cutotune_configs(BLOCK_SIZE_B=BACKWARD_VARIANTS),
+    default_config=CutoTuneConfig({"BLOCK_SIZE_B": 2}),
+    triggers=_TRIGGERS,
+    functional_triggers=_FUNCTIONAL_TRIGGERS,
+)
+def rmsnorm_backward_launch(
+    x: torch.Tensor,
+    weight: torch.Tensor | None,
+    output_grad: torch.Tensor,
+    rmsnorm_denominator: torch.Tensor | None,
+    x_grad: torch.Tensor,
+    weight_grad: torch.Tensor | None,
+    eps: float,
+    BLOCK_SIZE_B: int,
+) -> None:
+    rmsnorm_backward_hip(x=x, weight=weight, output_grad=output_grad, rmsnorm_denominator=rmsnorm_denominator,
+                         x_grad=x_grad, weight_grad=weight_grad, eps=eps, BLOCK_SIZE_B=BLOCK_SIZE_B)
 
 
 @cutotune(configs=[_ONLY_CONFIG], default_config=_ONLY_CONFIG, triggers={"x.dtype"})
@@ -77,7 +129,8 @@ def _forward(
 
     output = torch.empty_like(x)
     rmsnorm_denominator = None if memory_efficient else torch.empty(num_rows, device=x.device, dtype=torch.float32)
-    rmsnorm_forward_hip(x=x, weight=weight, output=output, eps=eps, rmsnorm_denominator=rmsnorm_denominator)
+    rmsnorm_forward_launch(x=x, weight=weight, output=output, eps=eps, rmsnorm_denominator=rmsnorm_denominator,
+                           BLOCK_SIZE_B=BLOCK_SIZE_B)
     return output, rmsnorm_denominator
 
 
@@ -98,7 +151,7 @@ def _backward(
 
     x_grad = torch.empty_like(x)
     weight_grad = None if weight is None else torch.empty_like(weight)
-    rmsnorm_backward_hip(
+    rmsnorm_backward_launch(
         x=x,
         weight=weight,
         output_grad=output_grad,
@@ -106,6 +159,7 @@ def _backward(
         x_grad=x_grad,
         weight_grad=weight_grad,
         eps=eps,
+        BLOCK_SIZE_B=BLOCK_SIZE_B,
     )
     return x_grad, weight_grad
 

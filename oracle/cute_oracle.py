@@ -405,6 +405,25 @@ def moe_forward_backward(x, w_gate, w_fc, w_proj, dy, top_k: int, compute_dtype=
     }
 
 
+def moe_expert_forward_backward(rows, gates, w_fc_e, w_proj_e, dy_rows, compute_dtype=torch.float32,
+                                activation=swiglu_unchunked_activation) -> dict:
+    """One expert of the layer on the rows routed to it: the loop body of Experts_Torch.forward
+    (torch_implementation.py:36-43) and the scaling by the routing weights (:161), differentiated.
+
+    rows [m, H] are the tokens that selected the expert, gates [m] their routing weights for it, dy_rows [m, H] the
+    gradient reaching those tokens' outputs.  Returns this expert's slices of the weight gradients (complete: no
+    other row contributes to them) and its contribution to the tokens' outputs and input gradients.
+    """
+    rows_ = rows.detach().to(compute_dtype).clone().requires_grad_(True)
+    w_fc_ = w_fc_e.detach().to(compute_dtype).clone().requires_grad_(True)
+    w_proj_ = w_proj_e.detach().to(compute_dtype).clone().requires_grad_(True)
+    out = F.linear(activation(F.linear(rows_, w_fc_)), w_proj_) * gates.to(compute_dtype).unsqueeze(-1)
+    (out * dy_rows.to(compute_dtype)).sum().backward()
+    dtype = rows.dtype
+    return {"out": out.detach().to(dtype), "d_rows": rows_.grad.to(dtype), "dw_fc": w_fc_.grad.to(dtype),
+            "dw_proj": w_proj_.grad.to(dtype)}
+
+
 def moe_dense_per_token(x, w_gate, w_fc, w_proj, top_k: int, activation=swiglu_unchunked_activation,
                         b_fc=None, b_proj=None):
     """Independent formulation used to pin ``moe_forward``: no sorting, no grouping.

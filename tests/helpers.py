@@ -50,3 +50,19 @@ def assert_close_long_sums(actual, expected, dtype, what=""):
     assert frac <= 1e-6, f"{what}: {frac:.2e} of the elements outside the tolerance"
     torch.testing.assert_close(actual.cpu(), expected.cpu(), rtol=3 * tol["rtol"], atol=3 * tol["atol"],
                                msg=lambda m: f"{what}: {m}")
+
+
+def assert_close_but_for(actual, expected, dtype, share, worst, what=""):
+    """Two 16-bit pipelines at the full BASELINE sizes.  A token's output (or input gradient) is the sum of k expert
+    rows of size O(1) that each implementation has rounded to 16 bits (2^-8 relative) before they are mixed, and a
+    weight gradient is a sum over thousands of rows of products of such rounded values: where the terms cancel, the
+    two results differ by a few units of the terms' last place while the tolerance follows the small sum.  Held to:
+    at most `share` of the elements outside the north-star tolerance, none outside `worst` times it, and the whole
+    tensor within 1e-2 norm-wise.  A wrong index or a dropped term moves a share of order one."""
+    tol = O.tolerance(dtype)
+    a, e = actual.detach().float().cpu(), expected.detach().float().cpu()
+    frac = O.fraction_outside(actual, expected, **tol)
+    assert frac <= share, f"{what}: {frac:.2e} of the elements outside the tolerance (allowed {share:.0e})"
+    ratio = ((a - e).abs() / (tol["atol"] + tol["rtol"] * e.abs())).max().item()
+    assert ratio <= worst, f"{what}: an element at {ratio:.1f} times the tolerance (allowed {worst})"
+    assert_norm_close(actual, expected, 1e-2, what)

@@ -51,26 +51,27 @@ def test_add_argument_checks(lib):
 
 
 def test_rmsnorm_argument_checks(lib):
-    assert lib.ck_rmsnorm_forward(P, None, P, None, 4, 65537, 1e-5, BF16, None) == SHAPE  # H above the limit
-    assert lib.ck_rmsnorm_forward(None, None, P, None, 4, 64, 1e-5, BF16, None) == NULL
-    assert lib.ck_rmsnorm_forward(P, None, P, None, 4, 64, 1e-5, 9, None) == DTYPE
-    assert lib.ck_rmsnorm_backward(P, P, P, None, P, None, P, 1 << 30, 4, 64, 1e-5, BF16, None) == NULL  # weight, no weight_grad
-    assert lib.ck_rmsnorm_backward(P, P, P, None, P, P, None, 0, 4, 64, 1e-5, BF16, None) == WORKSPACE
+    assert lib.ck_rmsnorm_forward(P, None, P, None, 4, 65537, 1e-5, BF16, 0, None) == SHAPE  # H above the limit
+    assert lib.ck_rmsnorm_forward(None, None, P, None, 4, 64, 1e-5, BF16, 0, None) == NULL
+    assert lib.ck_rmsnorm_forward(P, None, P, None, 4, 64, 1e-5, 9, 0, None) == DTYPE
+    assert lib.ck_rmsnorm_forward(P, None, P, None, 4, 64, 1e-5, BF16, -1, None) == SHAPE  # launch variants are 0, 1, 2, ...
+    assert lib.ck_rmsnorm_backward(P, P, P, None, P, None, P, 1 << 30, 4, 64, 1e-5, BF16, 0, None) == NULL  # weight, no weight_grad
+    assert lib.ck_rmsnorm_backward(P, P, P, None, P, P, None, 0, 4, 64, 1e-5, BF16, 0, None) == WORKSPACE
     need = lib.ck_rmsnorm_backward_workspace_size(4, 64)
     assert need > 0
-    assert lib.ck_rmsnorm_backward(P, P, P, None, P, P, P, need - 1, 4, 64, 1e-5, BF16, None) == WORKSPACE
-    assert lib.ck_rmsnorm_backward(P, P, P + 2, None, P, P, P, need, 4, 64, 1e-5, F32, None) == ALIGN
+    assert lib.ck_rmsnorm_backward(P, P, P, None, P, P, P, need - 1, 4, 64, 1e-5, BF16, 0, None) == WORKSPACE
+    assert lib.ck_rmsnorm_backward(P, P, P + 2, None, P, P, P, need, 4, 64, 1e-5, F32, 0, None) == ALIGN
 
 
 def test_residual_rmsnorm_argument_checks(lib):
     f = lib.ck_residual_rmsnorm_forward
-    #        x  res w     y  res_out rstd  B  H   eps   dtype stream
-    assert f(P, P, None, P, P, None, 4, 65537, 1e-5, BF16, None) == SHAPE
-    assert f(P, None, None, P, P, None, 4, 64, 1e-5, BF16, None) == NULL
-    assert f(P, P, None, P, None, None, 4, 64, 1e-5, BF16, None) == NULL
-    assert f(P, P, None, P, P, None, 4, 64, 1e-5, 9, None) == DTYPE
-    assert f(P, P + 1, None, P, P, None, 4, 64, 1e-5, BF16, None) == ALIGN
-    assert f(P, P, None, P, P, None, 0, 64, 1e-5, BF16, None) == OK  # no rows
+    #        x  res w     y  res_out rstd  B  H   eps   dtype variant stream
+    assert f(P, P, None, P, P, None, 4, 65537, 1e-5, BF16, 0, None) == SHAPE
+    assert f(P, None, None, P, P, None, 4, 64, 1e-5, BF16, 0, None) == NULL
+    assert f(P, P, None, P, None, None, 4, 64, 1e-5, BF16, 0, None) == NULL
+    assert f(P, P, None, P, P, None, 4, 64, 1e-5, 9, 0, None) == DTYPE
+    assert f(P, P + 1, None, P, P, None, 4, 64, 1e-5, BF16, 0, None) == ALIGN
+    assert f(P, P, None, P, P, None, 0, 64, 1e-5, BF16, 0, None) == OK  # no rows
 
 
 def test_embedding_argument_checks(lib):

@@ -411,6 +411,44 @@ def test_residual_rmsnorm_against_autograd_of_the_composition():
     assert torch.allclose(dx0, O.rmsnorm_backward(x + r, None, dy, eps, compute_dtype=F64)[0], rtol=0, atol=0)
 
 
+def test_moe_one_expert_slices_against_the_layer_and_a_hand_written_sum():
+    """moe_expert_forward_backward (one expert on the rows routed to it) is pinned by the layer restatement, itself
+    pinned by the per-token formulation above: its weight gradients are that expert's slices of the layer's, the
+    token outputs are the sum of the experts' contributions; and by the outer-product form dW_proj = sum_t g_t
+    dy_t act_t^T written out as a loop."""
+    T, H, I, E, k = 23, 8, 6, 5, 3
+    x, wg, wfc, wproj, dy = (t.double() for t in O.moe_inputs(T, H, I, E, torch.float32, seed=12))
+    wg = wg * 20
+    res = O.moe_forward_backward(x, wg, wfc, wproj, dy, k, compute_dtype=F64)
+    logits = x @ wg.T
+    vals, sel = logits.topk(k, dim=-1)
+    weights = torch.softmax(vals, dim=-1)
+    y = torch.zeros(T, H, dtype=F64)
+    dx_experts = torch.zeros(T, H, dtype=F64)
+    for e in range(E):
+        tok, slot = (sel == e).nonzero(as_tuple=True)
+        one = O.moe_expert_forward_backward(x[tok], weights[tok, slot], wfc[e], wproj[e], dy[tok], compute_dtype=F64)
+        assert torch.allclose(one["dw_fc"], res["dw_fc"][e], rtol=1e-10, atol=1e-12), e
+        assert torch.allclose(one["dw_proj"], res["dw_proj"][e], rtol=1e-10, atol=1e-12), e
+        y.index_add_(0, tok, one["out"])
+        dx_experts.index_add_(0, tok, one["d_rows"])
+        if e == 0 and tok.numel():
+            h = x[tok] @ wfc[e].T
+            act = h[:, :I] * F.silu(h[:, I:])
+            by_hand = sum(weights[t, s] * torch.outer(dy[t], act[i]) for i, (t, s) in enumerate(zip(tok.tolist(), slot.tolist())))
+            assert torch.allclose(one["dw_proj"], by_hand, rtol=1e-10, atol=1e-12)
+    assert torch.allclose(y, res["y"], rtol=1e-10, atol=1e-12)
+    # dx = the experts' part plus the router's part; the latter vanishes where the routing weights get no gradient
+    res1 = O.moe_forward_backward(x, wg, wfc, wproj, dy, 1, compute_dtype=F64)
+    sel1 = logits.argmax(-1)
+    dx1 = torch.zeros(T, H, dtype=F64)
+    for e in range(E):
+        tok = (sel1 == e).nonzero().flatten()
+        one = O.moe_expert_forward_backward(x[tok], torch.ones(tok.numel(), dtype=F64), wfc[e], wproj[e], dy[tok], compute_dtype=F64)
+        dx1.index_add_(0, tok, one["d_rows"])
+    assert torch.allclose(dx1, res1["dx"], rtol=1e-10, atol=1e-12)
+
+
 def test_moe_single_expert_is_a_plain_mlp():
     T, H, I = 7, 8, 5
     x, wg, wfc, wproj, dy = (t.double() for t in O.moe_inputs(T, H, I, 1, torch.float32, seed=4))
