@@ -9,7 +9,8 @@
 //                  per 9-bit digit), then one workgroup marks which table rows are selected at all
 //                  and records, for every sorted slot, the first slot of its run of equal ids.
 //               2. rows kernel, one launch for two jobs: rows no id selects are written as zeros (the
-//                  bulk of the traffic); a run of equal ids is cut into chunks of kChunk slots and one
+//                  bulk of the traffic; a part of them rides, as extra workgroups, on the small launches
+//                  of step 1 that come after the rows are marked); a run of equal ids is cut into chunks of kChunk slots and one
 //                  wave sums the dy rows of a chunk in fp32 registers, in ascending token position.  A
 //                  run that fits one chunk is rounded and stored straight into dW; longer runs leave
 //                  one fp32 partial row per chunk in the workspace.
@@ -133,37 +134,98 @@ struct PairStorer {
     }
 };
 
+// Zero fill of the table rows no id selects, as a side job of the launches that come after the row marks are known.
+// Those launches (the sort's scatter / histogram / scan kernels, the run heads) are a handful of workgroups each and
+// bound by latency, about 8 us apiece and one behind the other; the fill is the bulk of the operator's bytes and needs
+// nothing from them but the marks.  Each of them gets a share of the table's rows as extra workgroups behind its own
+// (`first_block` on), so the sort no longer costs time of its own.  One wave takes four consecutive rows: the four
+// marks first, then 16-byte packets of zeros (zero bits are zero in every storage type).
+struct FillJob {
+    const uint8_t* touched;
+    char* dw;
+    int64_t row_bytes;            // a multiple of 16
+    int64_t row_begin, row_end;   // this launch's share of the rows
+    int first_block;              // workgroups [first_block, gridDim.x) belong to the job
+};
+constexpr int kFillRowsPerWave = 4;
+
+__device__ __forceinline__ bool run_fill_job(const FillJob& f) {
+    if ((int)blockIdx.x < f.first_block) return false;
+    typedef uint32_t zero_t __attribute__((ext_vector_type(4)));
+    const int lane = lane_id();
+    const int waves = blockDim.x / CK_WAVE;
+    const int64_t row0 =
+        f.row_begin + (((int64_t)blockIdx.x - f.first_block) * waves + threadIdx.x / CK_WAVE) * kFillRowsPerWave;
+    uint8_t mark[kFillRowsPerWave];
+#pragma unroll
+    for (int r = 0; r < kFillRowsPerWave; ++r) mark[r] = row0 + r < f.row_end ? f.touched[row0 + r] : 1;
+    const zero_t z = {0u, 0u, 0u, 0u};
+    const int64_t packs = f.row_bytes / 16;
+#pragma unroll
+    for (int r = 0; r < kFillRowsPerWave; ++r) {
+        if (mark[r]) continue;
+        zero_t* dst = reinterpret_cast<zero_t*>(f.dw + (row0 + r) * f.row_bytes);
+        for (int64_t p = lane; p < packs; p += CK_WAVE) dst[p] = z;
+    }
+    return true;
+}
+// workgroups a launch with `threads` lanes per workgroup needs for the job's rows
+static inline int64_t fill_job_blocks(int64_t rows, int threads) {
+    const int64_t per_block = (int64_t)(threads / CK_WAVE) * kFillRowsPerWave;
+    return (rows + per_block - 1) / per_block;
+}
+
 template <typename Loader>
 __global__ void __launch_bounds__(256)
     embedding_sort_hist_kernel(Loader load, int n, int shift, int bits, uint32_t* __restrict__ hist, int num_waves,
-                               uint32_t* __restrict__ clear, int64_t clear_words) {
+                               uint32_t* __restrict__ clear, int64_t clear_words, FillJob fill) {
     __shared__ GridSortShared sh;
+    if (run_fill_job(fill)) return;
     // side job of the first pass: clear the row marks
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < clear_words; i += (int64_t)gridDim.x * blockDim.x)
         clear[i] = 0u;
     grid_sort_histogram(sh, n, shift, bits, hist, num_waves, load);
 }
 
-__global__ void __launch_bounds__(1024) embedding_sort_scan_kernel(uint32_t* __restrict__ hist, int total) {
-    grid_sort_scan(hist, total);
+// Workgroup 0 scans the histogram.  In the first pass the workgroups behind it mark the table rows some id selects
+// (the marks were cleared by the launch before; Loader gives the key V to ids outside the table); in later passes
+// they carry a share of the zero fill.
+template <typename Loader, bool MARK>
+__global__ void __launch_bounds__(1024)
+    embedding_sort_scan_kernel(uint32_t* __restrict__ hist, int total, Loader load, int n, int64_t V,
+                               uint8_t* __restrict__ touched, FillJob fill) {
+    if (blockIdx.x == 0) {
+        grid_sort_scan(hist, total);
+        return;
+    }
+    if (MARK) {
+        const int64_t stride = (int64_t)(gridDim.x - 1) * blockDim.x;
+        for (int64_t i = (int64_t)(blockIdx.x - 1) * blockDim.x + threadIdx.x; i < n; i += stride) {
+            uint32_t key, val;
+            load((int)i, key, val);
+            if ((int64_t)key < V) touched[key] = 1;
+        }
+    } else {
+        run_fill_job(fill);
+    }
 }
 
 template <typename Loader>
 __global__ void __launch_bounds__(256)
     embedding_sort_scatter_kernel(Loader load, PairStorer store, int n, int shift, int bits,
-                                  const uint32_t* __restrict__ offsets, int num_waves) {
+                                  const uint32_t* __restrict__ offsets, int num_waves, FillJob fill) {
     __shared__ GridSortShared sh;
+    if (run_fill_job(fill)) return;
     grid_sort_scatter(sh, n, shift, bits, offsets, num_waves, load, store);
 }
 
-// Runs of equal ids in the sorted order: marks the table rows that are selected at all and records, for every
-// sorted slot, the first slot of its run.  Every wave owns kRunsWaveSlots consecutive slots: it first looks
+// Runs of equal ids in the sorted order: records, for every sorted slot, the first slot of its run.  Every wave owns kRunsWaveSlots consecutive slots: it first looks
 // backwards from its first slot, 64 slots at a time, for the head of the run it starts in, then walks its
 // slots 64 at a time carrying the latest head forward with a wave max-scan.
 constexpr int kRunsWaveSlots = 4 * CK_WAVE;
 __global__ void __launch_bounds__(256)
-    embedding_runs_kernel(const uint32_t* __restrict__ skeys, uint32_t* __restrict__ run_head, uint8_t* __restrict__ touched,
-                          int n, int64_t V) {
+    embedding_runs_kernel(const uint32_t* __restrict__ skeys, uint32_t* __restrict__ run_head, int n, FillJob fill) {
+    if (run_fill_job(fill)) return;
     const int lane = lane_id();
     const int gw = (blockIdx.x * blockDim.x + threadIdx.x) / CK_WAVE;
     const int begin = gw * kRunsWaveSlots;
@@ -183,10 +245,7 @@ __global__ void __launch_bounds__(256)
         int head = -1;
         if (i < end) {
             const uint32_t k = skeys[i];
-            if (i == 0 || skeys[i - 1] != k) {
-                head = i;
-                if ((int64_t)k < V) touched[k] = 1;
-            }
+            if (i == 0 || skeys[i - 1] != k) head = i;
         }
         const int incl = max(wave_inclusive_max_i(head), carry);
         if (i < end) run_head[i] = (uint32_t)incl;
@@ -206,14 +265,15 @@ __global__ void __launch_bounds__(256)
     embedding_bwd_rows_kernel(const uint32_t* __restrict__ skeys, const uint32_t* __restrict__ spos,
                               const uint32_t* __restrict__ run_head, const uint8_t* __restrict__ touched,
                               const typename T::storage_t* __restrict__ dy, typename T::storage_t* __restrict__ dw,
-                              float* __restrict__ partial, int n, int chunk_groups, int64_t V, int64_t H) {
+                              float* __restrict__ partial, int n, int chunk_groups, int64_t V, int64_t H,
+                              int64_t fill_begin) {
     typedef VPack<T, VEC> P;
     const int lane = lane_id();
     const int64_t packs = H / VEC;
 
     if ((int)blockIdx.x >= chunk_groups) {
-        // ---- zero fill ----
-        const int64_t row = (int64_t)(blockIdx.x - chunk_groups) * 4 + threadIdx.x / CK_WAVE;
+        // ---- zero fill of the rows [fill_begin, V): what the launches before this one did not carry ----
+        const int64_t row = fill_begin + (int64_t)(blockIdx.x - chunk_groups) * 4 + threadIdx.x / CK_WAVE;
         if (row >= V) return;
         if (touched[row]) return;
         P z;
@@ -241,6 +301,28 @@ __global__ void __launch_bounds__(256)
     const int cnt = __ffsll((unsigned long long)~bal) - 1;  // lane 0 always matches, so cnt >= 1
     const bool continues = cnt == kChunk && __shfl(key_l, kChunk, CK_WAVE) == id;
     const bool multi = (i != head) || continues;
+
+    if (cnt == 1 && !multi) {
+        // the only row of its id (nearly every slot when ids are spread over a large table): widened and rounded
+        // back, the row comes out as it went in, so it is copied - eight packets per lane in flight, no accumulators
+        const uint32_t pos = __shfl(pos_l, 0, CK_WAVE);
+        const P* src = reinterpret_cast<const P*>(dy + (int64_t)pos * H);
+        P* dst = reinterpret_cast<P*>(dw + (int64_t)id * H);
+        for (int64_t p0 = 0; p0 < packs; p0 += (int64_t)CK_WAVE * kRowPacks) {
+            P v[kRowPacks];
+#pragma unroll
+            for (int q = 0; q < kRowPacks; ++q) {
+                const int64_t p = p0 + lane + (int64_t)q * CK_WAVE;
+                if (p < packs) v[q] = nt_load(src + p);
+            }
+#pragma unroll
+            for (int q = 0; q < kRowPacks; ++q) {
+                const int64_t p = p0 + lane + (int64_t)q * CK_WAVE;
+                if (p < packs) nt_store(v[q], dst + p);
+            }
+        }
+        return;
+    }
 
     // fp32 tables sum in fp64 so that the result is the correctly rounded sum whatever the order
     typedef typename AccOf<T>::type acc_t;
@@ -399,16 +481,21 @@ extern "C" int64_t ck_embedding_backward_workspace_size(int64_t num_ids, int64_t
     return ck::emb_carve(nullptr, num_ids, V, H, nullptr);
 }
 
+// (measured at a table of [128256, 4096] and 32768 ids: 313 us without, 306 / 297 / 292 / 306 us with 20 / 40 / 80 / 160 MB)
+constexpr int64_t kCarrierFillBytes = (int64_t)80 << 20;
+
 template <typename T, int VEC>
 static void launch_bwd(hipStream_t s, const ck::EmbWorkspace& ws, int passes, const void* dy, void* dw, int n,
-                       int64_t V, int64_t H) {
+                       int64_t V, int64_t H, int64_t fill_begin) {
     typedef typename T::storage_t S;
     const uint32_t* skeys = ws.keys[(passes - 1) & 1];
     const uint32_t* spos = ws.vals[(passes - 1) & 1];
     const int chunk_groups = (int)ck_ceil_div(n, 4);
-    const int64_t fill_groups = ck_ceil_div(V, 4);
-    hipLaunchKernelGGL((ck::embedding_bwd_rows_kernel<T, VEC>), dim3((unsigned)(chunk_groups + fill_groups)), dim3(256), 0,
-                       s, skeys, spos, ws.run_head, ws.touched, (const S*)dy, (S*)dw, ws.partial, n, chunk_groups, V, H);
+    const int64_t fill_groups = ck_ceil_div(V - fill_begin, 4);
+    if (chunk_groups + fill_groups > 0)
+        hipLaunchKernelGGL((ck::embedding_bwd_rows_kernel<T, VEC>), dim3((unsigned)(chunk_groups + fill_groups)), dim3(256),
+                           0, s, skeys, spos, ws.run_head, ws.touched, (const S*)dy, (S*)dw, ws.partial, n, chunk_groups, V, H,
+                           fill_begin);
     if (n > 0)
         hipLaunchKernelGGL((ck::embedding_bwd_combine_kernel<T>), dim3((unsigned)ck_ceil_div(n, CK_WAVE), ck::kCombineParts),
                            dim3(256), 0, s, skeys, ws.run_head, ws.partial, (S*)dw, n, V, H);
@@ -436,44 +523,82 @@ extern "C" int ck_embedding_backward(const void* ids, int ids_are_i32, const voi
     const int num_waves = ck::grid_sort_waves(n);
     const unsigned sort_grid = (unsigned)(num_waves > 0 ? ck_ceil_div(num_waves, ck::kGridSortBlockWaves) : 1);
     const int64_t clear_words = (V + 3) / 4;
+    // The zero fill of the rows nobody selects rides on the launches between the marking of the rows (second launch)
+    // and the row sums: the first pass's scatter, the three launches of every further pass, the run heads.  Needs rows
+    // of whole 16-byte packets; otherwise (and without ids) the rows kernel fills, as it sums.
+    const int64_t row_bytes = H * ck_elem_size(dtype);
+    const bool spread_fill = n > 0 && row_bytes % 16 == 0 && ck_aligned16(weight_grad);
+    const int carriers = 1 + 3 * (passes - 1) + 1;
+    // a carrier's own work leaves most of the GPU idle for about 8 us: that much fill is free, more only moves time
+    // from the row-sum launch, where the fill hides the latency of the sums, to here
+    int64_t spread_rows = spread_fill ? carriers * (kCarrierFillBytes / row_bytes) : 0;
+    if (spread_rows > V) spread_rows = V;
+    int carrier = 0;
+    auto fill_share = [&](int own_blocks, int threads, unsigned& grid) {
+        ck::FillJob f = {ws.touched, (char*)weight_grad, row_bytes, 0, 0, 0x7fffffff};
+        grid = (unsigned)own_blocks;
+        if (spread_fill) {
+            f.row_begin = spread_rows * carrier / carriers;
+            f.row_end = spread_rows * (carrier + 1) / carriers;
+            f.first_block = own_blocks;
+            grid = (unsigned)(own_blocks + ck::fill_job_blocks(f.row_end - f.row_begin, threads));
+            ++carrier;
+        }
+        return f;
+    };
+    const ck::FillJob no_fill = {ws.touched, (char*)weight_grad, row_bytes, 0, 0, 0x7fffffff};
+    // workgroups of the second launch that mark the selected rows (behind the one that scans)
+    const unsigned mark_blocks = (unsigned)(n > 0 ? ck_ceil_div(n, 4 * 1024) : 0);
     for (int p = 0; p < passes; ++p) {
         const int shift = p * bits_per_pass;
         const int bits = key_bits - shift < bits_per_pass ? key_bits - shift : bits_per_pass;
         const int total = (1 << bits) * num_waves;
         ck::PairStorer store = {ws.keys[p & 1], ws.vals[p & 1]};
+        unsigned grid = 0;
         if (p == 0) {
             // the clear of the row marks rides on the first histogram launch (needs at least one workgroup)
             if (ids_are_i32) {
                 ck::IdLoader<true> load = {ids, V};
                 hipLaunchKernelGGL((ck::embedding_sort_hist_kernel<ck::IdLoader<true>>), dim3(sort_grid), dim3(256), 0, s,
-                                   load, n, shift, bits, ws.hist, num_waves, (uint32_t*)ws.touched, clear_words);
-                hipLaunchKernelGGL(ck::embedding_sort_scan_kernel, dim3(1), dim3(1024), 0, s, ws.hist, total);
-                hipLaunchKernelGGL((ck::embedding_sort_scatter_kernel<ck::IdLoader<true>>), dim3(sort_grid), dim3(256), 0,
-                                   s, load, store, n, shift, bits, ws.hist, num_waves);
+                                   load, n, shift, bits, ws.hist, num_waves, (uint32_t*)ws.touched, clear_words, no_fill);
+                hipLaunchKernelGGL((ck::embedding_sort_scan_kernel<ck::IdLoader<true>, true>), dim3(1 + mark_blocks),
+                                   dim3(1024), 0, s, ws.hist, total, load, n, V, ws.touched, no_fill);
+                const ck::FillJob f = fill_share((int)sort_grid, 256, grid);
+                hipLaunchKernelGGL((ck::embedding_sort_scatter_kernel<ck::IdLoader<true>>), dim3(grid), dim3(256), 0, s,
+                                   load, store, n, shift, bits, ws.hist, num_waves, f);
             } else {
                 ck::IdLoader<false> load = {ids, V};
                 hipLaunchKernelGGL((ck::embedding_sort_hist_kernel<ck::IdLoader<false>>), dim3(sort_grid), dim3(256), 0, s,
-                                   load, n, shift, bits, ws.hist, num_waves, (uint32_t*)ws.touched, clear_words);
-                hipLaunchKernelGGL(ck::embedding_sort_scan_kernel, dim3(1), dim3(1024), 0, s, ws.hist, total);
-                hipLaunchKernelGGL((ck::embedding_sort_scatter_kernel<ck::IdLoader<false>>), dim3(sort_grid), dim3(256), 0,
-                                   s, load, store, n, shift, bits, ws.hist, num_waves);
+                                   load, n, shift, bits, ws.hist, num_waves, (uint32_t*)ws.touched, clear_words, no_fill);
+                hipLaunchKernelGGL((ck::embedding_sort_scan_kernel<ck::IdLoader<false>, true>), dim3(1 + mark_blocks),
+                                   dim3(1024), 0, s, ws.hist, total, load, n, V, ws.touched, no_fill);
+                const ck::FillJob f = fill_share((int)sort_grid, 256, grid);
+                hipLaunchKernelGGL((ck::embedding_sort_scatter_kernel<ck::IdLoader<false>>), dim3(grid), dim3(256), 0, s,
+                                   load, store, n, shift, bits, ws.hist, num_waves, f);
             }
         } else {
             ck::PairLoader load = {ws.keys[(p + 1) & 1], ws.vals[(p + 1) & 1]};
-            hipLaunchKernelGGL((ck::embedding_sort_hist_kernel<ck::PairLoader>), dim3(sort_grid), dim3(256), 0, s, load, n,
-                               shift, bits, ws.hist, num_waves, (uint32_t*)nullptr, (int64_t)0);
-            hipLaunchKernelGGL(ck::embedding_sort_scan_kernel, dim3(1), dim3(1024), 0, s, ws.hist, total);
-            hipLaunchKernelGGL((ck::embedding_sort_scatter_kernel<ck::PairLoader>), dim3(sort_grid), dim3(256), 0, s, load,
-                               store, n, shift, bits, ws.hist, num_waves);
+            ck::FillJob f = fill_share((int)sort_grid, 256, grid);
+            hipLaunchKernelGGL((ck::embedding_sort_hist_kernel<ck::PairLoader>), dim3(grid), dim3(256), 0, s, load, n, shift,
+                               bits, ws.hist, num_waves, (uint32_t*)nullptr, (int64_t)0, f);
+            f = fill_share(1, 1024, grid);
+            hipLaunchKernelGGL((ck::embedding_sort_scan_kernel<ck::PairLoader, false>), dim3(grid), dim3(1024), 0, s, ws.hist,
+                               total, load, n, V, ws.touched, f);
+            f = fill_share((int)sort_grid, 256, grid);
+            hipLaunchKernelGGL((ck::embedding_sort_scatter_kernel<ck::PairLoader>), dim3(grid), dim3(256), 0, s, load, store,
+                               n, shift, bits, ws.hist, num_waves, f);
         }
     }
-    if (n > 0)
-        hipLaunchKernelGGL(ck::embedding_runs_kernel, dim3((unsigned)ck_ceil_div(n, 4 * ck::kRunsWaveSlots)), dim3(256), 0,
-                           s, ws.keys[(passes - 1) & 1], ws.run_head, ws.touched, n, V);
+    if (n > 0) {
+        unsigned grid = 0;
+        const ck::FillJob f = fill_share((int)ck_ceil_div(n, 4 * ck::kRunsWaveSlots), 256, grid);
+        hipLaunchKernelGGL(ck::embedding_runs_kernel, dim3(grid), dim3(256), 0, s, ws.keys[(passes - 1) & 1], ws.run_head, n,
+                           f);
+    }
     CK_DISPATCH_DTYPE(dtype, {
         const bool vec = ck_aligned16(weight_grad) && (!output_grad || ck_aligned16(output_grad)) && (H % T::kVec == 0);
-        if (vec) launch_bwd<T, T::kVec>(s, ws, passes, output_grad, weight_grad, (int)num_ids, V, H);
-        else launch_bwd<T, 1>(s, ws, passes, output_grad, weight_grad, (int)num_ids, V, H);
+        if (vec) launch_bwd<T, T::kVec>(s, ws, passes, output_grad, weight_grad, (int)num_ids, V, H, spread_rows);
+        else launch_bwd<T, 1>(s, ws, passes, output_grad, weight_grad, (int)num_ids, V, H, spread_rows);
     });
     return ck_launch_status();
 }

@@ -741,6 +741,7 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
         row_start = 0;
         rows_valid = min(BM, p.K - i_base);
     }
+    const bool upper_rows_live = rows_valid > BM / 2;  // the same for every wave of the workgroup
     static_assert(GLU == 0 || !GROUP_K, "the fused activation belongs to the per-expert products");
     static_assert(GLU != 1 || B_KC, "the forward fusion reads the weight with the contraction contiguous");
     // GLU == 1: a tile holds BN / 2 "up" columns n_base .. and the BN / 2 "gate" columns glu_half + n_base ..
@@ -966,9 +967,11 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
         mma_quad(0, 0, fa, fb0);
         mma_quad(0, 1, fa, fb1);
         __builtin_amdgcn_sched_barrier(0);
-        read_a(st, 1, fa);
-        mma_quad(1, 1, fa, fb1);
-        mma_quad(1, 0, fa, fb0);
+        if (upper_rows_live) {
+            read_a(st, 1, fa);
+            mma_quad(1, 1, fa, fb1);
+            mma_quad(1, 0, fa, fb0);
+        }
     };
 
     // ---- the pipelined loop ----------------------------------------------------------------------------
@@ -1004,7 +1007,11 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
     } while (0)
     const int k_tiles = (k_end - k_begin + BK - 1) / BK;
     const int n_full = (k_end - k_begin) / BK;  // leading tiles that lie completely inside the range
-    auto pp_step = [&](int kt, char* X, char* Y, frag_t (*bl)[TNH], frag_t (*bu)[TNH]) __attribute__((always_inline)) {
+    // `upper` says, as a type, whether the upper half of the tile's rows holds any row of the segment: where it holds
+    // none (the last row tile of an expert with at most BM / 2 rows left) its fragments are not read and its matrix
+    // instructions not issued, while barriers and copies stay as they are, so the counts of the waits still hold.
+    auto pp_step = [&](auto upper, int kt, char* X, char* Y, frag_t (*bl)[TNH], frag_t (*bu)[TNH]) __attribute__((always_inline)) {
+        constexpr bool UPPER = decltype(upper)::value;
         // The last two steps of a range have no tile left to request; they request the last tile once more, into
         // halves that nobody reads again, which keeps the count of outstanding copies the same in every step (a
         // branch around the copies, with its own wait, measured slower than the 2 / 64 of copy work it saves).
@@ -1021,10 +1028,10 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
         mma_quad(0, 1, fa, bu);
         __builtin_amdgcn_s_setprio(0);
         CK_PHASE_END();
-        read_a(X, 1, fa);
+        if (UPPER) read_a(X, 1, fa);
         CK_M_END(3);
         __builtin_amdgcn_s_setprio(1);
-        mma_quad(1, 1, fa, bu);
+        if (UPPER) mma_quad(1, 1, fa, bu);
         __builtin_amdgcn_s_setprio(0);
         CK_PHASE_END();
         // lower columns of the next tile, over the registers of this tile's upper columns (after the last tile of a
@@ -1032,7 +1039,7 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
         read_b(Y, 0, bu);
         CK_M_END(1);
         __builtin_amdgcn_s_setprio(1);
-        mma_quad(1, 0, fa, bl);
+        if (UPPER) mma_quad(1, 0, fa, bl);
         __builtin_amdgcn_s_setprio(0);
         CK_PHASE_END();
     };
@@ -1057,9 +1064,16 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
         CK_PHASE_END();
         if (wm == 1) CK_PHASE_END();  // the upper group falls one phase behind
         // two steps per turn so that each names its buffers and registers statically
-        for (; kt + 1 < n_full; kt += 2) {
-            pp_step(kt, lds0, lds1, fb0, fb1);
-            pp_step(kt + 1, lds1, lds0, fb1, fb0);
+        if (upper_rows_live) {
+            for (; kt + 1 < n_full; kt += 2) {
+                pp_step(std::true_type{}, kt, lds0, lds1, fb0, fb1);
+                pp_step(std::true_type{}, kt + 1, lds1, lds0, fb1, fb0);
+            }
+        } else {
+            for (; kt + 1 < n_full; kt += 2) {
+                pp_step(std::false_type{}, kt, lds0, lds1, fb0, fb1);
+                pp_step(std::false_type{}, kt + 1, lds1, lds0, fb1, fb0);
+            }
         }
         if (wm == 0) CK_PHASE_END();
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
