@@ -223,6 +223,7 @@ def bench_moe_skewed(device, steps=10, warmup=3):
 
 def bench_extras(device):
     from cute_kernels import KernelBackend
+    from cute_kernels.cutotune import CutoTuneParameter
     from cute_kernels.kernels import embedding as EM
     from cute_kernels.kernels import rmsnorm as RN
     from cute_kernels.kernels import swiglu as SW
@@ -241,12 +242,13 @@ def bench_extras(device):
     xs = [torch.randn(B, H, device=device, dtype=dtype) for _ in range(sets)]
     dys = [torch.randn(B, H, device=device, dtype=dtype) for _ in range(sets)]
     w = (torch.randn(H, device=device) * 0.1 + 1).to(dtype)
-    rstd = RN._forward(x=xs[0], weight=w, eps=1e-5, memory_efficient=False, kernel_backend=hip, BLOCK_SIZE_B=1, BLOCK_SIZE_H=H)[1]
+    tuned = CutoTuneParameter()  # the launch variant comes from the package's tuning cache
+    rstd = RN._forward(x=xs[0], weight=w, eps=1e-5, memory_efficient=False, kernel_backend=hip, BLOCK_SIZE_B=tuned, BLOCK_SIZE_H=H)[1]
     ms = _time_rotating(lambda i: RN._forward(x=xs[i % sets], weight=w, eps=1e-5, memory_efficient=False,
-                                              kernel_backend=hip, BLOCK_SIZE_B=1, BLOCK_SIZE_H=H), sets)
+                                              kernel_backend=hip, BLOCK_SIZE_B=tuned, BLOCK_SIZE_H=H), sets)
     out["rmsnorm_fwd"] = gbs(2 * B * H * 2 + H * 2 + B * 4, ms)
     ms = _time_rotating(lambda i: RN._backward(x=xs[i % sets], weight=w, eps=1e-5, rmsnorm_denominator=rstd,
-                                               output_grad=dys[i % sets], kernel_backend=hip, BLOCK_SIZE_B=1, BLOCK_SIZE_H=H), sets)
+                                               output_grad=dys[i % sets], kernel_backend=hip, BLOCK_SIZE_B=tuned, BLOCK_SIZE_H=H), sets)
     out["rmsnorm_bwd"] = gbs(3 * B * H * 2 + 2 * H * 2 + B * 4, ms)
     # residual addition + RMSNorm in one pass on the same shape: two rows read, two written
     from cute_kernels.kernels.fused_residual_add_rmsnorm import fused_residual_add_rmsnorm_forward_hip

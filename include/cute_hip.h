@@ -169,12 +169,15 @@ int ck_moe_sort_noalloc(const void* expert_ids, int ids_are_i32, int64_t* sorted
  * X is [*, K] with row stride x_stride (elements, K contiguous); W is a strided view [E, K, N] with
  * element strides (w_stride_e, w_stride_k, w_stride_n), one of w_stride_k / w_stride_n being 1;
  * out is [num_slots, N] with row stride out_stride.  expert_offsets is int64 [E] (inclusive ends).
+ * bias is NULL or [E, N] contiguous, of the operands' type: out[out_row(i), :] then also gets bias[e(i), :], added
+ * to the fp32 sums before they are rounded - the bias of the reference's per-expert F.linear
+ * (scattermoe/torch_implementation.py:35-43; its Triton experts carry none).
  * ------------------------------------------------------------------------------------------- */
 int ck_scatter2scatter(const void* X, int64_t x_stride, const void* W, int64_t w_stride_e,
                        int64_t w_stride_k, int64_t w_stride_n, const int64_t* sorted_scattered_idxs,
                        const int64_t* expert_offsets, void* out, int64_t out_stride, int64_t num_slots,
                        int64_t K, int64_t N, int64_t E, int64_t fan_out, int x_grouped, int y_grouped,
-                       int dtype, void* stream);
+                       const void* bias, int dtype, void* stream);
 
 /* The same product with the tail of the tile grid split along the contraction (no counterpart in the reference).
  * A product with few column tiles leaves most CUs idle during its last round of tiles; given a workspace of
@@ -186,8 +189,8 @@ int64_t ck_scatter2scatter_workspace_size(int64_t num_slots, int64_t K, int64_t 
 int ck_scatter2scatter_ws(const void* X, int64_t x_stride, const void* W, int64_t w_stride_e, int64_t w_stride_k,
                           int64_t w_stride_n, const int64_t* sorted_scattered_idxs, const int64_t* expert_offsets,
                           void* out, int64_t out_stride, int64_t num_slots, int64_t K, int64_t N, int64_t E,
-                          int64_t fan_out, int x_grouped, int y_grouped, int dtype, void* workspace,
-                          int64_t workspace_bytes, void* stream);
+                          int64_t fan_out, int x_grouped, int y_grouped, const void* bias, int dtype,
+                          void* workspace, int64_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * scatter2scatter with the SwiGLU of the MoE layer in its epilogue.

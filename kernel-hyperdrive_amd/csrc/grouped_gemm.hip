@@ -74,6 +74,9 @@ struct GemmParams {
     // Tail splitting of the per-expert products (kernel template argument MODE, see find_tile_split): fp32 partial
     // tiles, kSplitSlots of them, BM * BN floats each
     float* partials;
+    // S2S without activation: bias [E, N] of the operands' type, or null.  Added to the fp32 sums before they are
+    // rounded, as F.linear(rows, W[e], bias[e]) rounds once (cute_kernels/kernels/scattermoe/torch_implementation.py:35-43).
+    const void* bias;
 };
 
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -585,7 +588,10 @@ __global__ void __launch_bounds__(TL::THREADS) grouped_gemm_kernel(GemmParams p)
             for (int r = 0; r < 16; ++r) {
                 const int row = wm * (BM / WM) + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
                 const int col = wn * (BN / WN) + j * 32 + lane % 32;
-                Ct[row * C_LD + col] = T::down(acc[i][j][r]);
+                float v = acc[i][j][r];
+                if (!GROUP_K && p.bias != nullptr)
+                    v += T::up(reinterpret_cast<const S*>(p.bias)[(int64_t)expert * p.N + min(n_base + col, p.N - 1)]);
+                Ct[row * C_LD + col] = T::down(v);
             }
     __syncthreads();
     S* Cbase = reinterpret_cast<S*>(p.C) + (GROUP_K ? (int64_t)expert * p.c_stride_e : 0);
@@ -662,6 +668,15 @@ __device__ __forceinline__ uint32_t pack2(float a, float b) {
     uint32_t w;
     __builtin_memcpy(&w, &h, 4);
     return w;
+}
+
+// the reverse: the two storage values of a dword as fp32
+template <typename T>
+__device__ __forceinline__ void unpack2(uint32_t w, float& a, float& b) {
+    typename T::storage_t h[2];
+    __builtin_memcpy(h, &w, 4);
+    a = T::up(h[0]);
+    b = T::up(h[1]);
 }
 
 // MODE 0: one workgroup per tile.  MODE 1: tiles dealt by find_tile_split; a workgroup with a piece of a tile writes its
@@ -1126,6 +1141,22 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
     // rounded and staged in LDS - the tile's upper half of the rows in one stage buffer, the lower half in the other -
     // then written out as 16-byte packets along rows, rows going to their mapped position.
     const int lane = opaque(lane_id());
+    if (GLU == 0 && !GROUP_K && p.bias != nullptr) {
+        // a lane's four columns of every 16-column block, the same for all of its rows
+        const S* brow = reinterpret_cast<const S*>(p.bias) + (int64_t)expert * p.N;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int col = n_base + (j / TNH) * (BN / 2) + wn * CW + (j % TNH) * 16 + 4 * (lane / 16);
+            const u32x2_t four = *reinterpret_cast<const u32x2_t*>(brow + (col < p.N ? col : 0));  // N is a multiple of 8
+            float b[4];
+            unpack2<T>(four.x, b[0], b[1]);
+            unpack2<T>(four.y, b[2], b[3]);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[i][j][r] += b[r];
+        }
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         S* Ch = reinterpret_cast<S*>(i / TH == 0 ? lds0 : lds1);  // tile rows [0, BM / 2) are staged in lds0, the rest in lds1
@@ -1233,7 +1264,8 @@ __global__ void __launch_bounds__(256)
     s2s_plain_kernel(const typename T::storage_t* __restrict__ X, int64_t ldx, const typename T::storage_t* __restrict__ W,
                      int64_t se, int64_t sk, int64_t sn, const int64_t* __restrict__ row_idx,
                      const int64_t* __restrict__ offsets, typename T::storage_t* __restrict__ out, int64_t ldo,
-                     int64_t slots, int K, int N, int E, int fan_out, int x_grouped, int y_grouped) {
+                     int64_t slots, int K, int N, int E, int fan_out, int x_grouped, int y_grouped,
+                     const typename T::storage_t* __restrict__ bias) {
     const int n = blockIdx.x * 64 + threadIdx.x % 64;
     const int64_t slot = (int64_t)blockIdx.y * 4 + threadIdx.x / 64;
     if (slot >= slots || n >= N) return;
@@ -1250,6 +1282,7 @@ __global__ void __launch_bounds__(256)
     const typename T::storage_t* w = W + (int64_t)lo * se + (int64_t)n * sn;
     double acc = 0.0;
     for (int k = 0; k < K; ++k) acc = fma((double)T::up(x[k]), (double)T::up(w[(int64_t)k * sk]), acc);
+    if (bias != nullptr) acc += (double)T::up(bias[(int64_t)lo * N + n]);
     out[dst_row * ldo + n] = T::down((float)acc);
 }
 
@@ -1401,9 +1434,9 @@ extern "C" int ck_scatter2scatter(const void* X, int64_t x_stride, const void* W
                                   int64_t w_stride_k, int64_t w_stride_n, const int64_t* sorted_scattered_idxs,
                                   const int64_t* expert_offsets, void* out, int64_t out_stride, int64_t num_slots,
                                   int64_t K, int64_t N, int64_t E, int64_t fan_out, int x_grouped, int y_grouped,
-                                  int dtype, void* stream) {
+                                  const void* bias, int dtype, void* stream) {
     return ck_scatter2scatter_ws(X, x_stride, W, w_stride_e, w_stride_k, w_stride_n, sorted_scattered_idxs, expert_offsets,
-                                 out, out_stride, num_slots, K, N, E, fan_out, x_grouped, y_grouped, dtype, nullptr, 0,
+                                 out, out_stride, num_slots, K, N, E, fan_out, x_grouped, y_grouped, bias, dtype, nullptr, 0,
                                  stream);
 }
 
@@ -1411,7 +1444,8 @@ extern "C" int ck_scatter2scatter_ws(const void* X, int64_t x_stride, const void
                                      int64_t w_stride_k, int64_t w_stride_n, const int64_t* sorted_scattered_idxs,
                                      const int64_t* expert_offsets, void* out, int64_t out_stride, int64_t num_slots,
                                      int64_t K, int64_t N, int64_t E, int64_t fan_out, int x_grouped, int y_grouped,
-                                     int dtype, void* workspace, int64_t workspace_bytes, void* stream) {
+                                     const void* bias, int dtype, void* workspace, int64_t workspace_bytes,
+                                     void* stream) {
     if (num_slots < 0 || K < 0 || N < 0 || E <= 0 || fan_out <= 0) return CK_ERR_SHAPE;
     if (num_slots > 0x7fffffff || K > 0x7fffffff || N > 0x7fffffff || E > 0x7fffffff) return CK_ERR_SHAPE;
     if (dtype != CK_F32 && dtype != CK_F16 && dtype != CK_BF16) return CK_ERR_DTYPE;
@@ -1419,12 +1453,13 @@ extern "C" int ck_scatter2scatter_ws(const void* X, int64_t x_stride, const void
     if (!out || !expert_offsets || (K > 0 && (!X || !W))) return CK_ERR_NULL;
     if ((!x_grouped || !y_grouped) && !sorted_scattered_idxs) return CK_ERR_NULL;
     if (!ck_aligned_elem(X, dtype) || !ck_aligned_elem(W, dtype) || !ck_aligned_elem(out, dtype)) return CK_ERR_ALIGN;
+    if (bias && !ck_aligned_elem(bias, dtype)) return CK_ERR_ALIGN;
     hipStream_t s = (hipStream_t)stream;
 
     const bool b_kc = w_stride_k == 1, b_nc = w_stride_n == 1;
     const bool fast = dtype != CK_F32 && K > 0 && (b_kc || b_nc) && ck_aligned16(X) && ck_aligned16(W) && mult8(K) &&
                       mult8(x_stride) && mult8(w_stride_e) && mult8(b_kc ? w_stride_n : w_stride_k) && mult8(N) &&
-                      ck_aligned16(out) && mult8(out_stride);
+                      ck_aligned16(out) && mult8(out_stride) && (!bias || ck_aligned16(bias));
     if (fast) {
         ck::GemmParams p = {};
         p.A = X;
@@ -1443,6 +1478,7 @@ extern "C" int ck_scatter2scatter_ws(const void* X, int64_t x_stride, const void
         p.fan_out = (int)fan_out;
         p.x_grouped = x_grouped;
         p.y_grouped = y_grouped;
+        p.bias = bias;
         // the direct-to-LDS kernel addresses a tile's sources with 32-bit byte offsets from a per-tile base
         p.wide = num_slots * x_stride * 2 >= (int64_t)1 << 32 || (b_kc ? N : K) * p.ldb * 2 >= (int64_t)1 << 32;
         p.m_tiles = (int)(num_slots / kBM + E);
@@ -1476,7 +1512,8 @@ extern "C" int ck_scatter2scatter_ws(const void* X, int64_t x_stride, const void
         typedef typename T::storage_t S;
         hipLaunchKernelGGL((ck::s2s_plain_kernel<T>), grid, dim3(256), 0, s, (const S*)X, x_stride, (const S*)W,
                            w_stride_e, w_stride_k, w_stride_n, sorted_scattered_idxs, expert_offsets, (S*)out,
-                           out_stride, num_slots, (int)K, (int)N, (int)E, (int)fan_out, x_grouped, y_grouped);
+                           out_stride, num_slots, (int)K, (int)N, (int)E, (int)fan_out, x_grouped, y_grouped,
+                           (const S*)bias);
     });
     return ck_launch_status();
 }
@@ -1531,7 +1568,8 @@ extern "C" int ck_scatter2scatter_glu(const void* X, int64_t x_stride, const voi
         return ck_launch_status();
     }
     const int st = ck_scatter2scatter(X, x_stride, W, w_stride_e, w_stride_k, w_stride_n, sorted_scattered_idxs,
-                                      expert_offsets, h, h_stride, num_slots, K, N, E, fan_out, x_grouped, 1, dtype, stream);
+                                      expert_offsets, h, h_stride, num_slots, K, N, E, fan_out, x_grouped, 1, nullptr, dtype,
+                                      stream);
     if (st != CK_OK) return st;
     const dim3 grid((unsigned)ck_ceil_div(I, 256), (unsigned)(num_slots < 65535 ? num_slots : 65535));
     CK_DISPATCH_DTYPE(dtype, {
@@ -1589,7 +1627,7 @@ extern "C" int ck_scatter2scatter_glu_bwd(const void* DY, int64_t dy_stride, con
     }
     // d_act goes into the first half of every d_h row, then one pass turns the row into (d_up | d_gate) in place
     const int st = ck_scatter2scatter(DY, dy_stride, W, w_stride_e, w_stride_k, w_stride_n, nullptr, expert_offsets, d_h,
-                                      d_h_stride, num_slots, K, I, E, 1, 1, 1, dtype, stream);
+                                      d_h_stride, num_slots, K, I, E, 1, 1, 1, nullptr, dtype, stream);
     if (st != CK_OK) return st;
     const dim3 grid((unsigned)ck_ceil_div(I, 256), (unsigned)(num_slots < 65535 ? num_slots : 65535));
     CK_DISPATCH_DTYPE(dtype, {

@@ -635,12 +635,6 @@ __global__ void __launch_bounds__(256)
 
 // ---- host side ------------------------------------------------------------------------------
 constexpr int kReduceSplits = 16;  // row splits of the first dweight reduction pass
-#ifndef CK_RMSNORM_FWD_DEFAULT_ROWS
-#define CK_RMSNORM_FWD_DEFAULT_ROWS 1
-#endif
-#ifndef CK_RMSNORM_BWD_DEFAULT_VARIANT
-#define CK_RMSNORM_BWD_DEFAULT_VARIANT 2
-#endif
 
 static int cu_count() {
     static int cached[64] = {0};
@@ -695,7 +689,12 @@ static int bwd_teams(int64_t B, int tpr, int per_cu = 1) {
 // program): forward 1, 2, 4 = rows a wave requests at once and then ends (rmsnorm_fwd_rows_kernel), 8 or more = waves
 // that walk rows with the next one in flight (rmsnorm_fwd_kernel); backward 1 = two workgroups per compute unit
 // without a row in flight, 2 or more = one with.  0 = the default.  Rows wider than a wave's registers have one variant.
-constexpr int kFwdDefaultRows = CK_RMSNORM_FWD_DEFAULT_ROWS, kBwdDefaultVariant = CK_RMSNORM_BWD_DEFAULT_VARIANT;
+// The defaults follow what the tuner measured on MI355X at 16384 rows, all three dtypes: rows of up to 2 KB are
+// fastest walked (10.9 against 18.4 us at 1024 bf16 elements), longer ones with one wave per row (43.1 against 45.7 us
+// at 4096); the backward runs two workgroups per compute unit up to 4 KB a row (22.5 against 27.7 us at 1024, 32.1
+// against 33.2 at 2048) and one with a row in flight beyond (66.1 against 71.4 us at 4096).
+static int fwd_default_rows(int64_t H, int dtype) { return H * (dtype == CK_F32 ? 4 : 2) <= 2048 ? 8 : 1; }
+static int bwd_default_variant(int64_t H, int dtype) { return H * (dtype == CK_F32 ? 4 : 2) <= 4096 ? 1 : 2; }
 
 // packets per lane when a row is exactly that many packets per lane of a TPR-lane team (2, 4 or 8), else 0
 static int exact_packs(int64_t H, int dtype, int tpr) {
@@ -753,7 +752,7 @@ static void launch_fwd_walk(hipStream_t s, const FwdArgs& a, int np) {
 template <typename T, bool RES>
 static void launch_fwd_fast(hipStream_t s, const FwdArgs& a, int tpr, int dtype, int block_size_b) {
     const int np = exact_packs(a.H, dtype, tpr);
-    const int rows = block_size_b == 0 ? kFwdDefaultRows : block_size_b;
+    const int rows = block_size_b == 0 ? fwd_default_rows(a.H, dtype) : block_size_b;
     if (tpr == 64 && rows == 1) launch_fwd_rows<T, 1, RES>(s, a, np);
     else if (tpr == 64 && rows < 8) launch_fwd_rows<T, 2, RES>(s, a, np);
     else if (tpr == 64) launch_fwd_walk<T, 64, RES>(s, a, np);
@@ -895,7 +894,7 @@ extern "C" int ck_rmsnorm_backward(const void* x, const void* weight, const void
     CK_DISPATCH_DTYPE(dtype, {
         typedef typename T::storage_t S;
         if (tpr != 0) {
-            const bool two = tpr == 64 && (block_size_b == 0 ? kBwdDefaultVariant : block_size_b) == 1;
+            const bool two = tpr == 64 && (block_size_b == 0 ? bwd_default_variant(H, dtype) : block_size_b) == 1;
             const int teams = bwd_teams(B, tpr, two ? 2 : 1);
             const int block = tpr > 256 ? tpr : 256;
             const unsigned grid = (unsigned)(teams / (block / tpr));

@@ -55,12 +55,12 @@ _SIGNATURES = {
     "ck_moe_sort_noalloc": (_i32, [_p, _i32, _p, _p, _p, _i64, _i64, _p]),
     "ck_scatter2scatter": (
         _i32,
-        [_p, _i64, _p, _i64, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _p],
+        [_p, _i64, _p, _i64, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _p, _i32, _p],
     ),
     "ck_scatter2scatter_ws": (
         _i32,
-        [_p, _i64, _p, _i64, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _p, _i64,
-         _p],
+        [_p, _i64, _p, _i64, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _p, _i32, _p,
+         _i64, _p],
     ),
     "ck_scatter2scatter_workspace_size": (_i64, [_i64, _i64, _i64, _i64, _i32]),
     "ck_scatter2scatter_glu": (
@@ -460,13 +460,16 @@ def scatter2scatter_workspace_size(num_slots: int, K: int, N: int, E: int, dtype
 
 
 def scatter2scatter(X, W, sorted_scattered_idxs, expert_offsets, out, fan_out: int, x_grouped: bool,
-                    y_grouped: bool, workspace=None) -> None:
+                    y_grouped: bool, workspace=None, bias=None) -> None:
     """X [*, K] (unit column stride), W strided view [E, K, N], out [slots, N] (unit column stride); ``workspace``:
-    uint8 tensor of ``scatter2scatter_workspace_size`` bytes or None."""
+    uint8 tensor of ``scatter2scatter_workspace_size`` bytes or None; ``bias``: [E, N] contiguous or None, added to
+    every row of its expert before the row is rounded."""
     lib = load_library()
     if X.stride(1) != 1 or out.stride(1) != 1:
         raise ValueError("scatter2scatter needs unit column stride for X and out")
-    _same_dtype(X, "scatter2scatter", W=W, out=out)
+    _same_dtype(X, "scatter2scatter", W=W, out=out, bias=bias)
+    if bias is not None and (tuple(bias.shape) != (W.size(0), out.size(1)) or not bias.is_contiguous()):
+        raise ValueError("scatter2scatter: bias must be a contiguous [E, N] tensor")
     if sorted_scattered_idxs is not None:
         sorted_scattered_idxs = _index_i64(sorted_scattered_idxs, "sorted_scattered_idxs")
     expert_offsets = _index_i64(expert_offsets, "expert_offsets")
@@ -474,12 +477,13 @@ def scatter2scatter(X, W, sorted_scattered_idxs, expert_offsets, out, fan_out: i
         raise ValueError("scatter2scatter: one expert offset per expert of W")
     flop = 2.0 * out.size(0) * X.size(1) * out.size(1)
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
-    with _Launch(X, W, sorted_scattered_idxs, expert_offsets, out, workspace) as L, _Timed("scatter2scatter", flop):
+    with _Launch(X, W, sorted_scattered_idxs, expert_offsets, out, workspace, bias) as L, _Timed("scatter2scatter", flop):
         _check(
             lib.ck_scatter2scatter_ws(_ptr(X), X.stride(0), _ptr(W), W.stride(0), W.stride(1), W.stride(2),
                                       _ptr(sorted_scattered_idxs), _ptr(expert_offsets), _ptr(out), out.stride(0),
                                       out.size(0), X.size(1), out.size(1), W.size(0), fan_out, int(x_grouped),
-                                      int(y_grouped), dtype_code(X.dtype), _ptr(workspace), ws_bytes, L.stream),
+                                      int(y_grouped), _ptr(bias), dtype_code(X.dtype), _ptr(workspace), ws_bytes,
+                                      L.stream),
             "ck_scatter2scatter_ws",
         )
 

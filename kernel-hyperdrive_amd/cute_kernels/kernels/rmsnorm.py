@@ -76,7 +76,7 @@ def _check_row_length(hidden_size: int) -> None:
 # (forward.py:10-46 around kernels_forward.py:63-107).  Same here, so a caller may fix either without the other.
 @cutotune(
     configs=get_cartesian_product_cutotune_configs(BLOCK_SIZE_B=FORWARD_ROWS),
-    default_config=CutoTuneConfig({"BLOCK_SIZE_B": 1}),
+    default_config=CutoTuneConfig({"BLOCK_SIZE_B": 0}),  # 0: the library's own choice by row size
     triggers=_TRIGGERS,
     functional_triggers=_FUNCTIONAL_TRIGGERS,
 )
@@ -94,7 +94,7 @@ def rmsnorm_forward_launch(
 
 @cutotune(
     configs=get_cartesian_product_cutotune_configs(BLOCK_SIZE_B=BACKWARD_VARIANTS),
-    default_config=CutoTuneConfig({"BLOCK_SIZE_B": 2}),
+    default_config=CutoTuneConfig({"BLOCK_SIZE_B": 0}),
     triggers=_TRIGGERS,
     functional_triggers=_FUNCTIONAL_TRIGGERS,
 )

@@ -48,6 +48,7 @@ def scatter2scatter(
     x_grouped: bool = False,
     y_grouped: bool = False,
     expert_offsets: torch.Tensor | None = None,
+    bias: torch.Tensor | None = None,
 ) -> None:
     assert sorted_scattered_idxs.size(0) == sorted_expert_idxs.size(0)
     assert sorted_scattered_idxs.size(0) == X.size(0) * FAN_OUT
@@ -67,7 +68,8 @@ def scatter2scatter(
         nbytes = _C.scatter2scatter_workspace_size(out.size(0), X.size(1), out.size(1), W.size(0), X.dtype)
         if nbytes > 0:
             workspace = torch.empty(nbytes, dtype=torch.uint8, device=X.device)
-    _C.scatter2scatter(X, W, sorted_scattered_idxs, expert_offsets, out, FAN_OUT, x_grouped, y_grouped, workspace)
+    _C.scatter2scatter(X, W, sorted_scattered_idxs, expert_offsets, out, FAN_OUT, x_grouped, y_grouped, workspace,
+                       bias)
 
 
 @cute_op(f"{LIBRARY_NAME}::scatter2scatter_glu", mutates_args={"h", "act"})
@@ -200,15 +202,9 @@ class _ScatteredExperts(torch.autograd.Function):
             x_grouped=grouped_in,
             y_grouped=grouped_out,
             expert_offsets=expert_offsets,
+            # added to the fp32 sums, before the routing weights mix the k outputs: F.linear(rows, W[e], bias[e])
+            bias=expert_biases,
         )
-        if expert_biases is not None:
-            # before the routing weights mix the k outputs, as F.linear(rows, W[e], bias[e]) has it
-            expert_bias_forward(
-                y=output,
-                bias=expert_biases,
-                expert_offsets=expert_offsets,
-                row_index=None if grouped_out else sorted_scattered_idxs,
-            )
 
         if gates is None:
             output_expanded = None

@@ -222,8 +222,9 @@ def _expert_of_slot(expert_offsets: torch.Tensor, num_slots: int) -> np.ndarray:
 
 
 def scatter2scatter(X, W, sorted_scattered_idxs, expert_offsets, fan_out, x_grouped, y_grouped,
-                    compute_dtype=torch.float32):
-    """out[out_row(i)] = X[in_row(i)] @ W[e(i)];  W is [E, K, N]  (kernels.py:66-102)."""
+                    compute_dtype=torch.float32, bias=None):
+    """out[out_row(i)] = X[in_row(i)] @ W[e(i)];  W is [E, K, N]  (kernels.py:66-102).  ``bias`` [E, N]: the term
+    F.linear(rows, W[e], bias[e]) adds per expert (torch_implementation.py:35-43), before the one rounding."""
     num_slots = sorted_scattered_idxs.numel()
     expert = _expert_of_slot(expert_offsets, num_slots)
     idx = sorted_scattered_idxs.cpu().numpy()
@@ -233,6 +234,8 @@ def scatter2scatter(X, W, sorted_scattered_idxs, expert_offsets, fan_out, x_grou
         src = i if x_grouped else idx[i] // fan_out
         dst = i if y_grouped else idx[i]
         out[dst] = Xc[src] @ Wc[expert[i]]
+        if bias is not None:
+            out[dst] += bias[expert[i]].to(compute_dtype)
     return out.to(X.dtype)
 
 

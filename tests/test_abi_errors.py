@@ -106,24 +106,25 @@ def test_routing_argument_checks(lib):
 
 def test_grouped_gemm_argument_checks(lib):
     s2s = lib.ck_scatter2scatter
-    #        X  ldx W  se    sk sn idx off out ldo slots K  N  E  fan xg yg dtype stream
-    assert s2s(P, 64, P, 4096, 1, 64, P, P, P, 64, 16, 64, 64, 0, 1, 0, 1, BF16, None) == SHAPE  # E = 0
-    assert s2s(P, 64, P, 4096, 1, 64, P, P, P, 64, 16, 64, 64, 2, 0, 0, 1, BF16, None) == SHAPE  # fan_out = 0
-    assert s2s(P, 64, P, 4096, 1, 64, P, P, P, 64, 16, 64, 64, 2, 1, 0, 1, 3, None) == DTYPE
-    assert s2s(P, 64, P, 4096, 1, 64, P, None, P, 64, 16, 64, 64, 2, 1, 0, 1, BF16, None) == NULL  # no offsets
-    assert s2s(P, 64, P, 4096, 1, 64, None, P, P, 64, 16, 64, 64, 2, 1, 0, 1, BF16, None) == NULL  # gather without index
-    assert s2s(P + 1, 64, P, 4096, 1, 64, P, P, P, 64, 16, 64, 64, 2, 1, 0, 1, BF16, None) == ALIGN
-    assert s2s(P, 64, P, 4096, 1, 64, P, P, P, 64, 0, 64, 64, 2, 1, 0, 1, BF16, None) == OK  # no rows
+    #        X  ldx W  se    sk sn idx off out ldo slots K  N  E  fan xg yg bias dtype stream
+    assert s2s(P, 64, P, 4096, 1, 64, P, P, P, 64, 16, 64, 64, 0, 1, 0, 1, None, BF16, None) == SHAPE  # E = 0
+    assert s2s(P, 64, P, 4096, 1, 64, P, P, P, 64, 16, 64, 64, 2, 0, 0, 1, None, BF16, None) == SHAPE  # fan_out = 0
+    assert s2s(P, 64, P, 4096, 1, 64, P, P, P, 64, 16, 64, 64, 2, 1, 0, 1, None, 3, None) == DTYPE
+    assert s2s(P, 64, P, 4096, 1, 64, P, None, P, 64, 16, 64, 64, 2, 1, 0, 1, None, BF16, None) == NULL  # no offsets
+    assert s2s(P, 64, P, 4096, 1, 64, None, P, P, 64, 16, 64, 64, 2, 1, 0, 1, None, BF16, None) == NULL  # gather without index
+    assert s2s(P + 1, 64, P, 4096, 1, 64, P, P, P, 64, 16, 64, 64, 2, 1, 0, 1, None, BF16, None) == ALIGN
+    assert s2s(P, 64, P, 4096, 1, 64, P, P, P, 64, 0, 64, 64, 2, 1, 0, 1, None, BF16, None) == OK  # no rows
+    assert s2s(P, 64, P, 4096, 1, 64, P, P, P, 64, 16, 64, 64, 2, 1, 0, 1, P + 1, BF16, None) == ALIGN  # bias
     ws = lib.ck_scatter2scatter_ws
     need = lib.ck_scatter2scatter_workspace_size(1024, 8192, 256, 4, BF16)
     assert need > 0
     assert lib.ck_scatter2scatter_workspace_size(1024, 1024, 256, 4, BF16) == 0  # contraction too short to cut
     assert lib.ck_scatter2scatter_workspace_size(1024, 8192, 256, 4, F32) == 0
-    #       X  ldx   W  se          sk sn    idx off out ldo slots K     N    E  fan xg yg dtype ws  bytes stream
-    assert ws(P, 8192, P, 8192 * 256, 1, 8192, P, P, P, 256, 1024, 8192, 256, 4, 1, 0, 1, BF16, P, need - 1, None) == WORKSPACE
-    assert ws(P, 8192, P, 8192 * 256, 1, 8192, P, P, P, 256, 1024, 8192, 256, 4, 1, 0, 1, BF16, P + 4, need, None) == WORKSPACE
-    assert ws(P, 8192, P, 8192 * 256, 1, 8192, P, None, P, 256, 1024, 8192, 256, 4, 1, 0, 1, BF16, P, need, None) == NULL
-    assert ws(P, 8192, P, 8192 * 256, 1, 8192, P, P, P, 256, 0, 8192, 256, 4, 1, 0, 1, BF16, P, need, None) == OK  # no rows
+    #       X  ldx   W  se          sk sn    idx off out ldo slots K     N    E  fan xg yg bias dtype ws  bytes stream
+    assert ws(P, 8192, P, 8192 * 256, 1, 8192, P, P, P, 256, 1024, 8192, 256, 4, 1, 0, 1, None, BF16, P, need - 1, None) == WORKSPACE
+    assert ws(P, 8192, P, 8192 * 256, 1, 8192, P, P, P, 256, 1024, 8192, 256, 4, 1, 0, 1, None, BF16, P + 4, need, None) == WORKSPACE
+    assert ws(P, 8192, P, 8192 * 256, 1, 8192, P, None, P, 256, 1024, 8192, 256, 4, 1, 0, 1, None, BF16, P, need, None) == NULL
+    assert ws(P, 8192, P, 8192 * 256, 1, 8192, P, P, P, 256, 0, 8192, 256, 4, 1, 0, 1, None, BF16, P, need, None) == OK  # no rows
     glu = lib.ck_scatter2scatter_glu
     #        X  ldx W  se    sk sn idx off h  ldh  act lda slots K  I  E  fan xg dtype stream
     assert glu(P, 64, P, 8192, 1, 64, P, P, P, 128, P, 64, 16, 64, 64, 0, 1, 0, BF16, None) == SHAPE  # E = 0

@@ -223,6 +223,12 @@ def test_scatter2scatter_against_dense_per_expert(x_grouped, y_grouped):
     dense = torch.cat([grouped[s_e == e] @ W[e] for e in range(E)])
     expected = dense if y_grouped else torch.zeros_like(dense).index_copy(0, s_idx, dense)
     assert torch.allclose(out, expected, rtol=1e-13, atol=1e-13)
+    # with a bias: torch's own F.linear on each expert's block (torch_implementation.py:35-43)
+    bias = torch.randn(E, N, dtype=F64)
+    out = O.scatter2scatter(X, W, s_idx, off, fan_out, x_grouped, y_grouped, F64, bias=bias)
+    dense = torch.cat([torch.nn.functional.linear(grouped[s_e == e], W[e].T, bias[e]) for e in range(E)])
+    expected = dense if y_grouped else torch.zeros_like(dense).index_copy(0, s_idx, dense)
+    assert torch.allclose(out, expected, rtol=1e-13, atol=1e-13)
 
 
 def test_group_bwd_w_and_group():
