@@ -58,6 +58,8 @@ def parse_args():
     p.add_argument("--no-extras", action="store_true", help="skip the SwiGLU / RMSNorm / embedding bandwidth figures")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     p.add_argument("--only-extras", action="store_true", help="only the HBM-bound ops (for profiling them)")
+    p.add_argument("--embedding-ids", choices=["both", "uniform", "zipf"], default="both",
+                   help="with --only-extras: one id distribution only (counter profiles sum over a kernel's dispatches)")
     p.add_argument("--tokens", type=int, default=8192, help="T of the MoE workload (default: the BASELINE shape)")
     p.add_argument("--copy-calibration", action="store_true",
                    help="also run three 1 GiB device copies before the steps (a kernel of known HBM traffic, to scale "
@@ -221,7 +223,7 @@ def bench_moe_skewed(device, steps=10, warmup=3):
             "empty_experts": int((counts == 0).sum().item()), "largest_expert_share": round(counts.max().item() / counts.sum().item(), 3)}
 
 
-def bench_extras(device):
+def bench_extras(device, embedding_ids="both"):
     from cute_kernels import KernelBackend
     from cute_kernels.cutotune import CutoTuneParameter
     from cute_kernels.kernels import embedding as EM
@@ -280,6 +282,8 @@ def bench_extras(device):
     dys = [torch.randn(8, 4096, H, device=device, dtype=dtype) for _ in range(2)]
     for label, ids in (("uniform", torch.randint(0, V, (8, 4096), generator=torch.Generator().manual_seed(0))),
                        ("zipf", zipf_ids((8, 4096), V, 1.1, seed=0))):
+        if embedding_ids not in ("both", label):
+            continue
         # distinct table rows: a row that several ids select is read from HBM once and from the caches after that
         distinct = int(torch.unique(ids).numel())
         ids = ids.to(device)
@@ -291,8 +295,9 @@ def bench_extras(device):
         out[f"embedding_bwd_{label}"] = gbs(n * H * 2 + V * H * 2 + 8 * n, ms)
     del table, dys
     torch.cuda.empty_cache()
-    out["moe_fine_grained_skewed"] = bench_moe_skewed(device)
-    torch.cuda.empty_cache()
+    if embedding_ids == "both":
+        out["moe_fine_grained_skewed"] = bench_moe_skewed(device)
+        torch.cuda.empty_cache()
     return out
 
 
@@ -363,11 +368,11 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     device = torch.device("cuda", 0)
-    if args.only_extras:
-        print(json.dumps({"extras": bench_extras(device)}))
-        return
     if args.copy_calibration:
         copy_calibration(device)
+    if args.only_extras:
+        print(json.dumps({"extras": bench_extras(device, args.embedding_ids)}))
+        return
     result, roofline, config = bench_moe(device, args)
     line = {
         "metric": "scattermoe_fwd_bwd_tflops",

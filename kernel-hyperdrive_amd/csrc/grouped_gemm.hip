@@ -625,7 +625,11 @@ __global__ void __launch_bounds__(TL::THREADS) grouped_gemm_kernel(GemmParams p)
 // avoided by an XOR swizzle applied on the global side (which 16-byte chunk a lane fetches) and undone
 // when fragments are read:
 //   k-contiguous operand, row = 128 B = 8 slots:   slot = chunk ^ ((row >> 1) & 7)
-//   other layout, contraction row = ROWS * 2 B:    slot = chunk ^ ((k & 3) << 2)
+//   other layout, contraction row = ROWS * 2 B:    slot = chunk ^ (((k & 3) << 2) | (((k >> 3) & 1) << 1))
+// (a transposing read takes contraction rows 8 g + r, g = lane / 16, r = 0 .. 3, 32 bytes of each per 16 lanes, and
+// the LDS serves 32 lanes at a time: the first term spreads the four r over the 256 bytes of the banks in steps of
+// 64, the second puts the odd g into the 32-byte gaps between them.  Without it the two g of a half-wave met in
+// the same banks: half of the LDS cycles of the weight-gradient product were conflict cycles.)
 // LDS positions whose contraction index lies beyond the end of the contraction range are cleared with a
 // plain store in the (single) partial step; positions of rows / columns outside the problem keep whatever
 // they held, which only reaches outputs that are never stored.
@@ -642,7 +646,7 @@ struct DtlOperand {
     static __device__ __forceinline__ void slot_source(int p, int& line, int& chunk) {
         line = p / SLOTS_PER_LINE;
         const int slot = p % SLOTS_PER_LINE;
-        chunk = KC ? (slot ^ ((line >> 1) & 7)) : (slot ^ ((line & 3) << 2));
+        chunk = KC ? (slot ^ ((line >> 1) & 7)) : (slot ^ (((line & 3) << 2) | (((line >> 3) & 1) << 1)));
     }
 };
 
@@ -877,6 +881,9 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
     // ---- fragment addresses (bytes inside a stage) -----------------------------------------------------
     int frag_row, frag_swz;
     int a_off[TM], b_off[TN];
+    // transposed layouts: the odd 16-row block of a pair lies 32 bytes after the even one, before the swizzle; the
+    // swizzle flips that bit for odd lane / 16, so there it lies 32 bytes before
+    const int odd_step = (lane_id() / 16) & 1 ? -32 : 32;
     {
         const int lane = lane_id();
         frag_row = (lane % 16) * 128;
@@ -889,7 +896,7 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
                 a_off[i] = (i / TH) * A_HALF + l0 * 128;
             } else {
                 const int col = l0 + (q % 4) * 4;
-                a_off[i] = (i / TH) * A_HALF + (g * 8 + q / 4) * BM + ((((col / 8) ^ ((q / 4) << 2))) << 4) + (col % 8) * 2;
+                a_off[i] = (i / TH) * A_HALF + (g * 8 + q / 4) * BM + (((col / 8) ^ ((q / 4) << 2) ^ ((g & 1) << 1)) << 4) + (col % 8) * 2;
             }
         }
 #pragma unroll
@@ -899,7 +906,7 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
                 b_off[j] = B_AT + (j / TNH) * B_HALF + l0 * 128;
             } else {
                 const int col = l0 + (q % 4) * 4;
-                b_off[j] = B_AT + (j / TNH) * B_HALF + (g * 8 + q / 4) * BN + ((((col / 8) ^ ((q / 4) << 2))) << 4) + (col % 8) * 2;
+                b_off[j] = B_AT + (j / TNH) * B_HALF + (g * 8 + q / 4) * BN + (((col / 8) ^ ((q / 4) << 2) ^ ((g & 1) << 1)) << 4) + (col % 8) * 2;
             }
         }
     }
@@ -916,7 +923,7 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
                     af[kki][i] = *reinterpret_cast<const frag_t*>(st + kc + a_off[ii]);
                 } else {
                     // a contraction row of a half operand is BM / 2 elements = BM bytes
-                    const char* q = st + a_off[ii & ~1] + (ii & 1) * 32 + kk * BM;
+                    const char* q = st + a_off[ii & ~1] + (ii & 1) * odd_step + kk * BM;
                     union {
                         v4i16_t h2[2];
                         frag_t f;
@@ -939,7 +946,7 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
                 if (B_KCC) {
                     bf[kki][j] = *reinterpret_cast<const frag_t*>(st + kc + b_off[jj]);
                 } else {
-                    const char* q = st + b_off[jj & ~1] + (jj & 1) * 32 + kk * BN;
+                    const char* q = st + b_off[jj & ~1] + (jj & 1) * odd_step + kk * BN;
                     union {
                         v4i16_t h2[2];
                         frag_t f;
@@ -959,6 +966,25 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
         for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
+    // The per-expert bias is what the sums start from (not in a piece of a split tile: there the launch that adds
+    // the pieces up starts from it): it joins the fp32 sums at no cost and is rounded with them, once.
+    if (GLU == 0 && !GROUP_K && p.bias != nullptr && !(MODE == 1 && part_slot >= 0)) {
+        // a lane's four columns of every 16-column block, the same for all of its rows (see the epilogue)
+        const S* brow = reinterpret_cast<const S*>(p.bias) + (int64_t)expert * p.N;
+        const int lane = lane_id();
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int col = n_base + (j / TNH) * (BN / 2) + wn * CW + (j % TNH) * 16 + 4 * (lane / 16);
+            const u32x2_t four = *reinterpret_cast<const u32x2_t*>(brow + (col < p.N ? col : 0));  // N is a multiple of 8
+            float b[4];
+            unpack2<T>(four.x, b[0], b[1]);
+            unpack2<T>(four.y, b[2], b[3]);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[i][j][r] = b[r];
+        }
+    }
 
     // one quarter of the wave's block: rows of half ha times columns of half hb, over the whole tile depth.  The
     // MFMA gets the column fragment as its first operand, i.e. it computes the 16 x 16 block transposed: a lane
@@ -1141,22 +1167,6 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
     // rounded and staged in LDS - the tile's upper half of the rows in one stage buffer, the lower half in the other -
     // then written out as 16-byte packets along rows, rows going to their mapped position.
     const int lane = opaque(lane_id());
-    if (GLU == 0 && !GROUP_K && p.bias != nullptr) {
-        // a lane's four columns of every 16-column block, the same for all of its rows
-        const S* brow = reinterpret_cast<const S*>(p.bias) + (int64_t)expert * p.N;
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const int col = n_base + (j / TNH) * (BN / 2) + wn * CW + (j % TNH) * 16 + 4 * (lane / 16);
-            const u32x2_t four = *reinterpret_cast<const u32x2_t*>(brow + (col < p.N ? col : 0));  // N is a multiple of 8
-            float b[4];
-            unpack2<T>(four.x, b[0], b[1]);
-            unpack2<T>(four.y, b[2], b[3]);
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) acc[i][j][r] += b[r];
-        }
-    }
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         S* Ch = reinterpret_cast<S*>(i / TH == 0 ? lds0 : lds1);  // tile rows [0, BM / 2) are staged in lds0, the rest in lds1

@@ -74,5 +74,31 @@ def build(verbose: bool = False, jobs: int | None = None) -> str:
     return LIB_PATH
 
 
+def kernel_resources(source: str) -> dict[str, dict[str, int]]:
+    """Registers and scratch of every kernel of one source, as the compiler reports them
+    (``-Rpass-analysis=kernel-resource-usage``): {mangled name: {"vgprs": n, "scratch": bytes per lane}}.  Scratch
+    above zero means the kernel spills registers to memory."""
+    import re
+    import tempfile
+
+    with tempfile.TemporaryDirectory() as tmp:
+        cmd = [find_hipcc(), *HIPCC_FLAGS, "-Rpass-analysis=kernel-resource-usage", "-c",
+               os.path.join(CSRC_DIR, source), "-o", os.path.join(tmp, "out.o")]
+        result = subprocess.run(cmd, capture_output=True, text=True)
+    if result.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {source}:\n{result.stderr}")
+    found: dict[str, dict[str, int]] = {}
+    name = None
+    for line in result.stderr.splitlines():
+        if match := re.search(r"Function Name: (\S+)", line):
+            name = match.group(1)
+            found[name] = {}
+        elif name and (match := re.search(r"remark:\s+VGPRs: (\d+)", line)):
+            found[name]["vgprs"] = int(match.group(1))
+        elif name and (match := re.search(r"ScratchSize \[bytes/lane\]: (\d+)", line)):
+            found[name]["scratch"] = int(match.group(1))
+    return found
+
+
 if __name__ == "__main__":
     print(build(verbose=True))

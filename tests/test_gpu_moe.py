@@ -658,12 +658,13 @@ def test_moe_layer_with_expert_biases(gpu, dtype, case):
             continue
         # Gradients.  The bias is added to the fp32 sums of the product before they are rounded, as the CPU's F.linear
         # does, so h and everything that reads it round where the oracle rounds: element-wise, as without biases.
-        # The bias gradients are unscaled sums of up to a thousand O(1) rows: fp32 norm-wise, 16 bits as long sums.
-        if key in ("db_fc", "db_proj"):
-            if dtype == torch.float32:
-                assert_norm_close(a, e, 1e-5, f"{name}/{key}")
-            else:
-                assert_close_long_sums(a, e, dtype, f"{name}/{key}")
+        # The bias gradients are unscaled sums of up to a thousand O(1) rows: fp32 norm-wise, 16 bits as long sums -
+        # as are the weight gradients of the experts that the skewed router gives most of the rows (measured: one
+        # element of dw_proj in a million at 1.7 times the tolerance).
+        if key in ("db_fc", "db_proj") and dtype == torch.float32:
+            assert_norm_close(a, e, 1e-5, f"{name}/{key}")
+        elif key in ("db_fc", "db_proj", "dw_fc", "dw_proj") and dtype != torch.float32:
+            assert_close_long_sums(a, e, dtype, f"{name}/{key}")
         else:
             assert_close(a, e, dtype, f"{name}/{key}")
     # and the plain-torch layer on the GPU, the reference's own way of testing (tests/kernels/scattermoe_test.py)

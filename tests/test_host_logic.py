@@ -342,3 +342,15 @@ def test_shipped_tuning_cache_loads_and_covers_the_tuned_launchers():
             assert config.get_key_values()["kernel_backend"].value == "hip"
     sw = cache.full_cache["kernels/swiglu.py->_forward"]
     assert all(len(entries) >= 2 for entries in sw.values()), "every candidate's timing is kept"
+
+
+def test_matrix_core_kernels_do_not_spill():
+    """The grouped GEMM's main kernel runs two waves per SIMD at up to 256 registers each; a change that pushes an
+    instantiation past that makes the compiler spill to scratch memory, which costs far more than the change is
+    likely to gain and shows nowhere but in the timing.  The compiler's own report is checked instead."""
+    from cute_kernels._build import kernel_resources
+
+    kernels = {n: r for n, r in kernel_resources("grouped_gemm.hip").items() if "grouped_gemm_m16_kernel" in n}
+    assert len(kernels) >= 18, sorted(kernels)  # bf16 and fp16: 3 modes x 2 layouts, 2 fused, dW
+    for name, res in kernels.items():
+        assert res["vgprs"] <= 256 and res["scratch"] == 0, (name, res)
