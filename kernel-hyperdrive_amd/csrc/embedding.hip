@@ -10,10 +10,11 @@
 //                  and records, for every sorted slot, the first slot of its run of equal ids.
 //               2. rows kernel, one launch for two jobs: rows no id selects are written as zeros (the
 //                  bulk of the traffic; a part of them rides, as extra workgroups, on the small launches
-//                  of step 1 that come after the rows are marked); a run of equal ids is cut into chunks of kChunk slots and one
-//                  wave sums the dy rows of a chunk in fp32 registers, in ascending token position.  A
-//                  run that fits one chunk is rounded and stored straight into dW; longer runs leave
-//                  one fp32 partial row per chunk in the workspace.
+//                  of step 1 that come after the rows are marked); a run of equal ids is cut into chunks of
+//                  kChunk slots.  A chunk of one row is copied by one wave; the others are summed by the four
+//                  waves of a workgroup, a quarter of the columns each, in fp32 registers and in ascending
+//                  token position.  A run that fits one chunk is rounded and stored straight into dW; longer
+//                  runs leave one fp32 partial row per chunk in the workspace.
 //               3. combine kernel: sums the partial rows of each long run and stores the dW row.
 //             No floating-point atomics, no zero-fill of rows that are written anyway, deterministic.
 #include "ck_block_sort.h"
@@ -21,7 +22,9 @@
 
 namespace ck {
 
-constexpr int kChunk = 32;      // slots of one run summed by one wave
+// slots of one run summed in one go (measured at 32768 Zipf(1.1) ids, table [128256, 4096]: 16 / 32 / 64 slots 353 /
+// 362 / 325 us - fewer partial rows to write and to add up again; ids spread evenly do not care)
+constexpr int kChunk = 64;
 constexpr int kRowPacks = 8;    // packets per lane per column tile (tile = 64 lanes * 8 packets)
 
 // accumulator of the backward sums
@@ -219,9 +222,10 @@ __global__ void __launch_bounds__(256)
     grid_sort_scatter(sh, n, shift, bits, offsets, num_waves, load, store);
 }
 
-// Runs of equal ids in the sorted order: records, for every sorted slot, the first slot of its run.  Every wave owns kRunsWaveSlots consecutive slots: it first looks
-// backwards from its first slot, 64 slots at a time, for the head of the run it starts in, then walks its
-// slots 64 at a time carrying the latest head forward with a wave max-scan.
+// Runs of equal ids in the sorted order: records, for every sorted slot, the first slot of its run.  Every wave owns
+// kRunsWaveSlots consecutive slots: it first finds the head of the run it starts in (among the 64 slots before its
+// first one, else by a 64-way search), then walks its slots 64 at a time carrying the latest head forward with a wave
+// max-scan.
 constexpr int kRunsWaveSlots = 4 * CK_WAVE;
 __global__ void __launch_bounds__(256)
     embedding_runs_kernel(const uint32_t* __restrict__ skeys, uint32_t* __restrict__ run_head, int n, FillJob fill) {
@@ -234,11 +238,30 @@ __global__ void __launch_bounds__(256)
     // head of the run that contains slot `begin`: the last slot j <= begin with skeys[j - 1] != skeys[j]
     int carry = -1;
     const uint32_t first_key = skeys[begin];
-    for (int hi = begin; carry < 0; hi -= CK_WAVE) {
-        const int j = hi - lane;  // lane 0 looks at hi, lane 63 at hi - 63
+    {
+        const int j = begin - lane;  // lane 0 looks at begin, lane 63 at begin - 63
         const bool is_head = j >= 0 && (j == 0 || skeys[j - 1] != first_key);
         const uint64_t found = __ballot(is_head);
-        if (found != 0) carry = hi - (__ffsll((unsigned long long)found) - 1);
+        if (found != 0) carry = begin - (__ffsll((unsigned long long)found) - 1);
+    }
+    if (carry < 0) {
+        // A run longer than that (a popular id): the keys are sorted, so its head is the first slot that holds the
+        // key.  The wave probes 64 evenly spaced slots of the range still in question per round trip, which narrows
+        // the range 64 times - three rounds for any number of ids, where a walk back costs one per 64 slots of the run.
+        int lo = 0, hi = begin - CK_WAVE;  // the head is in [lo, hi]: slots hi + 1 .. begin were just seen to hold the key
+        while (lo < hi) {
+            const int step = (hi - lo + CK_WAVE - 1) / CK_WAVE;
+            const int pos = min(lo + lane * step, hi);
+            const uint64_t eq = __ballot(skeys[pos] == first_key);  // false ... false true ... true along the lanes
+            if (eq == 0) {
+                lo = min(lo + (CK_WAVE - 1) * step, hi) + 1;
+            } else {
+                const int f = __ffsll((unsigned long long)eq) - 1;
+                hi = min(lo + f * step, hi);
+                if (f > 0) lo = min(lo + (f - 1) * step, hi) + 1;
+            }
+        }
+        carry = lo;
     }
     for (int i0 = begin; i0 < end; i0 += CK_WAVE) {
         const int i = i0 + lane;
@@ -257,8 +280,8 @@ __global__ void __launch_bounds__(256)
 // Workgroups [0, chunk_groups) sum chunks of runs (two dependent memory round trips per wave: latency-bound);
 // the remaining workgroups write zeros into the rows nobody selects (pure streaming writes, the bulk of the
 // bytes).  Running both in one grid lets the streaming part hide the latency of the other.
-//   chunk job: a run of equal ids is cut into chunks of kChunk slots; one wave sums the dy rows of a chunk in
-//   fp32 (fp64 for fp32 tables) in ascending token position.  A run that fits one chunk is rounded and stored
+//   chunk job: a run of equal ids is cut into chunks of kChunk slots; the dy rows of a chunk are summed in fp32
+//   (fp64 for fp32 tables) in ascending token position.  A run that fits one chunk is rounded and stored
 //   straight into dW; longer runs leave one fp32 partial row per chunk in the workspace.
 template <typename T, int VEC>
 __global__ void __launch_bounds__(256)
@@ -285,101 +308,144 @@ __global__ void __launch_bounds__(256)
     }
 
     // ---- chunk sums ----
-    const int i = blockIdx.x * 4 + threadIdx.x / CK_WAVE;
-    if (i >= n) return;
-    // every index load is issued before any of them is used: one round trip
-    const uint32_t id = skeys[i];
-    const int head = (int)run_head[i];
-    const bool in_range = lane <= kChunk && i + lane < n;
-    const uint32_t key_l = in_range ? skeys[i + lane] : 0xffffffffu;
-    const uint32_t pos_l = (in_range && lane < kChunk) ? spos[i + lane] : 0u;
-    if ((int64_t)id >= V) return;
-    if ((i - head) % kChunk != 0) return;
-
-    // slots of this chunk: leading slots i, i+1, ... with the same id, at most kChunk
-    const uint64_t bal = __ballot(lane < kChunk && key_l == id);
-    const int cnt = __ffsll((unsigned long long)~bal) - 1;  // lane 0 always matches, so cnt >= 1
-    const bool continues = cnt == kChunk && __shfl(key_l, kChunk, CK_WAVE) == id;
-    const bool multi = (i != head) || continues;
-
-    if (cnt == 1 && !multi) {
-        // the only row of its id (nearly every slot when ids are spread over a large table): widened and rounded
-        // back, the row comes out as it went in, so it is copied - eight packets per lane in flight, no accumulators
-        const uint32_t pos = __shfl(pos_l, 0, CK_WAVE);
-        const P* src = reinterpret_cast<const P*>(dy + (int64_t)pos * H);
-        P* dst = reinterpret_cast<P*>(dw + (int64_t)id * H);
-        for (int64_t p0 = 0; p0 < packs; p0 += (int64_t)CK_WAVE * kRowPacks) {
-            P v[kRowPacks];
-#pragma unroll
-            for (int q = 0; q < kRowPacks; ++q) {
-                const int64_t p = p0 + lane + (int64_t)q * CK_WAVE;
-                if (p < packs) v[q] = nt_load(src + p);
-            }
-#pragma unroll
-            for (int q = 0; q < kRowPacks; ++q) {
-                const int64_t p = p0 + lane + (int64_t)q * CK_WAVE;
-                if (p < packs) nt_store(v[q], dst + p);
+    // Wave w of the workgroup looks at sorted slot 4 * blockIdx.x + w.  A slot that starts a chunk with a single
+    // row is copied by its wave alone.  The other chunk starts are summed by the four waves together, one after the
+    // other: each wave takes a quarter of the columns and keeps four rows of the chunk in flight, so a chunk of 32
+    // rows is 8 dependent round trips instead of 32 - under the load of the fill a round trip takes several
+    // microseconds, and with skewed ids the longest chain set the time of the launch.  The rows are still added in
+    // ascending token position, one accumulator per element.
+    static_assert(kChunk <= CK_WAVE, "a wave looks at the slots of a chunk with one lane each");
+    __shared__ uint32_t sh_pos[4][kChunk];
+    __shared__ int sh_cnt[4];     // rows of the chunk that starts at the wave's slot; 0: nothing left to sum
+    __shared__ int sh_multi[4];   // 0: the run is this chunk, rounded and stored; else 1 + (slot is the run's head)
+    __shared__ uint32_t sh_id[4];
+    const int wave = threadIdx.x / CK_WAVE;
+    const int i = blockIdx.x * 4 + wave;
+    {
+        int cnt = 0;
+        bool multi = false;
+        uint32_t id = 0, pos_l = 0;
+        int head = 0;
+        if (i < n) {
+            // every index load is issued before any of them is used: one round trip
+            id = skeys[i];
+            head = (int)run_head[i];
+            const bool in_range = lane < kChunk && i + lane < n;
+            const uint32_t key_l = in_range ? skeys[i + lane] : 0xffffffffu;
+            const uint32_t key_next = i + kChunk < n ? skeys[i + kChunk] : 0xffffffffu;  // first slot past the chunk
+            pos_l = in_range ? spos[i + lane] : 0u;
+            if ((int64_t)id < V && (i - head) % kChunk == 0) {
+                // slots of this chunk: leading slots i, i+1, ... with the same id, at most kChunk
+                const uint64_t bal = __ballot(key_l == id);
+                cnt = bal == ~0ull ? CK_WAVE : __ffsll((unsigned long long)~bal) - 1;  // lane 0 always matches, so cnt >= 1
+                const bool continues = cnt == kChunk && key_next == id;
+                multi = (i != head) || continues;
             }
         }
-        return;
+        if (cnt == 1 && !multi) {
+            // the only row of its id (nearly every slot when ids are spread over a large table): widened and rounded
+            // back, the row comes out as it went in, so it is copied - eight packets per lane in flight, no accumulators
+            const uint32_t pos = __shfl(pos_l, 0, CK_WAVE);
+            const P* src = reinterpret_cast<const P*>(dy + (int64_t)pos * H);
+            P* dst = reinterpret_cast<P*>(dw + (int64_t)id * H);
+            for (int64_t p0 = 0; p0 < packs; p0 += (int64_t)CK_WAVE * kRowPacks) {
+                P v[kRowPacks];
+#pragma unroll
+                for (int q = 0; q < kRowPacks; ++q) {
+                    const int64_t p = p0 + lane + (int64_t)q * CK_WAVE;
+                    if (p < packs) v[q] = nt_load(src + p);
+                }
+#pragma unroll
+                for (int q = 0; q < kRowPacks; ++q) {
+                    const int64_t p = p0 + lane + (int64_t)q * CK_WAVE;
+                    if (p < packs) nt_store(v[q], dst + p);
+                }
+            }
+            cnt = 0;
+        }
+        if (lane < kChunk) sh_pos[wave][lane] = pos_l;
+        if (lane == 0) {
+            sh_cnt[wave] = cnt;
+            sh_multi[wave] = multi ? 1 + (i == head ? 1 : 0) : 0;
+            sh_id[wave] = id;
+        }
     }
+    __syncthreads();
 
     // fp32 tables sum in fp64 so that the result is the correctly rounded sum whatever the order
     typedef typename AccOf<T>::type acc_t;
+    constexpr int kWavePacks = kRowPacks / 4;  // packets per lane and column tile that one of the four waves takes
+    constexpr int kRowsInFlight = 4;
     const int64_t tile = (int64_t)CK_WAVE * kRowPacks;
-    for (int64_t p0 = 0; p0 < packs; p0 += tile) {
-        acc_t acc[kRowPacks][VEC];
+    for (int owner = 0; owner < 4; ++owner) {
+        const int cnt = sh_cnt[owner];
+        if (cnt == 0) continue;  // the same for all four waves
+        const int multi = sh_multi[owner];
+        const int64_t id = sh_id[owner];
+        const int slot_i = blockIdx.x * 4 + owner;
+        for (int64_t p0 = 0; p0 < packs; p0 += tile) {
+            acc_t acc[kWavePacks][VEC];
 #pragma unroll
-        for (int q = 0; q < kRowPacks; ++q)
+            for (int q = 0; q < kWavePacks; ++q)
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) acc[q][j] = 0;
-        for (int r = 0; r < cnt; ++r) {
-            const uint32_t pos = __shfl(pos_l, r, CK_WAVE);
-            const P* src = reinterpret_cast<const P*>(dy + (int64_t)pos * H);
-            P v[kRowPacks];
+                for (int j = 0; j < VEC; ++j) acc[q][j] = 0;
+            for (int r0 = 0; r0 < cnt; r0 += kRowsInFlight) {
+                P v[kRowsInFlight][kWavePacks];
 #pragma unroll
-            for (int q = 0; q < kRowPacks; ++q) {
-                const int64_t p = p0 + lane + (int64_t)q * CK_WAVE;
-                if (p < packs) v[q] = nt_load(src + p);
-            }
+                for (int u = 0; u < kRowsInFlight; ++u) {
+                    if (r0 + u < cnt) {
+                        const P* src = reinterpret_cast<const P*>(dy + (int64_t)sh_pos[owner][r0 + u] * H);
 #pragma unroll
-            for (int q = 0; q < kRowPacks; ++q) {
-                const int64_t p = p0 + lane + (int64_t)q * CK_WAVE;
-                if (p < packs) {
+                        for (int q = 0; q < kWavePacks; ++q) {
+                            const int64_t p = p0 + lane + (int64_t)(wave * kWavePacks + q) * CK_WAVE;
+                            if (p < packs) v[u][q] = nt_load(src + p);
+                        }
+                    }
+                }
 #pragma unroll
-                    for (int j = 0; j < VEC; ++j) acc[q][j] += (acc_t)T::up(v[q].v[j]);
+                for (int u = 0; u < kRowsInFlight; ++u) {
+                    if (r0 + u < cnt) {
+#pragma unroll
+                        for (int q = 0; q < kWavePacks; ++q) {
+                            const int64_t p = p0 + lane + (int64_t)(wave * kWavePacks + q) * CK_WAVE;
+                            if (p < packs) {
+#pragma unroll
+                                for (int j = 0; j < VEC; ++j) acc[q][j] += (acc_t)T::up(v[u][q].v[j]);
+                            }
+                        }
+                    }
                 }
             }
-        }
-        if (!multi) {
-            P* dst = reinterpret_cast<P*>(dw + (int64_t)id * H);
+            if (multi == 0) {
+                P* dst = reinterpret_cast<P*>(dw + id * H);
 #pragma unroll
-            for (int q = 0; q < kRowPacks; ++q) {
-                const int64_t p = p0 + lane + (int64_t)q * CK_WAVE;
-                if (p < packs) {
-                    P o;
+                for (int q = 0; q < kWavePacks; ++q) {
+                    const int64_t p = p0 + lane + (int64_t)(wave * kWavePacks + q) * CK_WAVE;
+                    if (p < packs) {
+                        P o;
 #pragma unroll
-                    for (int j = 0; j < VEC; ++j) o.v[j] = T::down((float)acc[q][j]);
-                    nt_store(o, dst + p);
+                        for (int j = 0; j < VEC; ++j) o.v[j] = T::down((float)acc[q][j]);
+                        nt_store(o, dst + p);
+                    }
                 }
-            }
-        } else {
-            // at most two chunk starts of long runs fall into one window of kChunk slots: the last chunk
-            // of one run and the head of the next, told apart by the low bit
-            const int64_t slot = 2 * (int64_t)(i / kChunk) + (i == head ? 1 : 0);
-            float* dst = partial + slot * H;
+            } else {
+                // at most two chunk starts of long runs fall into one window of kChunk slots: the last chunk
+                // of one run and the head of the next, told apart by the low bit
+                const int64_t slot = 2 * (int64_t)(slot_i / kChunk) + (multi == 2 ? 1 : 0);
+                float* dst = partial + slot * H;
 #pragma unroll
-            for (int q = 0; q < kRowPacks; ++q) {
-                const int64_t p = p0 + lane + (int64_t)q * CK_WAVE;
-                if (p < packs) {
-                    if (VEC % 4 == 0) {
+                for (int q = 0; q < kWavePacks; ++q) {
+                    const int64_t p = p0 + lane + (int64_t)(wave * kWavePacks + q) * CK_WAVE;
+                    if (p < packs) {
+                        if (VEC % 4 == 0) {
 #pragma unroll
-                        for (int j = 0; j + 3 < VEC; j += 4)
-                            *reinterpret_cast<float4*>(dst + p * VEC + j) = make_float4(
-                                (float)acc[q][j], (float)acc[q][j + 1], (float)acc[q][j + 2], (float)acc[q][j + 3]);
-                    } else {
+                            for (int j = 0; j + 3 < VEC; j += 4)
+                                *reinterpret_cast<float4*>(dst + p * VEC + j) = make_float4(
+                                    (float)acc[q][j], (float)acc[q][j + 1], (float)acc[q][j + 2], (float)acc[q][j + 3]);
+                        } else {
 #pragma unroll
-                        for (int j = 0; j < VEC; ++j) dst[p * VEC + j] = (float)acc[q][j];
+                            for (int j = 0; j < VEC; ++j) dst[p * VEC + j] = (float)acc[q][j];
+                        }
                     }
                 }
             }

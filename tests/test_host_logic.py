@@ -41,7 +41,7 @@ def test_size_queries_run_without_a_gpu():
     assert lib.ck_moe_sort_workspace_size(1000, 1000) == 4 * 1000 * 4
     n, V, H = 32768, 128256, 4096
     size = lib.ck_embedding_backward_workspace_size(n, V, H)
-    assert size >= 5 * n * 4 + V + 2 * (n // 32) * H * 4
+    assert size >= 5 * n * 4 + V + 2 * (n // 64) * H * 4  # two fp32 partial rows per window of 64 sorted slots
     assert lib.ck_embedding_backward_workspace_size(0, 10, 8) >= 10
 
 
