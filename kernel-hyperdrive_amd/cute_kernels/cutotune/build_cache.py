@@ -13,6 +13,7 @@ from typing import Callable
 import torch
 
 from .. import (
+    MoE_Triton,
     add_scalar_cute,
     add_tensor_cute,
     embedding_cute,
@@ -60,6 +61,17 @@ def main() -> None:
             table = torch.randn(table_size, device=device, dtype=dtype, requires_grad=True)
             forward_backward(embedding_cute, input_ids=ids, weight=table)
             del table
+        if dtype != torch.float32:
+            # the grouped products of the benchmark's layers (tokens, hidden, intermediate, experts, top-k): whether the
+            # last round of tiles is split along the contraction
+            for T, H, I, E, k in ((8192, 4096, 14336, 8, 2), (16384, 2048, 1408, 64, 6)):
+                moe = MoE_Triton(num_experts=E, num_experts_per_tok=k, hidden_size=H, intermediate_size=I,
+                                 activation_function=swiglu_unchunked_cute, is_glu=True, add_bias=False, std=0.02)
+                moe = moe.to(device=device, dtype=dtype)
+                x = torch.randn(T, H, dtype=dtype, device=device, requires_grad=True)
+                moe(x)[0].sum().backward()
+                del moe, x
+                torch.cuda.empty_cache()
         print(dtype, "done", flush=True)
 
     cache = get_cutotune_cache()

@@ -27,14 +27,48 @@ import torch
 
 from ... import _C
 from ...constants import LIBRARY_NAME
+from ...cutotune import CutoTuneConfig, CutoTuneParameter, cutotune, get_cartesian_product_cutotune_configs
 from ...utils import cute_op
 
 
 torch._dynamo.config.capture_scalar_outputs = True
 
-# scatter2scatter splits the tail of its tile grid along the contraction when the shape allows it (False: one
-# workgroup per tile throughout)
-SPLIT_TILE_TAIL = True
+# Whether scatter2scatter splits the tail of its tile grid along the contraction where the shape allows it: None
+# leaves it to the tuner (per dtype, contraction length, output width, expert count and order of magnitude of the
+# row count), True / False fix it.  One workgroup per tile throughout is the other form of the same launch.
+SPLIT_TILE_TAIL: bool | None = None
+
+
+# The reference tunes the tile of its grouped products per shape (triton_implementation/kernels.py:152-159, BLOCK_M of
+# groupXtY); the choice that moves these kernels is how the last, partly filled round of tiles is run: whole tiles
+# (the CUs without one idle for a tile time) or cut along the contraction over the idle CUs and summed by a second
+# launch (a few per cent either way, depending on how full the last round is and how long the contraction).
+@cutotune(
+    configs=get_cartesian_product_cutotune_configs(split_tile_tail=[True, False]),
+    default_config=CutoTuneConfig({"split_tile_tail": True}),
+    triggers={"X.dtype", "X.size(1)", "out.size(1)", "W.size(0)"},
+    functional_triggers={"rows_log2": lambda **kwargs: int(kwargs["out"].size(0)).bit_length()},
+)
+def scatter2scatter_launch(
+    X: torch.Tensor,
+    W: torch.Tensor,
+    sorted_scattered_idxs: torch.Tensor,
+    expert_offsets: torch.Tensor,
+    out: torch.Tensor,
+    FAN_OUT: int,
+    x_grouped: bool,
+    y_grouped: bool,
+    bias: torch.Tensor | None,
+    split_tile_tail: bool,
+) -> None:
+    workspace = None
+    if split_tile_tail:
+        # room for the partial sums of the pieces
+        nbytes = _C.scatter2scatter_workspace_size(out.size(0), X.size(1), out.size(1), W.size(0), X.dtype)
+        if nbytes > 0:
+            workspace = torch.empty(nbytes, dtype=torch.uint8, device=X.device)
+    _C.scatter2scatter(X, W, sorted_scattered_idxs, expert_offsets, out, FAN_OUT, x_grouped, y_grouped, workspace,
+                       bias)
 
 
 @cute_op(f"{LIBRARY_NAME}::scatter2scatter", mutates_args={"out"})
@@ -61,15 +95,17 @@ def scatter2scatter(
         _C.offsets_from_sorted(sorted_expert_idxs.contiguous(), expert_offsets)
     if X.stride(1) != 1:
         X = X.contiguous()
-    # long contractions over few column tiles: the last round of tiles is split over the idle CUs (needs room for
-    # the pieces' partial sums)
-    workspace = None
-    if SPLIT_TILE_TAIL:
-        nbytes = _C.scatter2scatter_workspace_size(out.size(0), X.size(1), out.size(1), W.size(0), X.dtype)
-        if nbytes > 0:
-            workspace = torch.empty(nbytes, dtype=torch.uint8, device=X.device)
-    _C.scatter2scatter(X, W, sorted_scattered_idxs, expert_offsets, out, FAN_OUT, x_grouped, y_grouped, workspace,
-                       bias)
+    # only long contractions over few column tiles have a tail worth splitting; everything else has one form
+    eligible = _C.scatter2scatter_workspace_size(out.size(0), X.size(1), out.size(1), W.size(0), X.dtype) > 0
+    if not eligible:
+        choice = False
+    elif SPLIT_TILE_TAIL is None:
+        choice = CutoTuneParameter()
+    else:
+        choice = SPLIT_TILE_TAIL
+    scatter2scatter_launch(X=X, W=W, sorted_scattered_idxs=sorted_scattered_idxs, expert_offsets=expert_offsets,
+                           out=out, FAN_OUT=FAN_OUT, x_grouped=x_grouped, y_grouped=y_grouped, bias=bias,
+                           split_tile_tail=choice)
 
 
 @cute_op(f"{LIBRARY_NAME}::scatter2scatter_glu", mutates_args={"h", "act"})

@@ -1,5 +1,8 @@
 """The tuning cache that ships with the package is the one the launchers follow on the GPU.
 
+Same for the grouped product's one tunable (the last round of tiles split along the contraction or not): for the two
+eligible products of the Mixtral-shape step the launch has to carry a workspace exactly when the cache says so.
+
 For every RMSNorm entry of the committed cache file (function, dtype, row length, weight or not) one call of the
 public operator has to hand the cached BLOCK_SIZE_B - the launch variant - to the library, forward and backward,
 and still give torch's values.  Reference: the cache keys and the two-layer tuning of
@@ -82,3 +85,56 @@ def test_rmsnorm_launches_the_cached_variant(monkeypatch, dtype, hidden, has_wei
     y_ref.backward(dy)
     assert_close(y, y_ref, dtype)
     assert_close(x.grad, x_ref.grad, dtype)
+
+
+_S2S = "kernels/scattermoe/ops.py->scatter2scatter_launch"
+
+
+def test_the_committed_cache_holds_the_grouped_products_of_the_benchmark():
+    with open(_CUTOTUNE_CACHE_FILENAME) as f:
+        document = yaml.safe_load(f)
+    keys = document["best_configs"].get(_S2S, {})
+    # forward c_proj (K = I) and dX of c_fc (K = 2 I) of the Mixtral shape, 16384 routed rows, 8 experts
+    for K in (14336, 28672):
+        wanted = [k for k in keys if "torch.bfloat16" in k and f"X.size(1) = {K}" in k and "out.size(1) = 4096" in k
+                  and "W.size(0) = 8" in k and "rows_log2 = 15" in k]
+        assert len(wanted) == 1, (K, list(keys))
+        timed = document["all_configs"][_S2S][wanted[0]]
+        assert sorted(e["config"]["split_tile_tail"] for e in timed) == [False, True]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("K", [14336, 28672])
+def test_scatter2scatter_launches_the_cached_choice(monkeypatch, K):
+    from cute_kernels.kernels.scattermoe import ops
+
+    with open(_CUTOTUNE_CACHE_FILENAME) as f:
+        keys = yaml.safe_load(f)["best_configs"][_S2S]
+    (key,) = [k for k in keys if "torch.bfloat16" in k and f"X.size(1) = {K}" in k and "out.size(1) = 4096" in k
+              and "W.size(0) = 8" in k and "rows_log2 = 15" in k]
+    cached = keys[key]["config"]["split_tile_tail"]
+
+    seen = {}
+    real = _C.scatter2scatter
+
+    def spy(X, W, idx, offsets, out, fan_out, x_grouped, y_grouped, workspace=None, bias=None):
+        seen["split"] = workspace is not None
+        return real(X, W, idx, offsets, out, fan_out, x_grouped, y_grouped, workspace, bias)
+
+    monkeypatch.setattr(_C, "scatter2scatter", spy)
+    assert ops.SPLIT_TILE_TAIL is None, "the tuner decides unless somebody fixed the choice"
+
+    E, N, M = 8, 4096, 16384
+    g = torch.Generator(device="cuda").manual_seed(K)
+    X = torch.randn(M, K, device="cuda", dtype=torch.bfloat16, generator=g)
+    W = (torch.randn(E, N, K, device="cuda", dtype=torch.bfloat16, generator=g) * 0.02).permute(0, 2, 1)
+    sorted_experts = torch.arange(M, device="cuda") * E // M
+    sorted_slots = torch.randperm(M, device="cuda", generator=g)
+    offsets = torch.bincount(sorted_experts, minlength=E).cumsum(0)
+    out = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
+    ops.scatter2scatter(X, W, sorted_experts, sorted_slots, out, 1, True, False, offsets)
+    assert seen == {"split": cached}
+    # and the product itself, on a few rows, against the plain matrix product of their expert
+    rows = torch.tensor([0, 2047, 2048, 9000, M - 1], device="cuda")
+    expected = torch.stack([X[r].float() @ W[int(sorted_experts[r])].float() for r in rows])
+    assert_close(out[sorted_slots[rows]], expected.to(torch.bfloat16), torch.bfloat16)
