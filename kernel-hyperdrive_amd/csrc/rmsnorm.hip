@@ -293,6 +293,11 @@ __device__ __forceinline__ void rmsnorm_bwd_body(const typename T::storage_t* __
                                                  float* __restrict__ dw_partial, int64_t B, int H, float eps) {
     typedef VPack<T, T::kVec> P;
     constexpr int N = NP != 0 ? NP : kMaxPacks;
+    // The 1024-lane team has 128 registers per lane.  With a weight, the packed x, dy and weight of the row plus the
+    // 64 fp32 dweight accumulators are 160: the compiler then spills 500 bytes per lane and the kernel runs seven
+    // times longer than without a weight (538 against 75 us at 2048 x 32768).  So there only the accumulators are
+    // kept: x, dy and the weight are read twice, the second time from the cache the first read left them in.
+    constexpr bool LEAN = HAS_W && TPR == 1024;
     __shared__ float red[16];
     const int teams_per_block = blockDim.x / TPR;
     const int team = blockIdx.x * teams_per_block + threadIdx.x / TPR;
@@ -301,20 +306,21 @@ __device__ __forceinline__ void rmsnorm_bwd_body(const typename T::storage_t* __
     const int packs = H / T::kVec;
     const float inv_h = 1.0f / (float)H;
 
-    P wv[kMaxPacks];
+    P wv[LEAN ? 1 : kMaxPacks];
     float dw[kMaxPacks][T::kVec];
     if (HAS_W) {
 #pragma unroll
         for (int i = 0; i < N; ++i) {
             const int p = t + i * TPR;
-            if (NP != 0 || p < packs) wv[i] = reinterpret_cast<const P*>(w)[p];
+            if (!LEAN && (NP != 0 || p < packs)) wv[i] = reinterpret_cast<const P*>(w)[p];
 #pragma unroll
             for (int j = 0; j < T::kVec; ++j) dw[i][j] = 0.f;
         }
     }
 
     // rows are dealt round-robin; with TPR > 64 the block is one team so the trip count is block-uniform
-    P xv[kMaxPacks], gv[kMaxPacks], xn[PREFETCH ? kMaxPacks : 1], gn[PREFETCH ? kMaxPacks : 1];
+    static_assert(!(LEAN && PREFETCH), "the lean form has no row in flight");
+    P xv[LEAN ? 1 : kMaxPacks], gv[LEAN ? 1 : kMaxPacks], xn[PREFETCH ? kMaxPacks : 1], gn[PREFETCH ? kMaxPacks : 1];
     if (PREFETCH && team < B) {
         const P* xr = reinterpret_cast<const P*>(x + (int64_t)team * H);
         const P* gr = reinterpret_cast<const P*>(dy + (int64_t)team * H);
@@ -347,7 +353,7 @@ __device__ __forceinline__ void rmsnorm_bwd_body(const typename T::storage_t* __
                     }
                 }
             }
-        } else {
+        } else if (!LEAN) {
             const P* xr = reinterpret_cast<const P*>(x + row * H);
             const P* gr = reinterpret_cast<const P*>(dy + row * H);
 #pragma unroll
@@ -360,22 +366,44 @@ __device__ __forceinline__ void rmsnorm_bwd_body(const typename T::storage_t* __
             }
         }
         float ss = 0.f, dot = 0.f;
+        if (LEAN) {
+            // everything passes through (plain loads: the packets are wanted again below), two packets at a time
+            const P* xr = reinterpret_cast<const P*>(x + row * H);
+            const P* gr = reinterpret_cast<const P*>(dy + row * H);
 #pragma unroll
-        for (int i = 0; i < N; ++i) {
-            const int p = t + i * TPR;
-            if (NP != 0 || p < packs) {
+            for (int i = 0; i < N; ++i) {
+                const int p = t + i * TPR;
+                if (NP != 0 || p < packs) {
+                    const P x8 = xr[p];
+                    const P g8 = gr[p];
+                    const P w8 = reinterpret_cast<const P*>(w)[p];
 #pragma unroll
-                for (int j = 0; j < T::kVec; ++j) {
-                    const float xf = T::up(xv[i].v[j]);
-                    float g = T::up(gv[i].v[j]);
-                    if (HAS_W) g *= T::up(wv[i].v[j]);
-                    ss += xf * xf;
-                    dot += g * xf;
+                    for (int j = 0; j < T::kVec; ++j) {
+                        const float xf = T::up(x8.v[j]);
+                        ss += xf * xf;
+                        dot += T::up(g8.v[j]) * T::up(w8.v[j]) * xf;
+                    }
                 }
+                if (i % 2 == 1) __builtin_amdgcn_sched_barrier(0);
             }
-            __builtin_amdgcn_sched_barrier(0);
+        } else {
+#pragma unroll
+            for (int i = 0; i < N; ++i) {
+                const int p = t + i * TPR;
+                if (NP != 0 || p < packs) {
+#pragma unroll
+                    for (int j = 0; j < T::kVec; ++j) {
+                        const float xf = T::up(xv[i].v[j]);
+                        float g = T::up(gv[i].v[j]);
+                        if (HAS_W) g *= T::up(wv[i].v[j]);
+                        ss += xf * xf;
+                        dot += g * xf;
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
-        if (sizeof(typename T::storage_t) == 2) {
+        if (!LEAN && sizeof(typename T::storage_t) == 2) {
             // 16-bit rows: keep only the packed form across the reductions
 #pragma unroll
             for (int i = 0; i < N; ++i) {
@@ -400,13 +428,23 @@ __device__ __forceinline__ void rmsnorm_bwd_body(const typename T::storage_t* __
             const int p = t + i * TPR;
             if (NP != 0 || p < packs) {
                 P o;
+                P x8, g8, w8;
+                if (LEAN) {
+                    x8 = reinterpret_cast<const P*>(x + row * H)[p];
+                    g8 = reinterpret_cast<const P*>(dy + row * H)[p];
+                    w8 = reinterpret_cast<const P*>(w)[p];
+                } else {
+                    x8 = xv[LEAN ? 0 : i];
+                    g8 = gv[LEAN ? 0 : i];
+                    if (HAS_W) w8 = wv[LEAN ? 0 : i];
+                }
 #pragma unroll
                 for (int j = 0; j < T::kVec; ++j) {
-                    const float xf = T::up(xv[i].v[j]);
-                    const float d = T::up(gv[i].v[j]);
+                    const float xf = T::up(x8.v[j]);
+                    const float d = T::up(g8.v[j]);
                     float g = d;
                     if (HAS_W) {
-                        g *= T::up(wv[i].v[j]);
+                        g *= T::up(w8.v[j]);
                         dw[i][j] += d * (xf * rstd);
                     }
                     o.v[j] = T::down(rstd * g - c * xf);
@@ -855,10 +893,12 @@ static void launch_bwd(unsigned grid, int block, hipStream_t s, const BwdArgs& a
 template <typename T, int NP>
 static void launch_bwd_two_np(unsigned grid, hipStream_t s, const BwdArgs& a) {
     typedef typename T::storage_t S;
-    if (a.weight)
-        hipLaunchKernelGGL((ck::rmsnorm_bwd_two_kernel<T, true, NP>), dim3(grid), dim3(256), 0, s, (const S*)a.x,
-                           (const S*)a.weight, (const S*)a.dy, a.rstd, (S*)a.dx, a.ws, a.B, a.H, a.eps);
-    else
+    if (a.weight) {
+        // (16-bit rows of a generic packet count with a weight never come here - see two_fits - and are not compiled)
+        if constexpr (NP != 0 || sizeof(S) == 4)
+            hipLaunchKernelGGL((ck::rmsnorm_bwd_two_kernel<T, true, NP>), dim3(grid), dim3(256), 0, s, (const S*)a.x,
+                               (const S*)a.weight, (const S*)a.dy, a.rstd, (S*)a.dx, a.ws, a.B, a.H, a.eps);
+    } else
         hipLaunchKernelGGL((ck::rmsnorm_bwd_two_kernel<T, false, NP>), dim3(grid), dim3(256), 0, s, (const S*)a.x,
                            (const S*)a.weight, (const S*)a.dy, a.rstd, (S*)a.dx, a.ws, a.B, a.H, a.eps);
 }
@@ -894,15 +934,23 @@ extern "C" int ck_rmsnorm_backward(const void* x, const void* weight, const void
     CK_DISPATCH_DTYPE(dtype, {
         typedef typename T::storage_t S;
         if (tpr != 0) {
-            const bool two = tpr == 64 && (block_size_b == 0 ? bwd_default_variant(H, dtype) : block_size_b) == 1;
+            const int np = tpr == 1024 ? 0 : exact_packs(H, dtype, tpr);
+            const int64_t row_packs = H / (dtype == CK_F32 ? 4 : 8);
+            // 16-bit rows with a weight that are neither 1, 2 nor 4 packets per lane: the two-workgroup form would
+            // spill (it is compiled for 256 registers), the one-workgroup form holds them
+            const bool two_fits = !(weight && dtype != CK_F32 && (np == 0 || np == 8) && row_packs != 64);
+            const bool two = tpr == 64 && two_fits &&
+                             (block_size_b == 0 ? bwd_default_variant(H, dtype) : block_size_b) == 1;
             const int teams = bwd_teams(B, tpr, two ? 2 : 1);
             const int block = tpr > 256 ? tpr : 256;
             const unsigned grid = (unsigned)(teams / (block / tpr));
             const BwdArgs a = {x, weight, output_grad, rstd, x_grad, ws, B, (int)H, eps};
-            const int np = tpr == 1024 ? 0 : exact_packs(H, dtype, tpr);
             if (two) {
-                // (the branch-free forms of this variant need more than the 256 registers two waves per SIMD leave)
+                // (the branch-free form for eight packets per lane needs more than the 256 registers two waves per
+                // SIMD leave; the short exact rows are the ones this variant is the default for)
                 if (np == 4) launch_bwd_two_np<T, 4>(grid, s, a);
+                else if (np == 2) launch_bwd_two_np<T, 2>(grid, s, a);
+                else if (row_packs == 64) launch_bwd_two_np<T, 1>(grid, s, a);
                 else launch_bwd_two_np<T, 0>(grid, s, a);
             } else if (tpr == 64) launch_bwd<T, 64>(grid, block, s, a, np);
             else if (tpr == 256) launch_bwd<T, 256>(grid, block, s, a, np);

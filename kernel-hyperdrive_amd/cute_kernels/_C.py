@@ -233,11 +233,42 @@ def _same_dtype(ref: torch.Tensor, what: str, **others: torch.Tensor) -> None:
 
 
 # ---- one Python function per C entry point ----------------------------------------------------------
+def _walks_linearly(t: torch.Tensor) -> bool:
+    """Dense in memory in some order of its dimensions (a transposed tensor, for instance)."""
+    if t.is_contiguous():
+        return True
+    order = sorted(range(t.dim()), key=lambda d: t.stride(d), reverse=True)
+    return t.permute(order).is_contiguous()
+
+
+def _dense_like(ref: torch.Tensor, what: str, **others: torch.Tensor | None) -> None:
+    """The kernels that take no strides read `numel` consecutive elements from every pointer: the operands have to be
+    dense, of the first operand's type and number of elements, and laid out like it."""
+    for name, t in dict(first=ref, **others).items():
+        if t is None:
+            continue
+        label = name if name != "first" else "the first operand"
+        if not _walks_linearly(t) or (t.numel() > 0 and t.stride() != ref.stride() and not
+                                      (t.is_contiguous() and ref.is_contiguous())):
+            raise ValueError(f"{what}: {label} must be dense in memory and laid out like the first operand")
+        if t.dtype != ref.dtype:
+            raise ValueError(f"{what}: {name} is {t.dtype}, expected {ref.dtype} like the first operand")
+        if t.numel() != ref.numel():
+            raise ValueError(f"{what}: {name} has {t.numel()} elements, the first operand {ref.numel()}")
+
+
+def _dense(what: str, **tensors: torch.Tensor | None) -> None:
+    for name, t in tensors.items():
+        if t is not None and not t.is_contiguous():
+            raise ValueError(f"{what}: {name} must be contiguous")
+
+
 # All tensors must be contiguous unless a stride is passed explicitly.
 
 
 def add_tensor_forward(x, y, output, block_size: int) -> None:
     lib = load_library()
+    _dense_like(x, "add_tensor_forward", y=y, output=output)
     with _Launch(x, y, output) as L:
         _check(
             lib.ck_add_tensor_forward(_ptr(x), _ptr(y), _ptr(output), x.numel(), dtype_code(x.dtype), block_size,
@@ -248,6 +279,7 @@ def add_tensor_forward(x, y, output, block_size: int) -> None:
 
 def add_scalar_forward(x, y: float, output, block_size: int) -> None:
     lib = load_library()
+    _dense_like(x, "add_scalar_forward", output=output)
     with _Launch(x, output) as L:
         _check(
             lib.ck_add_scalar_forward(_ptr(x), float(y), _ptr(output), x.numel(), dtype_code(x.dtype), block_size,
@@ -258,6 +290,7 @@ def add_scalar_forward(x, y: float, output, block_size: int) -> None:
 
 def swiglu_forward(gate, up, output, block_size: int) -> None:
     lib = load_library()
+    _dense_like(gate, "swiglu_forward", up=up, output=output)
     with _Launch(gate, up, output) as L:
         _check(
             lib.ck_swiglu_forward(_ptr(gate), _ptr(up), _ptr(output), gate.numel(), dtype_code(gate.dtype),
@@ -268,6 +301,7 @@ def swiglu_forward(gate, up, output, block_size: int) -> None:
 
 def swiglu_backward(gate, up, output_grad, gate_grad, up_grad, block_size: int) -> None:
     lib = load_library()
+    _dense_like(gate, "swiglu_backward", up=up, output_grad=output_grad, gate_grad=gate_grad, up_grad=up_grad)
     with _Launch(gate, up, output_grad, gate_grad, up_grad) as L:
         _check(
             lib.ck_swiglu_backward(_ptr(gate), _ptr(up), _ptr(output_grad), _ptr(gate_grad), _ptr(up_grad),
@@ -278,6 +312,10 @@ def swiglu_backward(gate, up, output_grad, gate_grad, up_grad, block_size: int) 
 
 def swiglu_unchunked_forward(x, output, block_size: int) -> None:
     lib = load_library()
+    _same_dtype(x, "swiglu_unchunked_forward", output=output)
+    _dense("swiglu_unchunked_forward", x=x, output=output)
+    if x.size(-1) % 2 != 0 or 2 * output.numel() != x.numel():
+        raise ValueError("swiglu_unchunked_forward: the last dimension is (up | gate), the output holds half of it")
     H = x.size(-1)
     B = x.numel() // H if H > 0 else 0
     with _Launch(x, output) as L:
@@ -289,6 +327,11 @@ def swiglu_unchunked_forward(x, output, block_size: int) -> None:
 
 def swiglu_unchunked_backward(x, output_grad, x_grad, block_size: int) -> None:
     lib = load_library()
+    _dense_like(x, "swiglu_unchunked_backward", x_grad=x_grad)
+    _same_dtype(x, "swiglu_unchunked_backward", output_grad=output_grad)
+    _dense("swiglu_unchunked_backward", output_grad=output_grad)
+    if x.size(-1) % 2 != 0 or 2 * output_grad.numel() != x.numel():
+        raise ValueError("swiglu_unchunked_backward: the last dimension is (up | gate), output_grad holds half of it")
     H = x.size(-1)
     B = x.numel() // H if H > 0 else 0
     with _Launch(x, output_grad, x_grad) as L:
@@ -299,11 +342,21 @@ def swiglu_unchunked_backward(x, output_grad, x_grad, block_size: int) -> None:
         )
 
 
+def _row_operands(what: str, x, B: int, H: int, weight, rstd, **same_shape) -> None:
+    """Dense [B, H] tensors of x's type, a dense weight of H elements, fp32 1/rms of B elements (each may be None)."""
+    _dense_like(x, what, **same_shape)
+    if weight is not None and (weight.numel() != H or not weight.is_contiguous()):
+        raise ValueError(f"{what}: the weight must be a dense vector of {H} elements")
+    if rstd is not None and (rstd.dtype != torch.float32 or rstd.numel() != B or not rstd.is_contiguous()):
+        raise ValueError(f"{what}: the 1 / rms buffer must be dense fp32 with one element per row ({B})")
+
+
 def rmsnorm_forward(x, weight, output, rstd, eps: float, block_size_b: int = 0) -> None:
     lib = load_library()
     _same_dtype(x, "rmsnorm_forward", weight=weight, output=output)
     H = x.size(-1)
     B = x.numel() // H if H > 0 else 0
+    _row_operands("rmsnorm_forward", x, B, H, weight, rstd, output=output)
     with _Launch(x, weight, output, rstd) as L:
         _check(
             lib.ck_rmsnorm_forward(_ptr(x), _ptr(weight), _ptr(output), _ptr(rstd), B, H, eps, dtype_code(x.dtype),
@@ -322,6 +375,8 @@ def residual_rmsnorm_forward(x, residual, weight, output, residual_out, rstd, ep
             raise ValueError("residual_rmsnorm_forward: x, residual, output and residual_out must be dense and alike")
     if not x.is_contiguous():
         raise ValueError("residual_rmsnorm_forward: x must be dense")
+    _same_dtype(x, "residual_rmsnorm_forward", weight=weight)
+    _row_operands("residual_rmsnorm_forward", x, B, H, weight, rstd)
     with _Launch(x, residual, weight, output, residual_out, rstd) as L:
         _check(
             lib.ck_residual_rmsnorm_forward(_ptr(x), _ptr(residual), _ptr(weight), _ptr(output), _ptr(residual_out),
@@ -342,6 +397,10 @@ def rmsnorm_backward(x, weight, output_grad, rstd, x_grad, weight_grad, workspac
     _same_dtype(x, "rmsnorm_backward", weight=weight, output_grad=output_grad, x_grad=x_grad, weight_grad=weight_grad)
     H = x.size(-1)
     B = x.numel() // H if H > 0 else 0
+    _row_operands("rmsnorm_backward", x, B, H, weight, rstd, output_grad=output_grad, x_grad=x_grad)
+    if (weight is None) != (weight_grad is None) or (weight_grad is not None and (
+            weight_grad.numel() != H or not weight_grad.is_contiguous())):
+        raise ValueError("rmsnorm_backward: weight_grad goes with the weight, a dense vector of its size")
     with _Launch(x, weight, output_grad, rstd, x_grad, weight_grad, workspace) as L:
         _check(
             lib.ck_rmsnorm_backward(_ptr(x), _ptr(weight), _ptr(output_grad), _ptr(rstd), _ptr(x_grad),
@@ -354,6 +413,10 @@ def rmsnorm_backward(x, weight, output_grad, rstd, x_grad, weight_grad, workspac
 
 def embedding_forward(input_ids, weight, output) -> None:
     lib = load_library()
+    _same_dtype(weight, "embedding_forward", output=output)
+    _dense("embedding_forward", input_ids=input_ids, weight=weight, output=output)
+    if weight.dim() != 2 or output.numel() != input_ids.numel() * weight.size(1):
+        raise ValueError("embedding_forward: weight [V, H], output one row of H per id")
     with _Launch(input_ids, weight, output) as L:
         _check(
             lib.ck_embedding_forward(_ptr(input_ids), _ids_are_i32(input_ids), _ptr(weight), _ptr(output),
@@ -369,6 +432,11 @@ def embedding_backward_workspace_size(num_ids: int, V: int, H: int) -> int:
 
 def embedding_backward(input_ids, output_grad, weight_grad, workspace) -> None:
     lib = load_library()
+    _same_dtype(weight_grad, "embedding_backward", output_grad=output_grad)
+    _dense("embedding_backward", input_ids=input_ids, output_grad=output_grad, weight_grad=weight_grad,
+           workspace=workspace)
+    if weight_grad.dim() != 2 or output_grad.numel() != input_ids.numel() * weight_grad.size(1):
+        raise ValueError("embedding_backward: weight_grad [V, H], output_grad one row of H per id")
     with _Launch(input_ids, output_grad, weight_grad, workspace) as L:
         _check(
             lib.ck_embedding_backward(_ptr(input_ids), _ids_are_i32(input_ids), _ptr(output_grad), _ptr(weight_grad),
@@ -572,6 +640,9 @@ def moe_combine_forward(expanded, gates, out) -> None:
     lib = load_library()
     T, k, H = expanded.shape
     _same_dtype(expanded, "moe_combine_forward", gates=gates, out=out)
+    _dense("moe_combine_forward", expanded=expanded, gates=gates, out=out)
+    if out.numel() != T * H or (gates is not None and gates.numel() != T * k):
+        raise ValueError("moe_combine_forward: expanded [T, k, H], gates [T, k], out [T, H]")
     with _Launch(expanded, gates, out) as L:
         _check(
             lib.ck_moe_combine_forward(_ptr(expanded), _ptr(gates), _ptr(out), T, k, H, dtype_code(expanded.dtype),
@@ -585,6 +656,9 @@ def moe_combine_backward_gates(expanded, grad_out, d_gates) -> None:
     lib = load_library()
     T, k, H = expanded.shape
     _same_dtype(expanded, "moe_combine_backward_gates", grad_out=grad_out, d_gates=d_gates)
+    _dense("moe_combine_backward_gates", expanded=expanded, grad_out=grad_out, d_gates=d_gates)
+    if grad_out.numel() != T * H or d_gates.numel() != T * k:
+        raise ValueError("moe_combine_backward_gates: expanded [T, k, H], grad_out [T, H], d_gates [T, k]")
     with _Launch(expanded, grad_out, d_gates) as L:
         _check(
             lib.ck_moe_combine_backward_gates(_ptr(expanded), _ptr(grad_out), _ptr(d_gates), T, k, H,

@@ -263,6 +263,32 @@ def test_binding_checks_index_and_operand_types_before_any_launch():
                     torch.zeros(2, dtype=torch.int64), None, 2)
     with pytest.raises(ValueError, match="weight is torch.float32"):
         _C.rmsnorm_forward(X, torch.ones(8), torch.empty_like(X), None, 1e-5)
+    # kernels without stride arguments: dense operands of one type and size
+    a = torch.zeros(4, 8, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="dense in memory"):
+        _C.swiglu_forward(a, a.t(), torch.empty_like(a), 256)
+    with pytest.raises(ValueError, match="up is torch.float32"):
+        _C.swiglu_forward(a, a.float(), torch.empty_like(a), 256)
+    with pytest.raises(ValueError, match="output has 16 elements"):
+        _C.add_tensor_forward(a, a, torch.zeros(4, 4, dtype=torch.bfloat16), 256)
+    with pytest.raises(ValueError, match="holds half"):
+        _C.swiglu_unchunked_forward(a, torch.zeros(4, 8, dtype=torch.bfloat16), 256)
+    with pytest.raises(ValueError, match="dense vector of 8"):
+        _C.rmsnorm_forward(a, torch.ones(4, dtype=torch.bfloat16), torch.empty_like(a), None, 1e-5)
+    with pytest.raises(ValueError, match="one element per row"):
+        _C.rmsnorm_forward(a, None, torch.empty_like(a), torch.zeros(3), 1e-5)
+    with pytest.raises(ValueError, match="dense in memory"):
+        _C.rmsnorm_backward(a, None, torch.zeros(8, 4, dtype=torch.bfloat16).t(), None, torch.empty_like(a), None, None, 1e-5)
+    with pytest.raises(ValueError, match="one row of H per id"):
+        _C.embedding_forward(torch.arange(3), a, torch.zeros(2, 8, dtype=torch.bfloat16))
+    with pytest.raises(ValueError, match="output_grad is torch.float32"):
+        _C.embedding_backward(torch.arange(3), torch.zeros(3, 8), a, torch.zeros(16, dtype=torch.uint8))
+    with pytest.raises(ValueError, match=r"gates \[T, k\]"):
+        _C.moe_combine_forward(torch.zeros(2, 2, 8, dtype=torch.bfloat16), torch.zeros(2, 3, dtype=torch.bfloat16),
+                               torch.zeros(2, 8, dtype=torch.bfloat16))
+    # a transposed pair laid out alike is as good as a contiguous one
+    with pytest.raises(RuntimeError, match="GPU tensors"):
+        _C.add_tensor_forward(a.t(), a.t(), torch.empty_like(a).t(), 256)
     # operands that pass the checks get as far as the device check
     with pytest.raises(RuntimeError, match="GPU tensors"):
         _C.scatter2scatter(X, W, idx.int(), off.int(), out, 1, True, True)
