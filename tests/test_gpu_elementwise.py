@@ -263,7 +263,7 @@ def test_embedding(gpu, dtype, ids_shape, table):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("case", ["zipf", "one_row", "int32_ids", "empty"])
+@pytest.mark.parametrize("case", ["zipf", "one_row", "run_lengths", "int32_ids", "empty"])
 def test_embedding_duplicates(gpu, dtype, case):
     from cute_kernels import embedding_cute
 
@@ -273,6 +273,12 @@ def test_embedding_duplicates(gpu, dtype, case):
         ids = O.zipf_ids((4, 2048), V, 1.1, seed=17)
     elif case == "one_row":
         ids = torch.full((3000,), 77, dtype=torch.long)  # one run far longer than a chunk
+    elif case == "run_lengths":
+        # runs at and around the chunk of 64 slots and the waves' ranges of 256 slots, among single ids, in shuffled
+        # token order: chunk boundaries, the last chunk of a run that ends on one, run heads far behind a wave's range
+        lengths = [1, 63, 64, 65, 1, 1, 127, 128, 129, 2, 191, 192, 193, 255, 256, 257, 3, 320, 511, 512, 513, 1, 1000]
+        ids = torch.cat([torch.full((n,), 10 + 7 * r, dtype=torch.long) for r, n in enumerate(lengths)])
+        ids = ids[torch.randperm(ids.numel(), generator=torch.Generator().manual_seed(18))]
     elif case == "int32_ids":
         ids = torch.randint(0, V, (2, 300), generator=torch.Generator().manual_seed(18)).int()
     else:
