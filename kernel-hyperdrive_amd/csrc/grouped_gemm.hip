@@ -767,6 +767,7 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
     // that pair with them (glu_half is a multiple of BN / 2, checked by the host)
     const int n_base = GLU == 1 ? nt * (BN / 2) : nt * BN;
     const int cols_valid = GLU == 1 ? BN : min(BN, p.N - n_base);  // > 0 and a multiple of 8
+    const bool upper_cols_live = cols_valid > BN / 2;  // likewise for the last column tile of an odd half-tile count
 
     // ---- global sources of the LDS slots this lane fills ---------------------------------------------
     typedef __attribute__((address_space(1))) const char* gchar_t;
@@ -1004,13 +1005,13 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
     auto multiply_tile = [&](const char* st) __attribute__((always_inline)) {
         read_a(st, 0, fa);
         read_b(st, 0, fb0);
-        read_b(st, 1, fb1);
+        if (upper_cols_live) read_b(st, 1, fb1);
         mma_quad(0, 0, fa, fb0);
-        mma_quad(0, 1, fa, fb1);
+        if (upper_cols_live) mma_quad(0, 1, fa, fb1);
         __builtin_amdgcn_sched_barrier(0);
         if (upper_rows_live) {
             read_a(st, 1, fa);
-            mma_quad(1, 1, fa, fb1);
+            if (upper_cols_live) mma_quad(1, 1, fa, fb1);
             mma_quad(1, 0, fa, fb0);
         }
     };
@@ -1051,8 +1052,11 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
     // `upper` says, as a type, whether the upper half of the tile's rows holds any row of the segment: where it holds
     // none (the last row tile of an expert with at most BM / 2 rows left) its fragments are not read and its matrix
     // instructions not issued, while barriers and copies stay as they are, so the counts of the waits still hold.
-    auto pp_step = [&](auto upper, int kt, char* X, char* Y, frag_t (*bl)[TNH], frag_t (*bu)[TNH]) __attribute__((always_inline)) {
+    // `upper_cols` says the same of the upper half of the tile's columns (an output width of an odd number of half
+    // tiles, 1408 = 5.5 x 256 for instance).
+    auto pp_step = [&](auto upper, auto upper_cols, int kt, char* X, char* Y, frag_t (*bl)[TNH], frag_t (*bu)[TNH]) __attribute__((always_inline)) {
         constexpr bool UPPER = decltype(upper)::value;
+        constexpr bool UCOLS = decltype(upper_cols)::value;
         // The last two steps of a range have no tile left to request; they request the last tile once more, into
         // halves that nobody reads again, which keeps the count of outstanding copies the same in every step (a
         // branch around the copies, with its own wait, measured slower than the 2 / 64 of copy work it saves).
@@ -1063,16 +1067,16 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
         mma_quad(0, 0, fa, bl);
         __builtin_amdgcn_s_setprio(0);
         CK_PHASE_END();
-        read_b(X, 1, bu);
+        if (UCOLS) read_b(X, 1, bu);
         CK_M_END(0);
         __builtin_amdgcn_s_setprio(1);
-        mma_quad(0, 1, fa, bu);
+        if (UCOLS) mma_quad(0, 1, fa, bu);
         __builtin_amdgcn_s_setprio(0);
         CK_PHASE_END();
         if (UPPER) read_a(X, 1, fa);
         CK_M_END(3);
         __builtin_amdgcn_s_setprio(1);
-        if (UPPER) mma_quad(1, 1, fa, bu);
+        if (UPPER && UCOLS) mma_quad(1, 1, fa, bu);
         __builtin_amdgcn_s_setprio(0);
         CK_PHASE_END();
         // lower columns of the next tile, over the registers of this tile's upper columns (after the last tile of a
@@ -1105,17 +1109,16 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
         CK_PHASE_END();
         if (wm == 1) CK_PHASE_END();  // the upper group falls one phase behind
         // two steps per turn so that each names its buffers and registers statically
-        if (upper_rows_live) {
+        auto run = [&](auto upper, auto upper_cols) __attribute__((always_inline)) {
             for (; kt + 1 < n_full; kt += 2) {
-                pp_step(std::true_type{}, kt, lds0, lds1, fb0, fb1);
-                pp_step(std::true_type{}, kt + 1, lds1, lds0, fb1, fb0);
+                pp_step(upper, upper_cols, kt, lds0, lds1, fb0, fb1);
+                pp_step(upper, upper_cols, kt + 1, lds1, lds0, fb1, fb0);
             }
-        } else {
-            for (; kt + 1 < n_full; kt += 2) {
-                pp_step(std::false_type{}, kt, lds0, lds1, fb0, fb1);
-                pp_step(std::false_type{}, kt + 1, lds1, lds0, fb1, fb0);
-            }
-        }
+        };
+        if (upper_rows_live && upper_cols_live) run(std::true_type{}, std::true_type{});
+        else if (upper_cols_live) run(std::false_type{}, std::true_type{});
+        else if (upper_rows_live) run(std::true_type{}, std::false_type{});
+        else run(std::false_type{}, std::false_type{});
         if (wm == 0) CK_PHASE_END();
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
