@@ -140,7 +140,8 @@ def test_swiglu_unchunked(gpu, dtype, size):
 @pytest.mark.parametrize("has_weight", [True, False])
 @pytest.mark.parametrize("memory_efficient", [False, True])
 @pytest.mark.parametrize(
-    "size", [(1,), (13,), (2050,), (400, 1), (400, 8), (400, 257), (400, 1024), (37, 4096), (19, 5120), (7, 16384), (3, 65536), (5, 33000)]
+    "size", [(1,), (13,), (2050,), (400, 1), (400, 8), (400, 257), (300, 256), (400, 512), (400, 1024), (150, 2048), (37, 4096),
+             (19, 5120), (7, 16384), (3, 65536), (5, 33000)]
 )
 def test_rmsnorm(gpu, dtype, has_weight, memory_efficient, size):
     from cute_kernels import rmsnorm_cute
