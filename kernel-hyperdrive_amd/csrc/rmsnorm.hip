@@ -285,7 +285,10 @@ __global__ void __launch_bounds__(256)
 
 // Backward: one wave per SIMD with the whole register file (packed current row and next row of x and dy, packed
 // weight, 64 fp32 dweight accumulators); the next row's loads are in flight while the current row is reduced.
-template <typename T, int TPR, bool HAS_W, bool PREFETCH, int NP>
+// NEED_SS = false: 1 / rms is given, and the row's sum of squares - one multiply-add per element and a reduction over
+// the team - is not computed at all (5 us of 81 at 16384 x 4096).  NEED_SS = true forms it unless rstd_in is given
+// (the 1024-lane team is compiled this way only: without the sum its register allocation spills).
+template <typename T, int TPR, bool HAS_W, bool PREFETCH, int NP, bool NEED_SS>
 __device__ __forceinline__ void rmsnorm_bwd_body(const typename T::storage_t* __restrict__ x,
                                                  const typename T::storage_t* __restrict__ w,
                                                  const typename T::storage_t* __restrict__ dy,
@@ -338,7 +341,7 @@ __device__ __forceinline__ void rmsnorm_bwd_body(const typename T::storage_t* __
         // so a value requested behind them would not arrive before they all have - the wait for it would be a wait
         // for the whole row that is meant to stay in flight during this row's arithmetic
         float rstd_given = 0.f;
-        if (rstd_in != nullptr) rstd_given = rstd_in[row];
+        if (!NEED_SS || rstd_in != nullptr) rstd_given = rstd_in[row];
         if (PREFETCH) {
             const int64_t next_row = row + num_teams;
             if (next_row < B) {
@@ -380,7 +383,7 @@ __device__ __forceinline__ void rmsnorm_bwd_body(const typename T::storage_t* __
 #pragma unroll
                     for (int j = 0; j < T::kVec; ++j) {
                         const float xf = T::up(x8.v[j]);
-                        ss += xf * xf;
+                        if (NEED_SS) ss += xf * xf;
                         dot += T::up(g8.v[j]) * T::up(w8.v[j]) * xf;
                     }
                 }
@@ -396,7 +399,7 @@ __device__ __forceinline__ void rmsnorm_bwd_body(const typename T::storage_t* __
                         const float xf = T::up(xv[i].v[j]);
                         float g = T::up(gv[i].v[j]);
                         if (HAS_W) g *= T::up(wv[i].v[j]);
-                        ss += xf * xf;
+                        if (NEED_SS) ss += xf * xf;
                         dot += g * xf;
                     }
                 }
@@ -413,7 +416,7 @@ __device__ __forceinline__ void rmsnorm_bwd_body(const typename T::storage_t* __
             }
         }
         float rstd;
-        if (rstd_in != nullptr) {
+        if (!NEED_SS || rstd_in != nullptr) {
             rstd = rstd_given;
         } else {
             ss = team_sum<TPR>(ss, red);
@@ -503,24 +506,24 @@ __device__ __forceinline__ void rmsnorm_bwd_body(const typename T::storage_t* __
 // The next row of x and dy in flight while the current one is reduced: 288 registers with a weight at a row length
 // of 4096, i.e. one wave per SIMD and one workgroup per compute unit (the 1024-lane variant has 128 registers per
 // lane and no room for it).
-template <typename T, int TPR, bool HAS_W, int NP = 0>
+template <typename T, int TPR, bool HAS_W, int NP, bool NEED_SS>
 __global__ void __launch_bounds__(TPR > 256 ? TPR : 256)
     rmsnorm_bwd_kernel(const typename T::storage_t* __restrict__ x, const typename T::storage_t* __restrict__ w,
                        const typename T::storage_t* __restrict__ dy, const float* __restrict__ rstd_in,
                        typename T::storage_t* __restrict__ dx, float* __restrict__ dw_partial, int64_t B, int H,
                        float eps) {
-    rmsnorm_bwd_body<T, TPR, HAS_W, TPR <= 256, NP>(x, w, dy, rstd_in, dx, dw_partial, B, H, eps);
+    rmsnorm_bwd_body<T, TPR, HAS_W, TPR <= 256, NP, NEED_SS>(x, w, dy, rstd_in, dx, dw_partial, B, H, eps);
 }
 
 // One wave per row without the row in flight: fits two waves per SIMD, so two workgroups per compute unit walk the
 // rows and one wave's loads overlap the other's reductions and stores.
-template <typename T, bool HAS_W, int NP = 0>
+template <typename T, bool HAS_W, int NP, bool NEED_SS>
 __global__ void __launch_bounds__(256, 2)
     rmsnorm_bwd_two_kernel(const typename T::storage_t* __restrict__ x, const typename T::storage_t* __restrict__ w,
                            const typename T::storage_t* __restrict__ dy, const float* __restrict__ rstd_in,
                            typename T::storage_t* __restrict__ dx, float* __restrict__ dw_partial, int64_t B, int H,
                            float eps) {
-    rmsnorm_bwd_body<T, 64, HAS_W, false, NP>(x, w, dy, rstd_in, dx, dw_partial, B, H, eps);
+    rmsnorm_bwd_body<T, 64, HAS_W, false, NP, NEED_SS>(x, w, dy, rstd_in, dx, dw_partial, B, H, eps);
 }
 
 // dweight[j] = sum over `parts` partial rows of partial[r][j].  One wave per block owns 16 columns:
@@ -874,15 +877,28 @@ struct BwdArgs {
     float eps;
 };
 
+template <typename T, int TPR, int NP, bool W, bool SS>
+static void launch_bwd_one(unsigned grid, int block, hipStream_t s, const BwdArgs& a) {
+    typedef typename T::storage_t S;
+    hipLaunchKernelGGL((ck::rmsnorm_bwd_kernel<T, TPR, W, NP, SS>), dim3(grid), dim3(block), 0, s, (const S*)a.x,
+                       (const S*)a.weight, (const S*)a.dy, a.rstd, (S*)a.dx, a.ws, a.B, a.H, a.eps);
+}
 template <typename T, int TPR, int NP>
 static void launch_bwd_np(unsigned grid, int block, hipStream_t s, const BwdArgs& a) {
-    typedef typename T::storage_t S;
-    if (a.weight)
-        hipLaunchKernelGGL((ck::rmsnorm_bwd_kernel<T, TPR, true, NP>), dim3(grid), dim3(block), 0, s, (const S*)a.x,
-                           (const S*)a.weight, (const S*)a.dy, a.rstd, (S*)a.dx, a.ws, a.B, a.H, a.eps);
-    else
-        hipLaunchKernelGGL((ck::rmsnorm_bwd_kernel<T, TPR, false, NP>), dim3(grid), dim3(block), 0, s, (const S*)a.x,
-                           (const S*)a.weight, (const S*)a.dy, a.rstd, (S*)a.dx, a.ws, a.B, a.H, a.eps);
+    if constexpr (TPR == 1024) {
+        // (the form that never sums the squares spills at 128 registers per lane and is not compiled)
+        if (a.weight) launch_bwd_one<T, TPR, NP, true, true>(grid, block, s, a);
+        else launch_bwd_one<T, TPR, NP, false, true>(grid, block, s, a);
+    } else {
+        const bool ss = a.rstd == nullptr;  // 1 / rms was not saved: the kernel forms it
+        if (a.weight) {
+            if (ss) launch_bwd_one<T, TPR, NP, true, true>(grid, block, s, a);
+            else launch_bwd_one<T, TPR, NP, true, false>(grid, block, s, a);
+        } else {
+            if (ss) launch_bwd_one<T, TPR, NP, false, true>(grid, block, s, a);
+            else launch_bwd_one<T, TPR, NP, false, false>(grid, block, s, a);
+        }
+    }
 }
 template <typename T, int TPR>
 static void launch_bwd(unsigned grid, int block, hipStream_t s, const BwdArgs& a, int np) {
@@ -890,17 +906,26 @@ static void launch_bwd(unsigned grid, int block, hipStream_t s, const BwdArgs& a
     else if (np == 4) launch_bwd_np<T, TPR, 4>(grid, block, s, a);
     else launch_bwd_np<T, TPR, 0>(grid, block, s, a);
 }
+template <typename T, int NP, bool W, bool SS>
+static void launch_bwd_two_one(unsigned grid, hipStream_t s, const BwdArgs& a) {
+    typedef typename T::storage_t S;
+    hipLaunchKernelGGL((ck::rmsnorm_bwd_two_kernel<T, W, NP, SS>), dim3(grid), dim3(256), 0, s, (const S*)a.x,
+                       (const S*)a.weight, (const S*)a.dy, a.rstd, (S*)a.dx, a.ws, a.B, a.H, a.eps);
+}
 template <typename T, int NP>
 static void launch_bwd_two_np(unsigned grid, hipStream_t s, const BwdArgs& a) {
     typedef typename T::storage_t S;
+    const bool ss = a.rstd == nullptr;
     if (a.weight) {
         // (16-bit rows of a generic packet count with a weight never come here - see two_fits - and are not compiled)
-        if constexpr (NP != 0 || sizeof(S) == 4)
-            hipLaunchKernelGGL((ck::rmsnorm_bwd_two_kernel<T, true, NP>), dim3(grid), dim3(256), 0, s, (const S*)a.x,
-                               (const S*)a.weight, (const S*)a.dy, a.rstd, (S*)a.dx, a.ws, a.B, a.H, a.eps);
-    } else
-        hipLaunchKernelGGL((ck::rmsnorm_bwd_two_kernel<T, false, NP>), dim3(grid), dim3(256), 0, s, (const S*)a.x,
-                           (const S*)a.weight, (const S*)a.dy, a.rstd, (S*)a.dx, a.ws, a.B, a.H, a.eps);
+        if constexpr (NP != 0 || sizeof(S) == 4) {
+            if (ss) launch_bwd_two_one<T, NP, true, true>(grid, s, a);
+            else launch_bwd_two_one<T, NP, true, false>(grid, s, a);
+        }
+    } else {
+        if (ss) launch_bwd_two_one<T, NP, false, true>(grid, s, a);
+        else launch_bwd_two_one<T, NP, false, false>(grid, s, a);
+    }
 }
 
 extern "C" int ck_rmsnorm_backward(const void* x, const void* weight, const void* output_grad, const float* rstd,
@@ -911,8 +936,15 @@ extern "C" int ck_rmsnorm_backward(const void* x, const void* weight, const void
     hipStream_t s = (hipStream_t)stream;
     if (B == 0 || H == 0) {
         // an empty batch still defines dweight = 0
-        if (weight && weight_grad && H > 0)
-            if (hipMemsetAsync(weight_grad, 0, (size_t)H * ck_elem_size(dtype), s) != hipSuccess) return CK_ERR_LAUNCH;
+        if (weight && weight_grad && H > 0) {
+            // (a launch, not a memset: the call may be recorded into a graph)
+            CK_DISPATCH_DTYPE(dtype, {
+                typedef typename T::storage_t S;
+                hipLaunchKernelGGL((ck::rmsnorm_dw_reduce_generic_kernel<T>), dim3((unsigned)ck_ceil_div(H, 256)), dim3(256), 0,
+                                   s, (const float*)nullptr, (S*)weight_grad, 0, (int)H, (int)H);
+            });
+            return ck_launch_status();
+        }
         return CK_OK;
     }
     if (!x || !output_grad || !x_grad) return CK_ERR_NULL;
