@@ -10,7 +10,8 @@
 //                  and records, for every sorted slot, the first slot of its run of equal ids.
 //               2. rows kernel, one launch for two jobs: rows no id selects are written as zeros (the
 //                  bulk of the traffic; a part of them rides, as extra workgroups, on the small launches
-//                  of step 1 that come after the rows are marked); a run of equal ids is cut into chunks of
+//                  of step 1 - whole ranges of rows on the two launches before the marks exist, the unmarked
+//                  rows of a range on the later ones); a run of equal ids is cut into chunks of
 //                  kChunk slots.  A chunk of one row is copied by one wave; the others are summed by the four
 //                  waves of a workgroup, a quarter of the columns each, in fp32 registers and in ascending
 //                  token position.  A run that fits one chunk is rounded and stored straight into dW; longer
@@ -144,7 +145,8 @@ struct PairStorer {
 // (`first_block` on), so the sort no longer costs time of its own.  One wave takes four consecutive rows: the four
 // marks first, then 16-byte packets of zeros (zero bits are zero in every storage type).
 struct FillJob {
-    const uint8_t* touched;
+    const uint8_t* touched;       // null: the marks are not known yet, every row of the share is cleared (the row sums,
+                                  // which run later, overwrite the selected ones among them)
     char* dw;
     int64_t row_bytes;            // a multiple of 16
     int64_t row_begin, row_end;   // this launch's share of the rows
@@ -161,7 +163,8 @@ __device__ __forceinline__ bool run_fill_job(const FillJob& f) {
         f.row_begin + (((int64_t)blockIdx.x - f.first_block) * waves + threadIdx.x / CK_WAVE) * kFillRowsPerWave;
     uint8_t mark[kFillRowsPerWave];
 #pragma unroll
-    for (int r = 0; r < kFillRowsPerWave; ++r) mark[r] = row0 + r < f.row_end ? f.touched[row0 + r] : 1;
+    for (int r = 0; r < kFillRowsPerWave; ++r)
+        mark[r] = row0 + r < f.row_end ? (f.touched != nullptr ? f.touched[row0 + r] : 0) : 1;
     const zero_t z = {0u, 0u, 0u, 0u};
     const int64_t packs = f.row_bytes / 16;
 #pragma unroll
@@ -185,8 +188,8 @@ __global__ void __launch_bounds__(256)
     __shared__ GridSortShared sh;
     if (run_fill_job(fill)) return;
     // side job of the first pass: clear the row marks
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < clear_words; i += (int64_t)gridDim.x * blockDim.x)
-        clear[i] = 0u;
+    const int64_t own = min((int64_t)gridDim.x, (int64_t)fill.first_block);  // the workgroups that are not the fill's
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < clear_words; i += own * blockDim.x) clear[i] = 0u;
     grid_sort_histogram(sh, n, shift, bits, hist, num_waves, load);
 }
 
@@ -201,15 +204,16 @@ __global__ void __launch_bounds__(1024)
         grid_sort_scan(hist, total);
         return;
     }
+    if (run_fill_job(fill)) return;
     if (MARK) {
-        const int64_t stride = (int64_t)(gridDim.x - 1) * blockDim.x;
+        // workgroups 1 .. fill.first_block - 1 (all the others, where the launch carries no fill)
+        const int64_t markers = min((int64_t)gridDim.x, (int64_t)fill.first_block) - 1;
+        const int64_t stride = markers * blockDim.x;
         for (int64_t i = (int64_t)(blockIdx.x - 1) * blockDim.x + threadIdx.x; i < n; i += stride) {
             uint32_t key, val;
             load((int)i, key, val);
             if ((int64_t)key < V) touched[key] = 1;
         }
-    } else {
-        run_fill_job(fill);
     }
 }
 
@@ -547,8 +551,9 @@ extern "C" int64_t ck_embedding_backward_workspace_size(int64_t num_ids, int64_t
     return ck::emb_carve(nullptr, num_ids, V, H, nullptr);
 }
 
-// (measured at a table of [128256, 4096] and 32768 ids: 313 us without, 306 / 297 / 292 / 306 us with 20 / 40 / 80 / 160 MB)
-constexpr int64_t kCarrierFillBytes = (int64_t)80 << 20;
+// (measured at a table of [128256, 4096] and 32768 ids, seven carrying launches: 290 / 285 / 285 / 288 / 292 us with
+// 60 / 80 / 100 / 120 / 150 MB each; Zipf(1.1) ids 352 / 343 / 339 / 338 / 339 us)
+constexpr int64_t kCarrierFillBytes = (int64_t)100 << 20;
 
 template <typename T, int VEC>
 static void launch_bwd(hipStream_t s, const ck::EmbWorkspace& ws, int passes, const void* dy, void* dw, int n,
@@ -589,19 +594,20 @@ extern "C" int ck_embedding_backward(const void* ids, int ids_are_i32, const voi
     const int num_waves = ck::grid_sort_waves(n);
     const unsigned sort_grid = (unsigned)(num_waves > 0 ? ck_ceil_div(num_waves, ck::kGridSortBlockWaves) : 1);
     const int64_t clear_words = (V + 3) / 4;
-    // The zero fill of the rows nobody selects rides on the launches between the marking of the rows (second launch)
-    // and the row sums: the first pass's scatter, the three launches of every further pass, the run heads.  Needs rows
-    // of whole 16-byte packets; otherwise (and without ids) the rows kernel fills, as it sums.
+    // The zero fill of the rows nobody selects rides on the launches before the row sums: the three launches of every
+    // pass and the run heads.  The first two launches run before the marks exist (the second one sets them): their
+    // shares are cleared whole, and the row sums overwrite the selected rows among them later.  Needs rows of whole
+    // 16-byte packets; otherwise (and without ids) the rows kernel fills, as it sums.
     const int64_t row_bytes = H * ck_elem_size(dtype);
     const bool spread_fill = n > 0 && row_bytes % 16 == 0 && ck_aligned16(weight_grad);
-    const int carriers = 1 + 3 * (passes - 1) + 1;
+    const int carriers = 3 * passes + 1;
     // a carrier's own work leaves most of the GPU idle for about 8 us: that much fill is free, more only moves time
     // from the row-sum launch, where the fill hides the latency of the sums, to here
     int64_t spread_rows = spread_fill ? carriers * (kCarrierFillBytes / row_bytes) : 0;
     if (spread_rows > V) spread_rows = V;
     int carrier = 0;
-    auto fill_share = [&](int own_blocks, int threads, unsigned& grid) {
-        ck::FillJob f = {ws.touched, (char*)weight_grad, row_bytes, 0, 0, 0x7fffffff};
+    auto fill_share = [&](int own_blocks, int threads, unsigned& grid, bool marks_known = true) {
+        ck::FillJob f = {marks_known ? ws.touched : nullptr, (char*)weight_grad, row_bytes, 0, 0, 0x7fffffff};
         grid = (unsigned)own_blocks;
         if (spread_fill) {
             f.row_begin = spread_rows * carrier / carriers;
@@ -612,7 +618,6 @@ extern "C" int ck_embedding_backward(const void* ids, int ids_are_i32, const voi
         }
         return f;
     };
-    const ck::FillJob no_fill = {ws.touched, (char*)weight_grad, row_bytes, 0, 0, 0x7fffffff};
     // workgroups of the second launch that mark the selected rows (behind the one that scans)
     const unsigned mark_blocks = (unsigned)(n > 0 ? ck_ceil_div(n, 4 * 1024) : 0);
     for (int p = 0; p < passes; ++p) {
@@ -625,20 +630,24 @@ extern "C" int ck_embedding_backward(const void* ids, int ids_are_i32, const voi
             // the clear of the row marks rides on the first histogram launch (needs at least one workgroup)
             if (ids_are_i32) {
                 ck::IdLoader<true> load = {ids, V};
-                hipLaunchKernelGGL((ck::embedding_sort_hist_kernel<ck::IdLoader<true>>), dim3(sort_grid), dim3(256), 0, s,
-                                   load, n, shift, bits, ws.hist, num_waves, (uint32_t*)ws.touched, clear_words, no_fill);
-                hipLaunchKernelGGL((ck::embedding_sort_scan_kernel<ck::IdLoader<true>, true>), dim3(1 + mark_blocks),
-                                   dim3(1024), 0, s, ws.hist, total, load, n, V, ws.touched, no_fill);
-                const ck::FillJob f = fill_share((int)sort_grid, 256, grid);
+                ck::FillJob f = fill_share((int)sort_grid, 256, grid, false);
+                hipLaunchKernelGGL((ck::embedding_sort_hist_kernel<ck::IdLoader<true>>), dim3(grid), dim3(256), 0, s,
+                                   load, n, shift, bits, ws.hist, num_waves, (uint32_t*)ws.touched, clear_words, f);
+                f = fill_share(1 + (int)mark_blocks, 1024, grid, false);
+                hipLaunchKernelGGL((ck::embedding_sort_scan_kernel<ck::IdLoader<true>, true>), dim3(grid), dim3(1024), 0, s,
+                                   ws.hist, total, load, n, V, ws.touched, f);
+                f = fill_share((int)sort_grid, 256, grid);
                 hipLaunchKernelGGL((ck::embedding_sort_scatter_kernel<ck::IdLoader<true>>), dim3(grid), dim3(256), 0, s,
                                    load, store, n, shift, bits, ws.hist, num_waves, f);
             } else {
                 ck::IdLoader<false> load = {ids, V};
-                hipLaunchKernelGGL((ck::embedding_sort_hist_kernel<ck::IdLoader<false>>), dim3(sort_grid), dim3(256), 0, s,
-                                   load, n, shift, bits, ws.hist, num_waves, (uint32_t*)ws.touched, clear_words, no_fill);
-                hipLaunchKernelGGL((ck::embedding_sort_scan_kernel<ck::IdLoader<false>, true>), dim3(1 + mark_blocks),
-                                   dim3(1024), 0, s, ws.hist, total, load, n, V, ws.touched, no_fill);
-                const ck::FillJob f = fill_share((int)sort_grid, 256, grid);
+                ck::FillJob f = fill_share((int)sort_grid, 256, grid, false);
+                hipLaunchKernelGGL((ck::embedding_sort_hist_kernel<ck::IdLoader<false>>), dim3(grid), dim3(256), 0, s,
+                                   load, n, shift, bits, ws.hist, num_waves, (uint32_t*)ws.touched, clear_words, f);
+                f = fill_share(1 + (int)mark_blocks, 1024, grid, false);
+                hipLaunchKernelGGL((ck::embedding_sort_scan_kernel<ck::IdLoader<false>, true>), dim3(grid), dim3(1024), 0, s,
+                                   ws.hist, total, load, n, V, ws.touched, f);
+                f = fill_share((int)sort_grid, 256, grid);
                 hipLaunchKernelGGL((ck::embedding_sort_scatter_kernel<ck::IdLoader<false>>), dim3(grid), dim3(256), 0, s,
                                    load, store, n, shift, bits, ws.hist, num_waves, f);
             }
