@@ -60,6 +60,8 @@ def parse_args():
     p.add_argument("--only-extras", action="store_true", help="only the HBM-bound ops (for profiling them)")
     p.add_argument("--embedding-ids", choices=["both", "uniform", "zipf"], default="both",
                    help="with --only-extras: one id distribution only (counter profiles sum over a kernel's dispatches)")
+    p.add_argument("--only-yardstick", action="store_true",
+                   help="only the vendor library's dense bf16 products (extras.dense_bmm_yardstick), for a kernel trace")
     p.add_argument("--tokens", type=int, default=8192, help="T of the MoE workload (default: the BASELINE shape)")
     p.add_argument("--copy-calibration", action="store_true",
                    help="also run three 1 GiB device copies before the steps (a kernel of known HBM traffic, to scale "
@@ -301,7 +303,55 @@ def bench_extras(device, embedding_ids="both"):
     if embedding_ids == "both":
         out["moe_fine_grained_skewed"] = bench_moe_skewed(device)
         torch.cuda.empty_cache()
+        out["dense_bmm_yardstick"] = bench_dense_yardstick(device)
+        torch.cuda.empty_cache()
     return out
+
+
+# ---- dense yardstick --------------------------------------------------------------------------------------
+def bench_dense_yardstick(device, iters=5, warmup=2):
+    """What the vendor library's dense bf16 kernels reach on this box, under the same power cap, on the six products
+    of the Mixtral step taken as batched dense GEMMs of E = 8 experts x 2048 rows (perfectly balanced routing, no
+    gather, no scatter, no activation): torch.bmm on random N(0,1) / N(0,0.02) data in the operand layouts the layer
+    has (weights [E, out, in]).  A stated yardstick, never the target and never part of `value`."""
+    E, R, H, I = 8, 2048, 4096, 14336
+    dtype = torch.bfloat16
+    g = torch.Generator(device=device).manual_seed(1)
+
+    def rnd(*shape, std=1.0):
+        return torch.randn(*shape, generator=g, device=device, dtype=torch.float32).mul_(std).to(dtype)
+
+    x, dy = rnd(E, R, H), rnd(E, R, H)
+    h, dh = rnd(E, R, 2 * I), rnd(E, R, 2 * I)
+    act, dact = rnd(E, R, I), rnd(E, R, I)
+    w_fc, w_proj = rnd(E, 2 * I, H, std=0.02), rnd(E, H, I, std=0.02)
+    products = {
+        "fwd_c_fc": (lambda: torch.bmm(x, w_fc.transpose(1, 2)), 2.0 * E * R * H * 2 * I),
+        "fwd_c_proj": (lambda: torch.bmm(act, w_proj.transpose(1, 2)), 2.0 * E * R * I * H),
+        "dx_c_proj": (lambda: torch.bmm(dy, w_proj), 2.0 * E * R * H * I),
+        "dx_c_fc": (lambda: torch.bmm(dh, w_fc), 2.0 * E * R * 2 * I * H),
+        "dw_c_fc": (lambda: torch.bmm(dh.transpose(1, 2), x), 2.0 * E * R * 2 * I * H),
+        "dw_c_proj": (lambda: torch.bmm(dy.transpose(1, 2), dact), 2.0 * E * R * H * I),
+    }
+    out, total_ms, total_flop = {}, 0.0, 0.0
+    for name, (fn, flop) in products.items():
+        for _ in range(warmup):
+            fn()
+        marks = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+        for start, end in marks:
+            start.record()
+            fn()
+            end.record()
+        torch.cuda.synchronize()
+        ms = sorted(s_.elapsed_time(e_) for s_, e_ in marks)[iters // 2]
+        out[name] = round(flop / (ms * 1e-3) / 1e12, 1)
+        total_ms += ms
+        total_flop += flop
+    tflops = total_flop / (total_ms * 1e-3) / 1e12
+    return {"TFLOP/s": round(tflops, 1), "frac_of_mfma_peak": round(tflops / BF16_MFMA_PEAK_TFLOPS, 4), "ms": round(total_ms, 3),
+            "per_product_tflops": out,
+            "what": "torch.bmm (vendor library) on the six products as dense batches of 8 x 2048 rows, same data "
+                    "distribution, same box and power cap; a yardstick, not the target"}
 
 
 # ---- CPU baseline -----------------------------------------------------------------------------------------
@@ -376,6 +426,11 @@ def main():
     if args.only_extras:
         print(json.dumps({"extras": bench_extras(device, args.embedding_ids)}))
         return
+    if args.only_yardstick:
+        print(json.dumps({"extras": {"dense_bmm_yardstick": bench_dense_yardstick(device)}}))
+        return
+    # The host baseline runs first: the GPU legs then end the run, where a utilisation sampler from outside sees them.
+    cpu = None if args.no_cpu else bench_cpu()
     result, roofline, config = bench_moe(device, args)
     line = {
         "metric": "scattermoe_fwd_bwd_tflops",
@@ -396,8 +451,8 @@ def main():
     }
     if not args.no_extras:
         line["extras"] = bench_extras(device)
-    if not args.no_cpu:
-        line["cpu_baseline"] = bench_cpu()
+    if cpu is not None:
+        line["cpu_baseline"] = cpu
     print(json.dumps(line))
 
 

@@ -150,7 +150,8 @@ int ck_moe_sort(const void* expert_ids, int ids_are_i32, int64_t* sorted_expert_
  * allocator.  Same arguments and results as ck_moe_sort, minus the workspace: that lives in a device array of
  * CK_MOE_SORT_NOALLOC_SCRATCH_BYTES inside the library, one copy per GPU, held until the process ends.  The call
  * makes no hipMalloc / hipFree and no allocating library call; the first call on a device looks the array's
- * address up once.  (M, E) whose ck_moe_sort_workspace_size exceeds the array gives CK_ERR_SCRATCH and launches
+ * address up once (hipGetSymbolAddress, which may load the code object and the 4 MiB array): make that first call
+ * per device outside any stream capture, every later one may be captured.  (M, E) whose ck_moe_sort_workspace_size exceeds the array gives CK_ERR_SCRATCH and launches
  * nothing (the limit is far away: 98304 ids of 64 experts need 48 KiB, a million ids of 512 experts 4 MiB).
  * All calls on one GPU share the array: calls that overlap there (different streams or threads) race; calls
  * ordered on one stream do not.  Nothing in the array has to be cleared between calls. */

@@ -343,8 +343,11 @@ def swiglu_unchunked_backward(x, output_grad, x_grad, block_size: int) -> None:
 
 
 def _row_operands(what: str, x, B: int, H: int, weight, rstd, **same_shape) -> None:
-    """Dense [B, H] tensors of x's type, a dense weight of H elements, fp32 1/rms of B elements (each may be None)."""
+    """Dense [B, H] tensors of x's type, a dense weight of H elements, fp32 1/rms of B elements (each may be None).
+    Row kernels reduce along the last dimension as it lies in memory, so "dense in some order of the dimensions" is
+    not enough here: a transposed tensor would be normalised along the wrong axis."""
     _dense_like(x, what, **same_shape)
+    _dense(what, x=x, **same_shape)
     if weight is not None and (weight.numel() != H or not weight.is_contiguous()):
         raise ValueError(f"{what}: the weight must be a dense vector of {H} elements")
     if rstd is not None and (rstd.dtype != torch.float32 or rstd.numel() != B or not rstd.is_contiguous()):

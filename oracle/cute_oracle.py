@@ -41,6 +41,9 @@ with and without biases as well):
                       place of the Triton histogram; checked against an independent per-token dense
                       formulation (y_t = sum_j softmax_j * FFN_{e_j}(x_t)) and its autograd in fp64, with and
                       without the per-expert biases
+  _linear             the layer's F.linear calls; fp16 operands go through fp32 products rounded once
+                      (_LinearRoundedOnce), checked against stock torch's native fp16 F.linear and its autograd
+                      and against float64 products rounded once
 No function here is "parity unpinned".
 
 Precision policy: inputs are values of the storage dtype (bf16 / fp16 / fp32).  ``compute_dtype=float32``
@@ -343,8 +346,41 @@ def swiglu_unchunked_activation(x: torch.Tensor) -> torch.Tensor:
     return (up.to(acc) * F.silu(gate.to(acc))).to(x.dtype)
 
 
+class _LinearRoundedOnce(torch.autograd.Function):
+    """``F.linear`` on fp16 tensors the way every 16-bit op of the reference's torch layer behaves - products summed
+    in fp32, the output rounded to the storage type once - with the same rule for the three gradients autograd derives
+    for it (d_rows = g W, d_W = g^T rows, d_b = column sums of g).  Stock torch on the CPU gives these values too, but
+    its native fp16 matrix products take minutes at the larger test shapes; this runs them as fp32 products.
+    (cute_kernels/kernels/scattermoe/torch_implementation.py:35-43, 122)"""
+
+    @staticmethod
+    def forward(ctx, rows, weight, bias):
+        ctx.save_for_backward(rows, weight)
+        ctx.has_bias = bias is not None
+        out = rows.float() @ weight.float().t()
+        if bias is not None:
+            out = out + bias.float()
+        return out.to(rows.dtype)
+
+    @staticmethod
+    def backward(ctx, g):
+        rows, weight = ctx.saved_tensors
+        g32 = g.float()
+        d_rows = (g32 @ weight.float()).to(rows.dtype)
+        d_weight = (g32.t() @ rows.float()).to(weight.dtype)
+        d_bias = g32.sum(0).to(g.dtype) if ctx.has_bias else None
+        return d_rows, d_weight, d_bias
+
+
+def _linear(rows, weight, bias=None):
+    """``F.linear``; for fp16 operands the same values through fp32 products (see ``_LinearRoundedOnce``)."""
+    if rows.dtype == torch.float16:
+        return _LinearRoundedOnce.apply(rows, weight, bias)
+    return F.linear(rows, weight, bias)
+
+
 def moe_forward(x, w_gate, w_fc, w_proj, top_k: int, activation=swiglu_unchunked_activation, selected=None,
-                b_fc=None, b_proj=None):
+                b_fc=None, b_proj=None, mix="index_add"):
     """Forward of MoE_Torch on tensors of one dtype; returns (y [T, H], router_logits [T, E]).
 
     x [T, H]; w_gate [E, H]; w_fc [E, F, H] (F = 2I for a GLU activation); w_proj [E, H, I]; optional per-expert
@@ -352,10 +388,19 @@ def moe_forward(x, w_gate, w_fc, w_proj, top_k: int, activation=swiglu_unchunked
     ``selected`` ([T, k] expert ids) replaces the top-k decision: logits rounded to 16 bits tie often, and
     two correct implementations may break a tie differently, so a test passes the decision of the run under
     test.  The values at the selected positions still come from this function's own logits.
+    ``mix`` names how a token's k expert outputs become its output, the one place where the reference's two layers
+    round differently in 16 bits (in exact arithmetic both are the same sum):
+      "index_add"  MoE_Torch: every expert row times its routing weight, rounded, then added per token (:161-163);
+                   the input rows are gathered by indexing, so autograd adds a token's k gradient rows one by one
+      "bmm"        the Triton layer: ``torch.bmm(gates, expanded)`` over the k unscaled rows of a token, fp32 sums
+                   rounded once (triton_implementation/ops.py:160-164); its backward scales the output gradient by
+                   the routing weight with one rounding (ops.py:204-221, kernels.py:284-286) and sums a token's k
+                   input-gradient rows with ``.sum(-2)`` (ops.py:258-261) - what autograd derives for the
+                   expressions below
     """
     T, H = x.shape
     E = w_gate.size(0)
-    router_logits = F.linear(x, w_gate)                                       # :122
+    router_logits = _linear(x, w_gate)                                        # :122
     if selected is not None:
         top_vals = router_logits.gather(1, selected)
     elif top_k == 1:                                                          # :193-199
@@ -370,22 +415,33 @@ def moe_forward(x, w_gate, w_fc, w_proj, top_k: int, activation=swiglu_unchunked
     fan_in_index = order // top_k
     batch_gates = router_weights.flatten()[order]
 
-    grouped = x[fan_in_index]                                                 # :150
+    if mix == "bmm":
+        grouped = x.unsqueeze(1).expand(T, top_k, H).reshape(T * top_k, H)[order]
+    else:
+        grouped = x[fan_in_index]                                             # :150
     splits = expert_frequency.tolist()
     outs = []
     for e, rows in enumerate(grouped.split(splits, dim=0)):                   # :36-43, 154-158
-        h = F.linear(rows, w_fc[e], None if b_fc is None else b_fc[e])
+        h = _linear(rows, w_fc[e], None if b_fc is None else b_fc[e])
         h = activation(h)
-        outs.append(F.linear(h, w_proj[e], None if b_proj is None else b_proj[e]))
+        outs.append(_linear(h, w_proj[e], None if b_proj is None else b_proj[e]))
+    acc = _acc_dtype(x)
+    if mix == "bmm":
+        inverse = torch.empty_like(order)
+        inverse[order] = torch.arange(order.numel())
+        expanded = torch.cat(outs)[inverse].view(T, top_k, H)                 # back in (token, slot) order
+        y = (router_weights.to(acc).unsqueeze(-1) * expanded.to(acc)).sum(1).to(x.dtype)
+        return y, router_logits
+    assert mix == "index_add"
     grouped = torch.cat(outs) * batch_gates.unsqueeze(-1)                     # :161
     # :162-163; the accumulation is done in fp32 and rounded once
-    acc = _acc_dtype(x)
     y = torch.zeros(T, H, dtype=acc).index_add(0, fan_in_index, grouped.to(acc)).to(x.dtype)
     return y, router_logits
 
 
 def moe_forward_backward(x, w_gate, w_fc, w_proj, dy, top_k: int, compute_dtype=torch.float32,
-                         activation=swiglu_unchunked_activation, selected=None, b_fc=None, b_proj=None) -> dict:
+                         activation=swiglu_unchunked_activation, selected=None, b_fc=None, b_proj=None,
+                         mix="index_add") -> dict:
     """Forward and all gradients for loss = sum(y * dy), torch ops run in ``compute_dtype``.
 
     Results are returned in the dtype of ``x``; with biases given, their gradients are ``db_fc`` / ``db_proj``.
@@ -393,7 +449,7 @@ def moe_forward_backward(x, w_gate, w_fc, w_proj, dy, top_k: int, compute_dtype=
     leaves = [t.detach().to(compute_dtype).clone().requires_grad_(True) for t in (x, w_gate, w_fc, w_proj)]
     biases = [None if b is None else b.detach().to(compute_dtype).clone().requires_grad_(True) for b in (b_fc, b_proj)]
     y, router_logits = moe_forward(*leaves, top_k=top_k, activation=activation, selected=selected,
-                                   b_fc=biases[0], b_proj=biases[1])
+                                   b_fc=biases[0], b_proj=biases[1], mix=mix)
     (y * dy.to(compute_dtype)).sum().backward()
     out_dtype = x.dtype
     bias_grads = {name: b.grad.to(out_dtype) for name, b in zip(("db_fc", "db_proj"), biases) if b is not None}
@@ -420,7 +476,7 @@ def moe_expert_forward_backward(rows, gates, w_fc_e, w_proj_e, dy_rows, compute_
     rows_ = rows.detach().to(compute_dtype).clone().requires_grad_(True)
     w_fc_ = w_fc_e.detach().to(compute_dtype).clone().requires_grad_(True)
     w_proj_ = w_proj_e.detach().to(compute_dtype).clone().requires_grad_(True)
-    out = F.linear(activation(F.linear(rows_, w_fc_)), w_proj_) * gates.to(compute_dtype).unsqueeze(-1)
+    out = _linear(activation(_linear(rows_, w_fc_)), w_proj_) * gates.to(compute_dtype).unsqueeze(-1)
     (out * dy_rows.to(compute_dtype)).sum().backward()
     dtype = rows.dtype
     return {"out": out.detach().to(dtype), "d_rows": rows_.grad.to(dtype), "dw_fc": w_fc_.grad.to(dtype),

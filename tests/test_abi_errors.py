@@ -269,6 +269,12 @@ def test_binding_checks_index_and_operand_types_before_any_launch():
         _C.swiglu_forward(a, a.t(), torch.empty_like(a), 256)
     with pytest.raises(ValueError, match="up is torch.float32"):
         _C.swiglu_forward(a, a.float(), torch.empty_like(a), 256)
+    # row kernels: dense in another order of the dimensions is not enough (rows must be the contiguous dimension)
+    xt = torch.zeros(8, 4, dtype=torch.bfloat16).t()
+    with pytest.raises(ValueError, match="must be contiguous"):
+        _C.rmsnorm_forward(xt, None, torch.empty_like(xt), None, 1e-5)
+    with pytest.raises(ValueError, match="must be contiguous"):
+        _C.rmsnorm_backward(xt, None, torch.empty_like(xt), None, torch.empty_like(xt), None, None, 1e-5)
     with pytest.raises(ValueError, match="output has 16 elements"):
         _C.add_tensor_forward(a, a, torch.zeros(4, 4, dtype=torch.bfloat16), 256)
     with pytest.raises(ValueError, match="holds half"):

@@ -455,6 +455,64 @@ def test_moe_one_expert_slices_against_the_layer_and_a_hand_written_sum():
     assert torch.allclose(dx1, res1["dx"], rtol=1e-10, atol=1e-12)
 
 
+@pytest.mark.parametrize("top_k", [1, 2, 4])
+def test_moe_mixing_forms_are_one_sum(top_k):
+    """``mix="bmm"`` (the Triton layer's order of roundings) and ``mix="index_add"`` (MoE_Torch's) are the same
+    mathematics: in float64 every output and gradient agrees to rounding noise, and in bf16 they differ by no more
+    than the roundings they place differently (and do differ somewhere once k > 1: the switch is not a no-op)."""
+    T, H, I, E = 96, 32, 24, 5
+    x, w_gate, w_fc, w_proj, dy = O.moe_inputs(T, H, I, E, torch.float32, seed=5)
+    a = O.moe_forward_backward(x.double(), w_gate.double(), w_fc.double(), w_proj.double(), dy.double(), top_k, compute_dtype=F64)
+    b = O.moe_forward_backward(x.double(), w_gate.double(), w_fc.double(), w_proj.double(), dy.double(), top_k, compute_dtype=F64, mix="bmm")
+    for key in ("y", "router_logits", "dx", "dw_gate", "dw_fc", "dw_proj"):
+        assert torch.allclose(a[key], b[key], rtol=1e-11, atol=1e-12), key
+    xb, wgb, wfb, wpb, dyb = (t.bfloat16() for t in (x, w_gate, w_fc * 10, w_proj * 10, dy))
+    sel = a["router_logits"].topk(top_k, dim=-1).indices if top_k > 1 else a["router_logits"].max(-1, keepdim=True).indices
+    c = O.moe_forward_backward(xb, wgb, wfb, wpb, dyb, top_k, compute_dtype=torch.bfloat16, selected=sel)
+    d = O.moe_forward_backward(xb, wgb, wfb, wpb, dyb, top_k, compute_dtype=torch.bfloat16, selected=sel, mix="bmm")
+    for key in ("y", "dx", "dw_fc", "dw_proj"):
+        assert O.fraction_outside(d[key], c[key], **O.tolerance(torch.bfloat16)) < 0.02, key
+    if top_k > 1:
+        assert not torch.equal(c["y"], d["y"])
+
+
+def test_fp16_linear_rounded_once_against_native_fp16_and_fp64():
+    """The oracle's fp16 linear (fp32 products, one rounding) against (a) stock torch's native fp16 F.linear and its
+    autograd gradients and (b) products formed in float64 and rounded once.  A transposed operand, a missing bias or
+    a gradient that skips its rounding fails either."""
+    g = torch.Generator().manual_seed(71)
+    rows = torch.randn(37, 96, generator=g).half()
+    weight = (torch.randn(24, 96, generator=g) * 0.2).half()
+    bias = torch.randn(24, generator=g).half()
+    dy = torch.randn(37, 24, generator=g).half()
+    for b in (None, bias):
+        mine = [t.clone().requires_grad_(True) for t in (rows, weight)] + ([b.clone().requires_grad_(True)] if b is not None else [None])
+        theirs = [t.clone().requires_grad_(True) for t in (rows, weight)] + ([b.clone().requires_grad_(True)] if b is not None else [None])
+        out_m = O._linear(*mine)
+        out_t = F.linear(*theirs)
+        out_m.backward(dy)
+        out_t.backward(dy)
+        exact = rows.double() @ weight.double().t() + (0 if b is None else b.double())
+        pairs = [(out_m, out_t, exact), (mine[0].grad, theirs[0].grad, dy.double() @ weight.double()),
+                 (mine[1].grad, theirs[1].grad, dy.double().t() @ rows.double())]
+        if b is not None:
+            pairs.append((mine[2].grad, theirs[2].grad, dy.double().sum(0)))
+        for got, native, exact64 in pairs:
+            assert got.dtype == torch.float16 and got.shape == native.shape
+            # one rounding of an fp32 sum: at most one unit in the last place from the rounded exact value, and equal
+            # to it nearly everywhere (an fp32 sum of < 100 terms is off by far less than half an fp16 step)
+            rounded = exact64.half()
+            ulp = torch.maximum(rounded.float().abs() * 2.0 ** -10, torch.tensor(2.0 ** -24))
+            assert ((got.float() - rounded.float()).abs() <= ulp).all()
+            assert (got == rounded).float().mean().item() > 0.99
+            assert ((got.float() - native.float()).abs() <= ulp).all()
+            assert (got == native).float().mean().item() > 0.99
+    # bf16 and fp32 operands take stock F.linear unchanged
+    for dtype in (torch.bfloat16, torch.float32):
+        assert torch.equal(O._linear(rows.to(dtype), weight.to(dtype), bias.to(dtype)),
+                           F.linear(rows.to(dtype), weight.to(dtype), bias.to(dtype)))
+
+
 def test_moe_single_expert_is_a_plain_mlp():
     T, H, I = 7, 8, 5
     x, wg, wfc, wproj, dy = (t.double() for t in O.moe_inputs(T, H, I, 1, torch.float32, seed=4))
