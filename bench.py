@@ -60,8 +60,9 @@ def parse_args():
     p.add_argument("--only-extras", action="store_true", help="only the HBM-bound ops (for profiling them)")
     p.add_argument("--embedding-ids", choices=["both", "uniform", "zipf"], default="both",
                    help="with --only-extras: one id distribution only (counter profiles sum over a kernel's dispatches)")
-    p.add_argument("--only-yardstick", action="store_true",
-                   help="only the vendor library's dense bf16 products (extras.dense_bmm_yardstick), for a kernel trace")
+    p.add_argument("--yardstick", action="store_true",
+                   help="also time the vendor library's dense bf16 kernels on the six products (extras.dense_yardstick)")
+    p.add_argument("--only-yardstick", action="store_true", help="only that leg (for a kernel trace)")
     p.add_argument("--tokens", type=int, default=8192, help="T of the MoE workload (default: the BASELINE shape)")
     p.add_argument("--copy-calibration", action="store_true",
                    help="also run three 1 GiB device copies before the steps (a kernel of known HBM traffic, to scale "
@@ -303,17 +304,20 @@ def bench_extras(device, embedding_ids="both"):
     if embedding_ids == "both":
         out["moe_fine_grained_skewed"] = bench_moe_skewed(device)
         torch.cuda.empty_cache()
-        out["dense_bmm_yardstick"] = bench_dense_yardstick(device)
-        torch.cuda.empty_cache()
     return out
 
 
 # ---- dense yardstick --------------------------------------------------------------------------------------
 def bench_dense_yardstick(device, iters=5, warmup=2):
     """What the vendor library's dense bf16 kernels reach on this box, under the same power cap, on the six products
-    of the Mixtral step taken as batched dense GEMMs of E = 8 experts x 2048 rows (perfectly balanced routing, no
-    gather, no scatter, no activation): torch.bmm on random N(0,1) / N(0,0.02) data in the operand layouts the layer
-    has (weights [E, out, in]).  A stated yardstick, never the target and never part of `value`."""
+    of the Mixtral step: per expert (E = 8, 2048 rows each, i.e. perfectly balanced routing; no gather, no scatter, no
+    activation) the 2-D calls the reference's plain-torch layer and its autograd make - ``F.linear(rows, W[e])``,
+    ``grad.mm(W[e])`` and ``grad.t().mm(rows)`` (cute_kernels/kernels/scattermoe/torch_implementation.py:36-43) - on
+    random N(0,1) / N(0,0.02) data.  A stated yardstick, never the target and never part of `value`.  Only with
+    --yardstick: `torch.bmm` on the same products as batches of 8 ended two GPU boxes with an illegal memory access
+    inside the library's kernel, so the batched form is not used and the default run does not depend on this leg."""
+    import torch.nn.functional as F
+
     E, R, H, I = 8, 2048, 4096, 14336
     dtype = torch.bfloat16
     g = torch.Generator(device=device).manual_seed(1)
@@ -322,25 +326,29 @@ def bench_dense_yardstick(device, iters=5, warmup=2):
         return torch.randn(*shape, generator=g, device=device, dtype=torch.float32).mul_(std).to(dtype)
 
     x, dy = rnd(E, R, H), rnd(E, R, H)
-    h, dh = rnd(E, R, 2 * I), rnd(E, R, 2 * I)
+    dh = rnd(E, R, 2 * I)
     act, dact = rnd(E, R, I), rnd(E, R, I)
     w_fc, w_proj = rnd(E, 2 * I, H, std=0.02), rnd(E, H, I, std=0.02)
     products = {
-        "fwd_c_fc": (lambda: torch.bmm(x, w_fc.transpose(1, 2)), 2.0 * E * R * H * 2 * I),
-        "fwd_c_proj": (lambda: torch.bmm(act, w_proj.transpose(1, 2)), 2.0 * E * R * I * H),
-        "dx_c_proj": (lambda: torch.bmm(dy, w_proj), 2.0 * E * R * H * I),
-        "dx_c_fc": (lambda: torch.bmm(dh, w_fc), 2.0 * E * R * 2 * I * H),
-        "dw_c_fc": (lambda: torch.bmm(dh.transpose(1, 2), x), 2.0 * E * R * 2 * I * H),
-        "dw_c_proj": (lambda: torch.bmm(dy.transpose(1, 2), dact), 2.0 * E * R * H * I),
+        "fwd_c_fc": (lambda e: F.linear(x[e], w_fc[e]), 2.0 * E * R * H * 2 * I),
+        "fwd_c_proj": (lambda e: F.linear(act[e], w_proj[e]), 2.0 * E * R * I * H),
+        "dx_c_proj": (lambda e: dy[e].mm(w_proj[e]), 2.0 * E * R * H * I),
+        "dx_c_fc": (lambda e: dh[e].mm(w_fc[e]), 2.0 * E * R * 2 * I * H),
+        "dw_c_fc": (lambda e: dh[e].t().mm(x[e]), 2.0 * E * R * 2 * I * H),
+        "dw_c_proj": (lambda e: dy[e].t().mm(dact[e]), 2.0 * E * R * H * I),
     }
     out, total_ms, total_flop = {}, 0.0, 0.0
     for name, (fn, flop) in products.items():
+        print(f"[yardstick] {name}", file=sys.stderr, flush=True)
         for _ in range(warmup):
-            fn()
+            for e in range(E):
+                fn(e)
+        torch.cuda.synchronize()
         marks = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
         for start, end in marks:
             start.record()
-            fn()
+            for e in range(E):
+                fn(e)
             end.record()
         torch.cuda.synchronize()
         ms = sorted(s_.elapsed_time(e_) for s_, e_ in marks)[iters // 2]
@@ -350,8 +358,8 @@ def bench_dense_yardstick(device, iters=5, warmup=2):
     tflops = total_flop / (total_ms * 1e-3) / 1e12
     return {"TFLOP/s": round(tflops, 1), "frac_of_mfma_peak": round(tflops / BF16_MFMA_PEAK_TFLOPS, 4), "ms": round(total_ms, 3),
             "per_product_tflops": out,
-            "what": "torch.bmm (vendor library) on the six products as dense batches of 8 x 2048 rows, same data "
-                    "distribution, same box and power cap; a yardstick, not the target"}
+            "what": "vendor library (F.linear / torch.mm, 2-D, per expert) on the six products with 8 x 2048 rows, same "
+                    "data distribution, same box and power cap; a yardstick, not the target"}
 
 
 # ---- CPU baseline -----------------------------------------------------------------------------------------
@@ -427,7 +435,7 @@ def main():
         print(json.dumps({"extras": bench_extras(device, args.embedding_ids)}))
         return
     if args.only_yardstick:
-        print(json.dumps({"extras": {"dense_bmm_yardstick": bench_dense_yardstick(device)}}))
+        print(json.dumps({"extras": {"dense_yardstick": bench_dense_yardstick(device)}}))
         return
     # The host baseline runs first: the GPU legs then end the run, where a utilisation sampler from outside sees them.
     cpu = None if args.no_cpu else bench_cpu()
@@ -451,6 +459,8 @@ def main():
     }
     if not args.no_extras:
         line["extras"] = bench_extras(device)
+    if args.yardstick:
+        line.setdefault("extras", {})["dense_yardstick"] = bench_dense_yardstick(device)
     if cpu is not None:
         line["cpu_baseline"] = cpu
     print(json.dumps(line))

@@ -928,6 +928,21 @@ def test_moe_full_size_against_oracle_on_tokens_and_one_expert(gpu, case):
                      "MoE_Torch on the GPU vs oracle": outliers(r, e), "oracle(bmm) vs oracle": outliers(e_bmm, e)}
             for label, (share_, worst_) in stats.items():
                 print(f"[full size] {name}/{key}: {label}: share outside {share_:.2e}, worst {worst_:.2f} x tol", flush=True)
+            # The allowances are floors that stock torch sets, measured here on the same sample:
+            #  - against the oracle with its own order of roundings (bmm mixing, the reference's Triton layer) the HIP
+            #    layer may stray no further than the reference's plain-torch layer on this device strays from its own
+            #    oracle form (twice its share, one and a half times its worst element; measured at the Mixtral shape:
+            #    y 6.7e-6 / 1.41 against 2.7e-5 / 1.52, dx 6.1e-4 / 3.70 against 5.5e-4 / 3.05)
+            ref_share, ref_worst = stats["MoE_Torch on the GPU vs oracle"]
+            share_, worst_ = stats["hip vs oracle(bmm mixing)"]
+            assert share_ <= max(2 * ref_share, 1e-5), f"{name}/{key}: {share_:.2e} outside against its own form, MoE_Torch {ref_share:.2e}"
+            assert worst_ <= max(1.5 * ref_worst, 1.0), f"{name}/{key}: worst {worst_:.2f} x tol, MoE_Torch {ref_worst:.2f}"
+            #  - against the plain-torch form, no further than that plus what the reference's two forms differ by
+            #    between themselves (y 3.8e-5 / 1.56, dx 3.1e-3 / 4.69 at the Mixtral shape: HIP 7.2e-5 / 1.56, 3.5e-3 / 4.69)
+            forms_share, forms_worst = stats["oracle(bmm) vs oracle"]
+            share_, worst_ = stats["hip vs oracle"]
+            assert share_ <= max(1.5 * (ref_share + forms_share), 1e-5), f"{name}/{key}: {share_:.2e} outside"
+            assert worst_ <= max(1.5 * max(ref_worst, forms_worst), 1.0), f"{name}/{key}: worst {worst_:.2f} x tol"
             # measured: y 7e-5 of the elements outside (worst 1.6 times the tolerance), dx 3.5e-3 (worst 4.7) at the
             # Mixtral shape, where rows of size 2-3 (last place 2^-6) meet; none outside at the fine-grained shape
             share, worst = (5e-4, 4) if key == "y" else (1e-2, 8)
@@ -944,8 +959,14 @@ def test_moe_full_size_against_oracle_on_tokens_and_one_expert(gpu, case):
         a, e = got[key][e_star].cpu(), one[key]
         outside = O.fraction_outside(a, e, **tol)
         print(f"[full size] {name}/{key}[{e_star}] ({tok.numel()} rows): {outside:.2e} of {a.numel()} elements outside", flush=True)
-        for label, (share_, worst_) in {"hip vs oracle": outliers(a, e), "MoE_Torch on the GPU vs oracle": outliers(got_ref[key][e_star], e)}.items():
+        stats = {"hip vs oracle": outliers(a, e), "MoE_Torch on the GPU vs oracle": outliers(got_ref[key][e_star], e)}
+        for label, (share_, worst_) in stats.items():
             print(f"[full size] {name}/{key}[{e_star}]: {label}: share outside {share_:.2e}, worst {worst_:.2f} x tol", flush=True)
+        # no further from the oracle than stock torch's per-expert products on this device are (measured: the same
+        # share to 20 %, the same worst element - the outliers are where the CPU's bf16 sums round differently)
+        (share_, worst_), (ref_share, ref_worst) = stats["hip vs oracle"], stats["MoE_Torch on the GPU vs oracle"]
+        assert share_ <= max(1.5 * ref_share, 1e-6), f"{name}/{key}[{e_star}]: {share_:.2e} outside, MoE_Torch {ref_share:.2e}"
+        assert worst_ <= max(1.25 * ref_worst, 1.0), f"{name}/{key}[{e_star}]: worst {worst_:.2f} x tol, MoE_Torch {ref_worst:.2f}"
         # measured: 5e-5 to 7e-5 of the elements outside, worst 4 to 8 times the tolerance (sums over 2132 / 16339 rows)
         assert_close_but_for(a, e, dtype, 5e-4, 16, f"{name}/{key}[{e_star}]")
 
