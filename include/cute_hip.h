@@ -185,12 +185,18 @@ int ck_scatter2scatter(const void* X, int64_t x_stride, const void* W, int64_t w
  * ck_scatter2scatter_workspace_size() bytes (16-byte aligned; 0: the shape is not eligible - fp32, or K below 4096),
  * the tiles of every XCD's last round are cut into pieces of the contraction range, summed by a second launch on the
  * same stream.  Results differ from ck_scatter2scatter in the order of the fp32 additions only.  workspace == NULL
- * is ck_scatter2scatter. */
+ * is ck_scatter2scatter.
+ * `waves` (here and in the three entry points below) names the loop of the matrix-core kernel, the counterpart of the
+ * num_warps / num_stages of the reference's tuned Triton configurations (scattermoe/triton_implementation/
+ * kernels.py:152-159): 8 = eight wavefronts per 256 x 256 tile, two per SIMD working in antiphase; 4 = four
+ * wavefronts, one per SIMD, each a software pipeline over a 128 x 128 block with its accumulators in the
+ * accumulation registers; 0 = the library's choice.  Same tile grid, same results up to the order of the fp32
+ * additions inside a matrix instruction's block; anything else is CK_ERR_SHAPE.  A product with a bias takes 8. */
 int64_t ck_scatter2scatter_workspace_size(int64_t num_slots, int64_t K, int64_t N, int64_t E, int dtype);
 int ck_scatter2scatter_ws(const void* X, int64_t x_stride, const void* W, int64_t w_stride_e, int64_t w_stride_k,
                           int64_t w_stride_n, const int64_t* sorted_scattered_idxs, const int64_t* expert_offsets,
                           void* out, int64_t out_stride, int64_t num_slots, int64_t K, int64_t N, int64_t E,
-                          int64_t fan_out, int x_grouped, int y_grouped, const void* bias, int dtype,
+                          int64_t fan_out, int x_grouped, int y_grouped, const void* bias, int dtype, int waves,
                           void* workspace, int64_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
@@ -217,11 +223,12 @@ int ck_scatter2scatter_glu(const void* X, int64_t x_stride, const void* W, int64
                            int64_t w_stride_k, int64_t w_stride_n, const int64_t* sorted_scattered_idxs,
                            const int64_t* expert_offsets, void* h, int64_t h_stride, void* act,
                            int64_t act_stride, int64_t num_slots, int64_t K, int64_t I, int64_t E,
-                           int64_t fan_out, int x_grouped, int dtype, void* stream);
+                           int64_t fan_out, int x_grouped, int dtype, int waves, void* stream);
 int ck_scatter2scatter_glu_bwd(const void* DY, int64_t dy_stride, const void* W, int64_t w_stride_e,
                                int64_t w_stride_k, int64_t w_stride_n, const int64_t* expert_offsets,
                                const void* h, int64_t h_stride, void* d_h, int64_t d_h_stride,
-                               int64_t num_slots, int64_t K, int64_t I, int64_t E, int dtype, void* stream);
+                               int64_t num_slots, int64_t K, int64_t I, int64_t E, int dtype, int waves,
+                               void* stream);
 
 /* Inclusive expert offsets from already-sorted expert ids (int64 [M] -> int64 [E]); used when a caller
  * of cute::scatter2scatter has the sorted ids but not the offsets (ops.py:16-24 takes only the ids). */
@@ -237,7 +244,8 @@ int ck_offsets_from_sorted(const int64_t* sorted_expert_idxs, int64_t* expert_of
  * ------------------------------------------------------------------------------------------- */
 int ck_group_bwd_W(const void* DY, int64_t dy_stride, const void* X, int64_t x_stride,
                    const int64_t* expert_offsets, void* DW, int64_t dw_stride_e, int64_t dw_stride_k,
-                   int64_t dw_stride_n, int64_t M, int64_t K, int64_t N, int64_t E, int dtype, void* stream);
+                   int64_t dw_stride_n, int64_t M, int64_t K, int64_t N, int64_t E, int dtype, int waves,
+                   void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Row gather with optional per-row coefficient ("group")

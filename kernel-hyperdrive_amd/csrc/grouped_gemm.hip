@@ -12,6 +12,7 @@
 // never mixes rows of two experts (the reference lets a 128-row block straddle experts and repeats the
 // product once per expert present in it).  fp32, and shapes whose contiguous dimensions are not
 // multiples of 8 elements, go through a plain kernel with exact (fp64) accumulation.
+#include <cstdlib>
 #include <type_traits>
 
 #include "ck_device.h"
@@ -44,12 +45,20 @@ struct Mma16<BF16> {
     static __device__ __forceinline__ f32x4_t mma(frag_t a, frag_t b, f32x4_t c) {
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
     }
+    // the same with the accumulator pinned to the accumulation half of the register file (a loop with 256
+    // accumulator registers per lane: left to itself the register allocator moves them between the halves)
+    static __device__ __forceinline__ void mma_acc(frag_t a, frag_t b, f32x4_t& c) {
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    }
 };
 template <>
 struct Mma16<F16> {
     typedef f16x8_t frag_t;
     static __device__ __forceinline__ f32x4_t mma(frag_t a, frag_t b, f32x4_t c) {
         return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ void mma_acc(frag_t a, frag_t b, f32x4_t& c) {
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     }
 };
 
@@ -77,6 +86,7 @@ struct GemmParams {
     // S2S without activation: bias [E, N] of the operands' type, or null.  Added to the fp32 sums before they are
     // rounded, as F.linear(rows, W[e], bias[e]) rounds once (cute_kernels/kernels/scattermoe/torch_implementation.py:35-43).
     const void* bias;
+    int waves;  // host side only: which loop the launch takes (0: the library's choice, 4, 8)
 };
 
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -689,7 +699,7 @@ __device__ __forceinline__ void unpack2(uint32_t w, float& a, float& b) {
 template <typename T, typename TL, bool B_KC, bool GROUP_K, int GLU = 0, int MODE = 0>
 // Two waves per SIMD is all the LDS footprint allows; telling the compiler keeps it from spilling to reach a
 // higher occupancy that cannot happen.
-__global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
+__global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_eu(TL::WM * TL::WN / 4, TL::WM * TL::WN / 4)))
     grouped_gemm_m16_kernel(GemmParams p) {
     static_assert(MODE == 0 || (GLU == 0 && !GROUP_K), "tail splitting is for the plain per-expert products");
     typedef typename T::storage_t S;
@@ -709,7 +719,8 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
     // (wm, wn) owns rows wm * RW .. + RW of either A half and columns wn * CW .. + CW of either B half.
     typedef DtlOperand<S, BM / 2, A_KC, NWAVES> AOp;
     typedef DtlOperand<S, BN / 2, B_KCC, NWAVES> BOp;
-    static_assert(AOp::IPW == BOp::IPW && AOp::IPW == 2, "square tile; the wait counts of the loop assume two copies per M phase");
+    static_assert(AOp::IPW == BOp::IPW && AOp::IPW * NWAVES == 16, "square tile; the wait counts of the loops assume 16 copies per half operand");
+    static_assert(NWAVES == 8 || NWAVES == 4, "two loops: two wave groups in antiphase (8 waves), one software-pipelined wave per SIMD (4)");
     constexpr int IPW = AOp::IPW;  // copy instructions per wave and half operand
     constexpr int A_HALF = AOp::STAGE_BYTES, B_HALF = BOp::STAGE_BYTES, B_AT = 2 * A_HALF;
     constexpr int STAGE_BYTES = 2 * A_HALF + 2 * B_HALF;
@@ -841,6 +852,13 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
                 dma(bt, b_voff[part - 2][j], st + B_AT + (part - 2) * B_HALF + (wave * IPW + j) * 1024);
         }
     };
+    // copy instruction j (of IPW) of one half operand
+    auto issue_one = [&](char* st, int part, int t, int j) __attribute__((always_inline)) {
+        if (part < 2)
+            dma(a_base + (int64_t)t * a_step, a_voff[part][j], st + part * A_HALF + (wave * IPW + j) * 1024);
+        else
+            dma(b_base + (int64_t)t * b_step, b_voff[part - 2][j], st + B_AT + (part - 2) * B_HALF + (wave * IPW + j) * 1024);
+    };
     // tile t whatever its position: slots past the end of the contraction range are cleared instead of copied
     auto issue = [&](int t, char* st) __attribute__((always_inline)) {
         const int k0 = k_begin + t * BK;
@@ -969,7 +987,9 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
             for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
     // The per-expert bias is what the sums start from (not in a piece of a split tile: there the launch that adds
     // the pieces up starts from it): it joins the fp32 sums at no cost and is rounded with them, once.
-    if (GLU == 0 && !GROUP_K && p.bias != nullptr && !(MODE == 1 && part_slot >= 0)) {
+    // (eight waves only: with four, 256 initial values that depend on a branch wait in ordinary registers until the
+    // loop takes them over, and spill; the host sends products with a bias to the eight-wave loop)
+    if (NWAVES == 8 && GLU == 0 && !GROUP_K && p.bias != nullptr && !(MODE == 1 && part_slot >= 0)) {
         // a lane's four columns of every 16-column block, the same for all of its rows (see the epilogue)
         const S* brow = reinterpret_cast<const S*>(p.bias) + (int64_t)expert * p.N;
         const int lane = lane_id();
@@ -998,7 +1018,10 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
             for (int i = 0; i < TH; ++i)
 #pragma unroll
                 for (int j = 0; j < TNH; ++j)
-                    acc[ha * TH + i][hb * TNH + j] = Mma16<T>::mma(bf[kki][j], af[kki][i], acc[ha * TH + i][hb * TNH + j]);
+                    if constexpr (NWAVES == 4)
+                        Mma16<T>::mma_acc(bf[kki][j], af[kki][i], acc[ha * TH + i][hb * TNH + j]);
+                    else
+                        acc[ha * TH + i][hb * TNH + j] = Mma16<T>::mma(bf[kki][j], af[kki][i], acc[ha * TH + i][hb * TNH + j]);
     };
     frag_t fa[2][TH], fb0[2][TNH], fb1[2][TNH];
     // one whole tile, outside the pipelined loop
@@ -1091,6 +1114,148 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
 
     int kt = 0;
     if (MODE == 2) kt = k_tiles;  // nothing to multiply: the accumulators come from the partial tiles below
+    if constexpr (NWAVES == 4) {
+        // ---- one wave per SIMD: the same pipeline inside a single instruction stream ----------------------------
+        // Every wave owns a 128 x 128 block (64 rows of either A half x 64 columns of either B half; 256 accumulator
+        // registers, which the compiler keeps in the accumulation half of the register file), so a step reads
+        // 128 KB of fragments from LDS per CU where eight waves of 128 x 64 read 192 KB.  A step is four quarters of
+        // 32 matrix instructions (row half x column half over the tile depth).  While a quarter multiplies, the wave
+        // reads the one half operand the next quarter lacks into registers that are free, and requests four copies:
+        //   Q0  A lower x B lower      reads B upper of X            copies B lower of X <- tile kt + 2
+        //   Q1  A lower x B upper      reads A upper of X            copies B upper of X <- tile kt + 2
+        //   Q2  A upper x B upper      reads A lower of Y            copies A upper of X <- tile kt + 2
+        //   Q3  A upper x B lower      reads B lower of Y            copies A lower of Y <- tile kt + 3
+        // (X holds tile kt, Y tile kt + 1.)  A half is overwritten in the quarter after the one that read it, and read
+        // seven quarters after its copy was requested.  A quarter ends with a wait that leaves the 24 most recent
+        // copies of the wave outstanding (four per quarter, so everything older than six quarters has landed), a
+        // wait for the wave's own LDS reads (the half they came from is overwritten next), and a workgroup barrier.
+        // The loads and copies are spread between the matrix instructions, two of those per slot, and the slots are
+        // fenced for the instruction scheduler so that the spacing survives.
+        static_assert(NWAVES != 4 || (TH == 4 && TNH == 4), "a quarter is 4 x 4 blocks");
+        auto ld_a = [&](const char* st, int h, int kki, int i) __attribute__((always_inline)) -> frag_t {
+            const int kk = kki * 32;
+            const int kc = frag_row + (opaque(frag_swz) ^ ((kk / 8) << 4));
+            const int ii = h * TH + i;
+            if (A_KC) {
+                return *reinterpret_cast<const frag_t*>(st + kc + a_off[ii]);
+            } else {
+                const char* q = st + a_off[ii & ~1] + (ii & 1) * odd_step + kk * BM;
+                union {
+                    v4i16_t h2[2];
+                    frag_t f;
+                } u;
+                u.h2[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(q));
+                u.h2[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(q + 4 * BM));
+                return u.f;
+            }
+        };
+        auto ld_b = [&](const char* st, int h, int kki, int j) __attribute__((always_inline)) -> frag_t {
+            const int kk = kki * 32;
+            const int kc = frag_row + (opaque(frag_swz) ^ ((kk / 8) << 4));
+            const int jj = h * TNH + j;
+            if (B_KCC) {
+                return *reinterpret_cast<const frag_t*>(st + kc + b_off[jj]);
+            } else {
+                const char* q = st + b_off[jj & ~1] + (jj & 1) * odd_step + kk * BN;
+                union {
+                    v4i16_t h2[2];
+                    frag_t f;
+                } u;
+                u.h2[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(q));
+                u.h2[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(q + 4 * BN));
+                return u.f;
+            }
+        };
+#define CK_Q_END()                                                \
+    do {                                                          \
+        __builtin_amdgcn_sched_barrier(0);                        \
+        asm volatile("s_waitcnt vmcnt(24)" ::: "memory");         \
+        __builtin_amdgcn_s_waitcnt(0xC07F); /* lgkmcnt(0) */      \
+        __builtin_amdgcn_s_barrier();                             \
+        __builtin_amdgcn_sched_barrier(0);                        \
+    } while (0)
+        // One quarter: the matrix instructions of rows half ha x columns half hb (if `mma`), fragment n of the next
+        // half operand through load_one(n) in every other slot (if `load`), copy instruction c of half `cpart` of
+        // tile ct into stage cst in slots 1, 5, 9, 13.
+        auto quarter = [&](auto mma, auto load, int ha, int hb, frag_t (*af)[TH], frag_t (*bf)[TNH], auto load_one,
+                           char* cst, int cpart, int ct) __attribute__((always_inline)) {
+            constexpr bool MMA = decltype(mma)::value;
+            constexpr bool LOAD = decltype(load)::value;
+#pragma unroll
+            for (int sl = 0; sl < 16; ++sl) {
+                if (LOAD && sl % 2 == 0) load_one(sl / 2);
+                if (sl % 4 == 1) issue_one(cst, cpart, ct, sl / 4);
+                if (MMA) {
+#pragma unroll
+                    for (int m = 2 * sl; m < 2 * sl + 2; ++m) {
+                        const int kki = m / 16, i = (m / 4) % 4, j = m % 4;
+                        Mma16<T>::mma_acc(bf[kki][j], af[kki][i], acc[ha * TH + i][hb * TNH + j]);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            CK_Q_END();
+        };
+        frag_t fa0[2][TH], fa1[2][TH], fbx[2][TNH], fby[2][TNH];
+        // one step: bl holds B lower of tile kt on entry and is free on exit, bu receives B upper of tile kt, then
+        // B lower of tile kt + 1
+        auto w4_step = [&](auto upper, auto upper_cols, int kt_, char* X, char* Y, frag_t (*bl)[TNH], frag_t (*bu)[TNH]) __attribute__((always_inline)) {
+            constexpr bool UPPER = decltype(upper)::value;
+            constexpr bool UCOLS = decltype(upper_cols)::value;
+            typedef std::integral_constant<bool, UPPER> up_t;
+            typedef std::integral_constant<bool, UCOLS> uc_t;
+            typedef std::integral_constant<bool, UPPER && UCOLS> both_t;
+            // the last steps of a range have no tile left to request: they request the last tile once more, into
+            // halves that nobody reads again, which keeps the count of outstanding copies the same in every quarter
+            const int t2 = min(kt_ + 2, n_full - 1), t3 = min(kt_ + 3, n_full - 1);
+            quarter(std::true_type{}, uc_t{}, 0, 0, fa0, bl, [&](int n) __attribute__((always_inline)) { bu[n / 4][n % 4] = ld_b(X, 1, n / 4, n % 4); }, X, 2, t2);
+            quarter(uc_t{}, up_t{}, 0, 1, fa0, bu, [&](int n) __attribute__((always_inline)) { fa1[n / 4][n % 4] = ld_a(X, 1, n / 4, n % 4); }, X, 3, t2);
+            quarter(both_t{}, std::true_type{}, 1, 1, fa1, bu, [&](int n) __attribute__((always_inline)) { fa0[n / 4][n % 4] = ld_a(Y, 0, n / 4, n % 4); }, X, 1, t2);
+            quarter(up_t{}, std::true_type{}, 1, 0, fa1, bl, [&](int n) __attribute__((always_inline)) { bu[n / 4][n % 4] = ld_b(Y, 0, n / 4, n % 4); }, Y, 0, t3);
+        };
+        if (MODE != 2 && n_full >= 2) {
+            // tiles 0 and 1 in the order of the loop's requests (A lower, B lower, B upper, A upper); A lower and B
+            // lower of tile 0 go to the registers, then A lower of tile 2 may follow over A lower of tile 0
+            issue_part(lds0, 0, 0);
+            issue_part(lds0, 2, 0);
+            issue_part(lds0, 3, 0);
+            issue_part(lds0, 1, 0);
+            issue_part(lds1, 0, 1);
+            issue_part(lds1, 2, 1);
+            issue_part(lds1, 3, 1);
+            issue_part(lds1, 1, 1);
+            CK_Q_END();  // the first 8 of 32 have landed: A lower and B lower of tile 0
+#pragma unroll
+            for (int n = 0; n < 8; ++n) {
+                fa0[n / 4][n % 4] = ld_a(lds0, 0, n / 4, n % 4);
+                fbx[n / 4][n % 4] = ld_b(lds0, 0, n / 4, n % 4);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+            issue_part(lds0, 0, min(2, n_full - 1));
+            CK_Q_END();  // B upper of tile 0 has landed: 24 younger copies
+            auto run = [&](auto upper, auto upper_cols) __attribute__((always_inline)) {
+                for (; kt + 1 < n_full; kt += 2) {
+                    w4_step(upper, upper_cols, kt, lds0, lds1, fbx, fby);
+                    w4_step(upper, upper_cols, kt + 1, lds1, lds0, fby, fbx);
+                }
+            };
+            if (upper_rows_live && upper_cols_live) run(std::true_type{}, std::true_type{});
+            else if (upper_cols_live) run(std::false_type{}, std::true_type{});
+            else if (upper_rows_live) run(std::true_type{}, std::false_type{});
+            else run(std::false_type{}, std::false_type{});
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (kt < n_full) {  // an odd number of full tiles: the last one is complete in lds0
+                multiply_tile(lds0);
+                ++kt;
+                __syncthreads();
+            }
+        }
+#undef CK_Q_END
+    } else
     if (MODE != 2 && n_full >= 2) {
 #pragma unroll
         for (int part = 0; part < 4; ++part) issue_part(lds0, part, 0);
@@ -1183,88 +1348,188 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
             *reinterpret_cast<u32x2_t*>(Ch + row * C_LD + col) = four;
         }
     }
-    S* Cbase = reinterpret_cast<S*>(p.C) + (GROUP_K ? (int64_t)expert * p.c_stride_e : 0);
-    typedef VPack<T, 8> P8;
-    // GLU == 1: a lane takes an "up" packet together with its "gate" packet, so packets are counted over half a row
-    constexpr int C_CHUNKS_PER_ROW = (GLU == 1 ? BN / 2 : BN) / 8;
-    constexpr int C_CH = BM * C_CHUNKS_PER_ROW / THREADS;
-    // The loads an output packet depends on are all requested before anything is stored, and without branches
-    // (positions outside the tile are redirected to a valid one): the destination rows of scattered outputs, the
-    // up / gate packets of h for GLU == 2 - both while the workgroup is on its way to the barrier - and, behind the
-    // barrier, the staged packets themselves.  Packet by packet, every store would wait for its own loads in turn
-    // (and, with one counter for loads and stores, for the store before it).
-    constexpr int H_CH = GLU == 2 ? C_CH : 1;
-    P8 h_up[H_CH], h_gate[H_CH];
-    int64_t out_row[C_CH];
-#pragma unroll
-    for (int i = 0; i < C_CH; ++i) {
-        const int row = min((tid + i * THREADS) / C_CHUNKS_PER_ROW, rows_valid - 1);
-        out_row[i] = GROUP_K ? i_base + row : row_start + row;
-    }
-    if (!GROUP_K && !p.y_grouped) {
-#pragma unroll
-        for (int i = 0; i < C_CH; ++i) out_row[i] = p.row_idx[out_row[i]];
-    }
-    if (GLU == 2) {
-#pragma unroll
+    if constexpr (NWAVES == 8) {
+        S* Cbase = reinterpret_cast<S*>(p.C) + (GROUP_K ? (int64_t)expert * p.c_stride_e : 0);
+        typedef VPack<T, 8> P8;
+        // GLU == 1: a lane takes an "up" packet together with its "gate" packet, so packets are counted over half a row
+        constexpr int C_CHUNKS_PER_ROW = (GLU == 1 ? BN / 2 : BN) / 8;
+        constexpr int C_CH = BM * C_CHUNKS_PER_ROW / THREADS;
+        // The loads an output packet depends on are all requested before anything is stored, and without branches
+        // (positions outside the tile are redirected to a valid one): the destination rows of scattered outputs, the
+        // up / gate packets of h for GLU == 2 - both while the workgroup is on its way to the barrier - and, behind the
+        // barrier, the staged packets themselves.  Packet by packet, every store would wait for its own loads in turn
+        // (and, with one counter for loads and stores, for the store before it).
+        constexpr int H_CH = GLU == 2 ? C_CH : 1;
+        P8 h_up[H_CH], h_gate[H_CH];
+        int64_t out_row[C_CH];
+    #pragma unroll
         for (int i = 0; i < C_CH; ++i) {
-            const int col = min(((tid + i * THREADS) % C_CHUNKS_PER_ROW) * 8, cols_valid - 8);
-            const S* hrow = reinterpret_cast<const S*>(p.aux) + out_row[i] * p.ld_aux + n_base + col;
-            h_up[i] = nt_load(reinterpret_cast<const P8*>(hrow));
-            h_gate[i] = nt_load(reinterpret_cast<const P8*>(hrow + p.glu_half));
+            const int row = min((tid + i * THREADS) / C_CHUNKS_PER_ROW, rows_valid - 1);
+            out_row[i] = GROUP_K ? i_base + row : row_start + row;
         }
-    }
-    __syncthreads();
-    constexpr int G_CH = GLU == 1 ? C_CH : 1;
-    P8 staged[C_CH], staged_gate[G_CH];
-#pragma unroll
-    for (int i = 0; i < C_CH; ++i) {
-        const int c = tid + i * THREADS;
-        const int row = c / C_CHUNKS_PER_ROW;
-        const int col = (c % C_CHUNKS_PER_ROW) * 8;
-        const S* src = reinterpret_cast<const S*>(row < BM / 2 ? lds0 : lds1) + (row % (BM / 2)) * C_LD + col;
-        staged[i] = *reinterpret_cast<const P8*>(src);
-        // GLU == 1: columns [0, BN / 2) of the tile are "up", [BN / 2, BN) the matching "gate"
-        if (GLU == 1) staged_gate[i] = *reinterpret_cast<const P8*>(src + BN / 2);
-    }
-#pragma unroll
-    for (int i = 0; i < C_CH; ++i) {
-        const int c = tid + i * THREADS;
-        const int row = c / C_CHUNKS_PER_ROW;
-        const int col = (c % C_CHUNKS_PER_ROW) * 8;
-        if (row < rows_valid && col < cols_valid) {
-            if (GLU == 0) {
-                *reinterpret_cast<P8*>(Cbase + out_row[i] * p.ldc + n_base + col) = staged[i];
-            } else if (GLU == 1) {
-                // both halves go to h, and the activation is computed from the rounded values exactly as the
-                // separate kernel would from h
-                const P8 u = staged[i];
-                const P8 g = staged_gate[GLU == 1 ? i : 0];
-                P8 y;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) y.v[e] = T::down(swiglu_fwd_1<T>(T::up(g.v[e]), T::up(u.v[e])));
-                S* hrow = Cbase + out_row[i] * p.ldc + n_base + col;
-                *reinterpret_cast<P8*>(hrow) = u;
-                *reinterpret_cast<P8*>(hrow + p.glu_half) = g;
-                *reinterpret_cast<P8*>(reinterpret_cast<S*>(p.aux) + out_row[i] * p.ld_aux + n_base + col) = y;
-            } else {
-                // the staged tile is d_act (rounded, as the separate kernels would hand it over); h supplies up
-                // and gate of the same positions, and d_h receives both derivatives
-                const P8 u = h_up[GLU == 2 ? i : 0];
-                const P8 g = h_gate[GLU == 2 ? i : 0];
-                const P8 d = staged[i];
-                P8 du, dg;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    float fg, fu;
-                    swiglu_bwd_1<T>(T::up(g.v[e]), T::up(u.v[e]), T::up(d.v[e]), fg, fu);
-                    dg.v[e] = T::down(fg);
-                    du.v[e] = T::down(fu);
-                }
-                S* drow = Cbase + out_row[i] * p.ldc + n_base + col;
-                *reinterpret_cast<P8*>(drow) = du;
-                *reinterpret_cast<P8*>(drow + p.glu_half) = dg;
+        if (!GROUP_K && !p.y_grouped) {
+    #pragma unroll
+            for (int i = 0; i < C_CH; ++i) out_row[i] = p.row_idx[out_row[i]];
+        }
+        if (GLU == 2) {
+    #pragma unroll
+            for (int i = 0; i < C_CH; ++i) {
+                const int col = min(((tid + i * THREADS) % C_CHUNKS_PER_ROW) * 8, cols_valid - 8);
+                const S* hrow = reinterpret_cast<const S*>(p.aux) + out_row[i] * p.ld_aux + n_base + col;
+                h_up[i] = nt_load(reinterpret_cast<const P8*>(hrow));
+                h_gate[i] = nt_load(reinterpret_cast<const P8*>(hrow + p.glu_half));
             }
+        }
+        __syncthreads();
+        constexpr int G_CH = GLU == 1 ? C_CH : 1;
+        P8 staged[C_CH], staged_gate[G_CH];
+    #pragma unroll
+        for (int i = 0; i < C_CH; ++i) {
+            const int c = tid + i * THREADS;
+            const int row = c / C_CHUNKS_PER_ROW;
+            const int col = (c % C_CHUNKS_PER_ROW) * 8;
+            const S* src = reinterpret_cast<const S*>(row < BM / 2 ? lds0 : lds1) + (row % (BM / 2)) * C_LD + col;
+            staged[i] = *reinterpret_cast<const P8*>(src);
+            // GLU == 1: columns [0, BN / 2) of the tile are "up", [BN / 2, BN) the matching "gate"
+            if (GLU == 1) staged_gate[i] = *reinterpret_cast<const P8*>(src + BN / 2);
+        }
+    #pragma unroll
+        for (int i = 0; i < C_CH; ++i) {
+            const int c = tid + i * THREADS;
+            const int row = c / C_CHUNKS_PER_ROW;
+            const int col = (c % C_CHUNKS_PER_ROW) * 8;
+            if (row < rows_valid && col < cols_valid) {
+                if (GLU == 0) {
+                    *reinterpret_cast<P8*>(Cbase + out_row[i] * p.ldc + n_base + col) = staged[i];
+                } else if (GLU == 1) {
+                    // both halves go to h, and the activation is computed from the rounded values exactly as the
+                    // separate kernel would from h
+                    const P8 u = staged[i];
+                    const P8 g = staged_gate[GLU == 1 ? i : 0];
+                    P8 y;
+    #pragma unroll
+                    for (int e = 0; e < 8; ++e) y.v[e] = T::down(swiglu_fwd_1<T>(T::up(g.v[e]), T::up(u.v[e])));
+                    S* hrow = Cbase + out_row[i] * p.ldc + n_base + col;
+                    *reinterpret_cast<P8*>(hrow) = u;
+                    *reinterpret_cast<P8*>(hrow + p.glu_half) = g;
+                    *reinterpret_cast<P8*>(reinterpret_cast<S*>(p.aux) + out_row[i] * p.ld_aux + n_base + col) = y;
+                } else {
+                    // the staged tile is d_act (rounded, as the separate kernels would hand it over); h supplies up
+                    // and gate of the same positions, and d_h receives both derivatives
+                    const P8 u = h_up[GLU == 2 ? i : 0];
+                    const P8 g = h_gate[GLU == 2 ? i : 0];
+                    const P8 d = staged[i];
+                    P8 du, dg;
+    #pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        float fg, fu;
+                        swiglu_bwd_1<T>(T::up(g.v[e]), T::up(u.v[e]), T::up(d.v[e]), fg, fu);
+                        dg.v[e] = T::down(fg);
+                        du.v[e] = T::down(fu);
+                    }
+                    S* drow = Cbase + out_row[i] * p.ldc + n_base + col;
+                    *reinterpret_cast<P8*>(drow) = du;
+                    *reinterpret_cast<P8*>(drow + p.glu_half) = dg;
+                }
+            }
+        }
+    } else {
+        // four waves: twice the packets per lane, taken in two passes over the same registers
+        S* Cbase = reinterpret_cast<S*>(p.C) + (GROUP_K ? (int64_t)expert * p.c_stride_e : 0);
+        typedef VPack<T, 8> P8;
+        // GLU == 1: a lane takes an "up" packet together with its "gate" packet, so packets are counted over half a row
+        constexpr int C_CHUNKS_PER_ROW = (GLU == 1 ? BN / 2 : BN) / 8;
+        // packets per lane: with four waves twice as many as with eight, taken in two passes over the same registers
+        constexpr int PASSES = NWAVES == 4 ? 2 : 1;
+        constexpr int C_CH = BM * C_CHUNKS_PER_ROW / THREADS / PASSES;
+        // The loads an output packet depends on are all requested before anything is stored, and without branches
+        // (positions outside the tile are redirected to a valid one): the destination rows of scattered outputs, the
+        // up / gate packets of h for GLU == 2 - in the first pass while the workgroup is on its way to the barrier - and,
+        // behind the barrier, the staged packets themselves.  Packet by packet, every store would wait for its own loads
+        // in turn (and, with one counter for loads and stores, for the store before it).
+        constexpr int H_CH = GLU == 2 ? C_CH : 1;
+        P8 h_up[H_CH], h_gate[H_CH];
+        int64_t out_row[C_CH];
+        auto request = [&](int pass) __attribute__((always_inline)) {
+    #pragma unroll
+            for (int i = 0; i < C_CH; ++i) {
+                const int row = min((tid + (pass * C_CH + i) * THREADS) / C_CHUNKS_PER_ROW, rows_valid - 1);
+                out_row[i] = GROUP_K ? i_base + row : row_start + row;
+            }
+            if (!GROUP_K && !p.y_grouped) {
+    #pragma unroll
+                for (int i = 0; i < C_CH; ++i) out_row[i] = p.row_idx[out_row[i]];
+            }
+            if (GLU == 2) {
+    #pragma unroll
+                for (int i = 0; i < C_CH; ++i) {
+                    const int col = min(((tid + (pass * C_CH + i) * THREADS) % C_CHUNKS_PER_ROW) * 8, cols_valid - 8);
+                    const S* hrow = reinterpret_cast<const S*>(p.aux) + out_row[i] * p.ld_aux + n_base + col;
+                    h_up[i] = nt_load(reinterpret_cast<const P8*>(hrow));
+                    h_gate[i] = nt_load(reinterpret_cast<const P8*>(hrow + p.glu_half));
+                }
+            }
+        };
+        constexpr int G_CH = GLU == 1 ? C_CH : 1;
+        auto write_out = [&](int pass) __attribute__((always_inline)) {
+            P8 staged[C_CH], staged_gate[G_CH];
+    #pragma unroll
+            for (int i = 0; i < C_CH; ++i) {
+                const int c = tid + (pass * C_CH + i) * THREADS;
+                const int row = c / C_CHUNKS_PER_ROW;
+                const int col = (c % C_CHUNKS_PER_ROW) * 8;
+                const S* src = reinterpret_cast<const S*>(row < BM / 2 ? lds0 : lds1) + (row % (BM / 2)) * C_LD + col;
+                staged[i] = *reinterpret_cast<const P8*>(src);
+                // GLU == 1: columns [0, BN / 2) of the tile are "up", [BN / 2, BN) the matching "gate"
+                if (GLU == 1) staged_gate[i] = *reinterpret_cast<const P8*>(src + BN / 2);
+            }
+    #pragma unroll
+            for (int i = 0; i < C_CH; ++i) {
+                const int c = tid + (pass * C_CH + i) * THREADS;
+                const int row = c / C_CHUNKS_PER_ROW;
+                const int col = (c % C_CHUNKS_PER_ROW) * 8;
+                if (row < rows_valid && col < cols_valid) {
+                    if (GLU == 0) {
+                        *reinterpret_cast<P8*>(Cbase + out_row[i] * p.ldc + n_base + col) = staged[i];
+                    } else if (GLU == 1) {
+                        // both halves go to h, and the activation is computed from the rounded values exactly as the
+                        // separate kernel would from h
+                        const P8 u = staged[i];
+                        const P8 g = staged_gate[GLU == 1 ? i : 0];
+                        P8 y;
+    #pragma unroll
+                        for (int e = 0; e < 8; ++e) y.v[e] = T::down(swiglu_fwd_1<T>(T::up(g.v[e]), T::up(u.v[e])));
+                        S* hrow = Cbase + out_row[i] * p.ldc + n_base + col;
+                        *reinterpret_cast<P8*>(hrow) = u;
+                        *reinterpret_cast<P8*>(hrow + p.glu_half) = g;
+                        *reinterpret_cast<P8*>(reinterpret_cast<S*>(p.aux) + out_row[i] * p.ld_aux + n_base + col) = y;
+                    } else {
+                        // the staged tile is d_act (rounded, as the separate kernels would hand it over); h supplies up
+                        // and gate of the same positions, and d_h receives both derivatives
+                        const P8 u = h_up[GLU == 2 ? i : 0];
+                        const P8 g = h_gate[GLU == 2 ? i : 0];
+                        const P8 d = staged[i];
+                        P8 du, dg;
+    #pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            float fg, fu;
+                            swiglu_bwd_1<T>(T::up(g.v[e]), T::up(u.v[e]), T::up(d.v[e]), fg, fu);
+                            dg.v[e] = T::down(fg);
+                            du.v[e] = T::down(fu);
+                        }
+                        S* drow = Cbase + out_row[i] * p.ldc + n_base + col;
+                        *reinterpret_cast<P8*>(drow) = du;
+                        *reinterpret_cast<P8*>(drow + p.glu_half) = dg;
+                    }
+                }
+            }
+        };
+        request(0);
+        __syncthreads();
+        write_out(0);
+        if (PASSES == 2) {
+            request(1);
+            write_out(1);
         }
     }
 }
@@ -1384,7 +1649,9 @@ namespace {
 #define CK_TILE_CONFIG 256, 256, 64, 2, 4
 #endif
 typedef ck::Tile<CK_TILE_CONFIG> MainTile;
+typedef ck::Tile<256, 256, 64, 2, 2> FourWaveTile;  // the same tile by four waves, one per SIMD
 constexpr int kBM = MainTile::BM, kBN = MainTile::BN;
+static_assert(FourWaveTile::BM == kBM && FourWaveTile::BN == kBN, "both loops work on one tile grid");
 
 // Workgroups for the products cut per expert: 8 XCD lists, each long enough for either way find_tile_balanced
 // deals the tiles (an eighth of the tiles, or whole rows of the tile grid), at the bound of the row tile count.
@@ -1392,6 +1659,29 @@ int64_t dealt_grid(const ck::GemmParams& p) {
     const int64_t even = ((int64_t)p.m_tiles * p.n_tiles + 7) / 8;
     const int64_t rows = (int64_t)((p.m_tiles + 7) / 8) * p.n_tiles;
     return 8 * (even > rows ? even : rows);
+}
+
+// Which of the two loops a launch takes (the tile grid is the same): 8 = two wave groups in antiphase, 4 = one
+// software-pipelined wave per SIMD.
+// `waves` of the entry points: 0 = the library's choice (eight, unless the environment variable CK_GEMM_WAVES says 4 -
+// a switch for measurements), 4 or 8 = that loop.  Products with a bias always take eight.
+int default_gemm_waves() {
+    static const int waves = [] {
+        const char* v = getenv("CK_GEMM_WAVES");
+        return v && v[0] == '4' ? 4 : 8;
+    }();
+    return waves;
+}
+bool valid_waves(int waves) { return waves == 0 || waves == 4 || waves == 8; }
+
+template <typename T, bool B_KC, bool GROUP_K, int GLU = 0, int MODE = 0>
+void launch_m16(unsigned grid, const ck::GemmParams& p, hipStream_t s) {
+    if ((p.waves == 0 ? default_gemm_waves() : p.waves) == 4 && p.bias == nullptr)
+        hipLaunchKernelGGL((ck::grouped_gemm_m16_kernel<T, FourWaveTile, B_KC, GROUP_K, GLU, MODE>), dim3(grid),
+                           dim3(FourWaveTile::THREADS), 0, s, p);
+    else
+        hipLaunchKernelGGL((ck::grouped_gemm_m16_kernel<T, MainTile, B_KC, GROUP_K, GLU, MODE>), dim3(grid),
+                           dim3(MainTile::THREADS), 0, s, p);
 }
 
 template <typename T, bool B_KC, bool GROUP_K>
@@ -1405,11 +1695,9 @@ void launch_mfma(const ck::GemmParams& p, hipStream_t s) {
         // 8 lists (one per XCD), each with ceil(tiles per expert / 8) entries per expert: see weight_grad_tile
         const int64_t per_expert = (int64_t)(p.m_tiles / p.E) * p.n_tiles;
         const int64_t listed = 8 * (int64_t)p.E * ((per_expert + 7) / 8);  // < 2^31: m_tiles * n_tiles is checked by the caller
-        hipLaunchKernelGGL((ck::grouped_gemm_m16_kernel<T, MainTile, B_KC, GROUP_K>), dim3((unsigned)listed),
-                           dim3(MainTile::THREADS), 0, s, p);
+        launch_m16<T, B_KC, GROUP_K>((unsigned)listed, p, s);
     } else
-        hipLaunchKernelGGL((ck::grouped_gemm_m16_kernel<T, MainTile, B_KC, GROUP_K>), dim3((unsigned)dealt_grid(p)),
-                           dim3(MainTile::THREADS), 0, s, p);
+        launch_m16<T, B_KC, GROUP_K>((unsigned)dealt_grid(p), p, s);
 }
 
 // per-expert product whose last round of tiles is split along the contraction (see find_tile_split): the tiles,
@@ -1417,10 +1705,8 @@ void launch_mfma(const ck::GemmParams& p, hipStream_t s) {
 template <typename T, bool B_KC>
 void launch_mfma_split(const ck::GemmParams& p, hipStream_t s) {
     const int64_t per_xcd = ((int64_t)p.m_tiles * p.n_tiles + 7) / 8 + 32;  // the pieces of a tail take up to 32 places
-    hipLaunchKernelGGL((ck::grouped_gemm_m16_kernel<T, MainTile, B_KC, false, 0, 1>), dim3((unsigned)(8 * per_xcd)),
-                       dim3(MainTile::THREADS), 0, s, p);
-    hipLaunchKernelGGL((ck::grouped_gemm_m16_kernel<T, MainTile, B_KC, false, 0, 2>), dim3(8 * 16),
-                       dim3(MainTile::THREADS), 0, s, p);
+    launch_m16<T, B_KC, false, 0, 1>((unsigned)(8 * per_xcd), p, s);
+    launch_m16<T, B_KC, false, 0, 2>(8 * 16, p, s);
 }
 
 constexpr int64_t kSplitWorkspaceBytes = (int64_t)ck::kSplitSlots * kBM * kBN * 4;
@@ -1430,8 +1716,7 @@ constexpr int64_t kSplitMinK = 2 * ck::kSplitMinTiles * 64;
 // per-expert product with the SwiGLU epilogue GLU (1: forward, 2: backward); never the wide kernel
 template <typename T, bool B_KC, int GLU>
 void launch_mfma_glu(const ck::GemmParams& p, hipStream_t s) {
-    hipLaunchKernelGGL((ck::grouped_gemm_m16_kernel<T, MainTile, B_KC, false, GLU>), dim3((unsigned)dealt_grid(p)),
-                       dim3(MainTile::THREADS), 0, s, p);
+    launch_m16<T, B_KC, false, GLU>((unsigned)dealt_grid(p), p, s);
 }
 
 bool mult8(int64_t v) { return (v & 7) == 0; }
@@ -1449,17 +1734,17 @@ extern "C" int ck_scatter2scatter(const void* X, int64_t x_stride, const void* W
                                   int64_t K, int64_t N, int64_t E, int64_t fan_out, int x_grouped, int y_grouped,
                                   const void* bias, int dtype, void* stream) {
     return ck_scatter2scatter_ws(X, x_stride, W, w_stride_e, w_stride_k, w_stride_n, sorted_scattered_idxs, expert_offsets,
-                                 out, out_stride, num_slots, K, N, E, fan_out, x_grouped, y_grouped, bias, dtype, nullptr, 0,
-                                 stream);
+                                 out, out_stride, num_slots, K, N, E, fan_out, x_grouped, y_grouped, bias, dtype, 0, nullptr,
+                                 0, stream);
 }
 
 extern "C" int ck_scatter2scatter_ws(const void* X, int64_t x_stride, const void* W, int64_t w_stride_e,
                                      int64_t w_stride_k, int64_t w_stride_n, const int64_t* sorted_scattered_idxs,
                                      const int64_t* expert_offsets, void* out, int64_t out_stride, int64_t num_slots,
                                      int64_t K, int64_t N, int64_t E, int64_t fan_out, int x_grouped, int y_grouped,
-                                     const void* bias, int dtype, void* workspace, int64_t workspace_bytes,
-                                     void* stream) {
-    if (num_slots < 0 || K < 0 || N < 0 || E <= 0 || fan_out <= 0) return CK_ERR_SHAPE;
+                                     const void* bias, int dtype, int waves, void* workspace,
+                                     int64_t workspace_bytes, void* stream) {
+    if (num_slots < 0 || K < 0 || N < 0 || E <= 0 || fan_out <= 0 || !valid_waves(waves)) return CK_ERR_SHAPE;
     if (num_slots > 0x7fffffff || K > 0x7fffffff || N > 0x7fffffff || E > 0x7fffffff) return CK_ERR_SHAPE;
     if (dtype != CK_F32 && dtype != CK_F16 && dtype != CK_BF16) return CK_ERR_DTYPE;
     if (num_slots == 0 || N == 0) return CK_OK;
@@ -1492,6 +1777,7 @@ extern "C" int ck_scatter2scatter_ws(const void* X, int64_t x_stride, const void
         p.x_grouped = x_grouped;
         p.y_grouped = y_grouped;
         p.bias = bias;
+        p.waves = waves;
         // the direct-to-LDS kernel addresses a tile's sources with 32-bit byte offsets from a per-tile base
         p.wide = num_slots * x_stride * 2 >= (int64_t)1 << 32 || (b_kc ? N : K) * p.ldb * 2 >= (int64_t)1 << 32;
         p.m_tiles = (int)(num_slots / kBM + E);
@@ -1535,8 +1821,8 @@ extern "C" int ck_scatter2scatter_glu(const void* X, int64_t x_stride, const voi
                                       int64_t w_stride_k, int64_t w_stride_n, const int64_t* sorted_scattered_idxs,
                                       const int64_t* expert_offsets, void* h, int64_t h_stride, void* act,
                                       int64_t act_stride, int64_t num_slots, int64_t K, int64_t I, int64_t E,
-                                      int64_t fan_out, int x_grouped, int dtype, void* stream) {
-    if (num_slots < 0 || K < 0 || I < 0 || E <= 0 || fan_out <= 0) return CK_ERR_SHAPE;
+                                      int64_t fan_out, int x_grouped, int dtype, int waves, void* stream) {
+    if (num_slots < 0 || K < 0 || I < 0 || E <= 0 || fan_out <= 0 || !valid_waves(waves)) return CK_ERR_SHAPE;
     if (num_slots > 0x7fffffff || K > 0x7fffffff || I > 0x3fffffff || E > 0x7fffffff) return CK_ERR_SHAPE;
     if (dtype != CK_F32 && dtype != CK_F16 && dtype != CK_BF16) return CK_ERR_DTYPE;
     if (num_slots == 0 || I == 0) return CK_OK;
@@ -1573,6 +1859,7 @@ extern "C" int ck_scatter2scatter_glu(const void* X, int64_t x_stride, const voi
         p.aux = act;
         p.ld_aux = act_stride;
         p.glu_half = (int)I;
+        p.waves = waves;
         p.m_tiles = (int)(num_slots / kBM + E);
         p.n_tiles = (int)(I / (kBN / 2));
         if ((int64_t)(p.m_tiles + 8) * p.n_tiles > 0x7ffffff0) return CK_ERR_SHAPE;
@@ -1596,8 +1883,9 @@ extern "C" int ck_scatter2scatter_glu(const void* X, int64_t x_stride, const voi
 extern "C" int ck_scatter2scatter_glu_bwd(const void* DY, int64_t dy_stride, const void* W, int64_t w_stride_e,
                                           int64_t w_stride_k, int64_t w_stride_n, const int64_t* expert_offsets,
                                           const void* h, int64_t h_stride, void* d_h, int64_t d_h_stride,
-                                          int64_t num_slots, int64_t K, int64_t I, int64_t E, int dtype, void* stream) {
-    if (num_slots < 0 || K < 0 || I < 0 || E <= 0) return CK_ERR_SHAPE;
+                                          int64_t num_slots, int64_t K, int64_t I, int64_t E, int dtype, int waves,
+                                          void* stream) {
+    if (num_slots < 0 || K < 0 || I < 0 || E <= 0 || !valid_waves(waves)) return CK_ERR_SHAPE;
     if (num_slots > 0x7fffffff || K > 0x7fffffff || I > 0x3fffffff || E > 0x7fffffff) return CK_ERR_SHAPE;
     if (dtype != CK_F32 && dtype != CK_F16 && dtype != CK_BF16) return CK_ERR_DTYPE;
     if (num_slots == 0 || I == 0) return CK_OK;
@@ -1631,6 +1919,7 @@ extern "C" int ck_scatter2scatter_glu_bwd(const void* DY, int64_t dy_stride, con
         p.aux = const_cast<void*>(h);
         p.ld_aux = h_stride;
         p.glu_half = (int)I;
+        p.waves = waves;
         p.m_tiles = (int)(num_slots / kBM + E);
         p.n_tiles = (int)ck_ceil_div(I, kBN);
         if ((int64_t)(p.m_tiles + 8) * p.n_tiles > 0x7ffffff0) return CK_ERR_SHAPE;
@@ -1653,8 +1942,9 @@ extern "C" int ck_scatter2scatter_glu_bwd(const void* DY, int64_t dy_stride, con
 
 extern "C" int ck_group_bwd_W(const void* DY, int64_t dy_stride, const void* X, int64_t x_stride,
                               const int64_t* expert_offsets, void* DW, int64_t dw_stride_e, int64_t dw_stride_k,
-                              int64_t dw_stride_n, int64_t M, int64_t K, int64_t N, int64_t E, int dtype, void* stream) {
-    if (M < 0 || K < 0 || N < 0 || E <= 0) return CK_ERR_SHAPE;
+                              int64_t dw_stride_n, int64_t M, int64_t K, int64_t N, int64_t E, int dtype, int waves,
+                              void* stream) {
+    if (M < 0 || K < 0 || N < 0 || E <= 0 || !valid_waves(waves)) return CK_ERR_SHAPE;
     if (M > 0x7fffffff || K > 0x7fffffff || N > 0x7fffffff || E > 65535) return CK_ERR_SHAPE;
     if (dtype != CK_F32 && dtype != CK_F16 && dtype != CK_BF16) return CK_ERR_DTYPE;
     if (K == 0 || N == 0) return CK_OK;
@@ -1682,6 +1972,7 @@ extern "C" int ck_group_bwd_W(const void* DY, int64_t dy_stride, const void* X, 
         p.K = (int)(swap ? N : K);  // I
         p.N = (int)(swap ? K : N);  // J
         p.E = (int)E;
+        p.waves = waves;
         p.wide = 64 * p.lda * 2 >= (int64_t)1 << 32 || 64 * p.ldb * 2 >= (int64_t)1 << 32;
         p.m_tiles = (int)(E * ck_ceil_div(p.K, kBM));
         p.n_tiles = (int)ck_ceil_div(p.N, kBN);

@@ -16,4 +16,4 @@ extern "C" const char* ck_status_string(int status) {
     }
 }
 
-extern "C" int ck_abi_version(void) { return 2; }
+extern "C" int ck_abi_version(void) { return 3; }

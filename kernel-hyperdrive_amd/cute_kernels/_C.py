@@ -19,7 +19,7 @@ import torch
 _LIB_PATH = os.environ.get("CUTE_HIP_LIBRARY") or os.path.join(
     os.path.dirname(os.path.abspath(__file__)), "lib", "libcute_hip.so"
 )
-_ABI_VERSION = 2
+_ABI_VERSION = 3
 
 _lib = None
 _lock = threading.Lock()
@@ -59,20 +59,20 @@ _SIGNATURES = {
     ),
     "ck_scatter2scatter_ws": (
         _i32,
-        [_p, _i64, _p, _i64, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _p, _i32, _p,
-         _i64, _p],
+        [_p, _i64, _p, _i64, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _p, _i32, _i32,
+         _p, _i64, _p],
     ),
     "ck_scatter2scatter_workspace_size": (_i64, [_i64, _i64, _i64, _i64, _i32]),
     "ck_scatter2scatter_glu": (
         _i32,
-        [_p, _i64, _p, _i64, _i64, _i64, _p, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _p],
+        [_p, _i64, _p, _i64, _i64, _i64, _p, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _p],
     ),
     "ck_scatter2scatter_glu_bwd": (
         _i32,
-        [_p, _i64, _p, _i64, _i64, _i64, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _i64, _i32, _p],
+        [_p, _i64, _p, _i64, _i64, _i64, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _p],
     ),
     "ck_offsets_from_sorted": (_i32, [_p, _p, _i64, _i64, _p]),
-    "ck_group_bwd_W": (_i32, [_p, _i64, _p, _i64, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _p]),
+    "ck_group_bwd_W": (_i32, [_p, _i64, _p, _i64, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _p]),
     "ck_group": (_i32, [_p, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _i32, _p]),
     "ck_moe_combine_forward": (_i32, [_p, _p, _p, _i64, _i64, _i64, _i32, _p]),
     "ck_moe_combine_backward_gates": (_i32, [_p, _p, _p, _i64, _i64, _i64, _i32, _p]),
@@ -530,11 +530,21 @@ def scatter2scatter_workspace_size(num_slots: int, K: int, N: int, E: int, dtype
     return int(load_library().ck_scatter2scatter_workspace_size(num_slots, K, N, E, dtype_code(dtype)))
 
 
+GEMM_WAVES = (0, 4, 8)  # loops of the matrix-core kernel: the library's choice, four wavefronts per tile, eight
+
+
+def _waves(waves: int, what: str) -> int:
+    if waves not in GEMM_WAVES:
+        raise ValueError(f"{what}: waves must be one of {GEMM_WAVES}, got {waves!r}")
+    return int(waves)
+
+
 def scatter2scatter(X, W, sorted_scattered_idxs, expert_offsets, out, fan_out: int, x_grouped: bool,
-                    y_grouped: bool, workspace=None, bias=None) -> None:
+                    y_grouped: bool, workspace=None, bias=None, waves: int = 0) -> None:
     """X [*, K] (unit column stride), W strided view [E, K, N], out [slots, N] (unit column stride); ``workspace``:
     uint8 tensor of ``scatter2scatter_workspace_size`` bytes or None; ``bias``: [E, N] contiguous or None, added to
-    every row of its expert before the row is rounded."""
+    every row of its expert before the row is rounded; ``waves``: the loop of the matrix-core kernel (``GEMM_WAVES``)."""
+    waves = _waves(waves, "scatter2scatter")
     lib = load_library()
     if X.stride(1) != 1 or out.stride(1) != 1:
         raise ValueError("scatter2scatter needs unit column stride for X and out")
@@ -553,15 +563,17 @@ def scatter2scatter(X, W, sorted_scattered_idxs, expert_offsets, out, fan_out: i
             lib.ck_scatter2scatter_ws(_ptr(X), X.stride(0), _ptr(W), W.stride(0), W.stride(1), W.stride(2),
                                       _ptr(sorted_scattered_idxs), _ptr(expert_offsets), _ptr(out), out.stride(0),
                                       out.size(0), X.size(1), out.size(1), W.size(0), fan_out, int(x_grouped),
-                                      int(y_grouped), _ptr(bias), dtype_code(X.dtype), _ptr(workspace), ws_bytes,
+                                      int(y_grouped), _ptr(bias), dtype_code(X.dtype), waves, _ptr(workspace), ws_bytes,
                                       L.stream),
             "ck_scatter2scatter_ws",
         )
 
 
-def scatter2scatter_glu(X, W, sorted_scattered_idxs, expert_offsets, h, act, fan_out: int, x_grouped: bool) -> None:
+def scatter2scatter_glu(X, W, sorted_scattered_idxs, expert_offsets, h, act, fan_out: int, x_grouped: bool,
+                        waves: int = 0) -> None:
     """h [slots, 2I] = gathered X rows times W [E, K, 2I], act [slots, I] = SwiGLU(h); rows grouped by expert."""
     lib = load_library()
+    waves = _waves(waves, "scatter2scatter_glu")
     if X.stride(1) != 1 or h.stride(1) != 1 or act.stride(1) != 1:
         raise ValueError("scatter2scatter_glu needs unit column stride for X, h and act")
     if h.size(1) != 2 * act.size(1) or h.size(0) != act.size(0):
@@ -578,14 +590,15 @@ def scatter2scatter_glu(X, W, sorted_scattered_idxs, expert_offsets, h, act, fan
             lib.ck_scatter2scatter_glu(_ptr(X), X.stride(0), _ptr(W), W.stride(0), W.stride(1), W.stride(2),
                                        _ptr(sorted_scattered_idxs), _ptr(expert_offsets), _ptr(h), h.stride(0),
                                        _ptr(act), act.stride(0), h.size(0), X.size(1), act.size(1), W.size(0),
-                                       fan_out, int(x_grouped), dtype_code(X.dtype), L.stream),
+                                       fan_out, int(x_grouped), dtype_code(X.dtype), waves, L.stream),
             "ck_scatter2scatter_glu",
         )
 
 
-def scatter2scatter_glu_bwd(DY, W, expert_offsets, h, d_h) -> None:
+def scatter2scatter_glu_bwd(DY, W, expert_offsets, h, d_h, waves: int = 0) -> None:
     """d_h [slots, 2I] = SwiGLU'(h) applied to DY [slots, K] times W [E, K, I]; all rows grouped by expert."""
     lib = load_library()
+    waves = _waves(waves, "scatter2scatter_glu_bwd")
     if DY.stride(1) != 1 or h.stride(1) != 1 or d_h.stride(1) != 1:
         raise ValueError("scatter2scatter_glu_bwd needs unit column stride for DY, h and d_h")
     if h.shape != d_h.shape or h.size(1) != 2 * W.size(2) or h.size(0) != DY.size(0):
@@ -599,13 +612,15 @@ def scatter2scatter_glu_bwd(DY, W, expert_offsets, h, d_h) -> None:
         _check(
             lib.ck_scatter2scatter_glu_bwd(_ptr(DY), DY.stride(0), _ptr(W), W.stride(0), W.stride(1), W.stride(2),
                                            _ptr(expert_offsets), _ptr(h), h.stride(0), _ptr(d_h), d_h.stride(0),
-                                           DY.size(0), DY.size(1), W.size(2), W.size(0), dtype_code(DY.dtype), L.stream),
+                                           DY.size(0), DY.size(1), W.size(2), W.size(0), dtype_code(DY.dtype), waves,
+                                           L.stream),
             "ck_scatter2scatter_glu_bwd",
         )
 
 
-def group_bwd_W(DY, X, expert_offsets, DW, E: int) -> None:
+def group_bwd_W(DY, X, expert_offsets, DW, E: int, waves: int = 0) -> None:
     lib = load_library()
+    waves = _waves(waves, "group_bwd_W")
     if X.stride(1) != 1 or DY.stride(1) != 1:
         raise ValueError("group_bwd_W needs unit column stride for X and DY")
     _same_dtype(X, "group_bwd_W", DY=DY, DW=DW)
@@ -617,7 +632,7 @@ def group_bwd_W(DY, X, expert_offsets, DW, E: int) -> None:
         _check(
             lib.ck_group_bwd_W(_ptr(DY), DY.stride(0), _ptr(X), X.stride(0), _ptr(expert_offsets), _ptr(DW),
                                DW.stride(0), DW.stride(1), DW.stride(2), X.size(0), X.size(1), DY.size(1), E,
-                               dtype_code(X.dtype), L.stream),
+                               dtype_code(X.dtype), waves, L.stream),
             "ck_group_bwd_W",
         )
 

@@ -124,6 +124,10 @@ class _CutoTune:
     def _merge(self, config: CutoTuneConfig, named: dict, caller_wins: bool) -> dict:
         merged = dict(named)
         if not caller_wins:
+            # a cached configuration written before a tunable argument existed takes the default for that argument
+            for name, value in self.default_config.get_key_values().items():
+                if name in self.tunable and name not in config.get_key_values():
+                    merged[name] = value
             for name, value in config.get_key_values().items():
                 merged[name] = value
         return merged

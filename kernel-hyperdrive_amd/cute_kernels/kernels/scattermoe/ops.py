@@ -23,6 +23,8 @@ epilogues of the grouped GEMMs that produce their inputs, so neither the activat
 separate trip through memory.  Every value is rounded where the separate ops round it.
 """
 
+import os
+
 import torch
 
 from ... import _C
@@ -39,13 +41,37 @@ torch._dynamo.config.capture_scalar_outputs = True
 SPLIT_TILE_TAIL: bool | None = None
 
 
+# The loop of the matrix-core kernel (`waves` of the C entry points): 8 = eight wavefronts per 256 x 256 tile, two per
+# SIMD in antiphase; 4 = four wavefronts, one per SIMD, a software pipeline over 128 x 128 blocks with the accumulators
+# in the accumulation registers (a third less LDS traffic per step).  The counterpart of num_warps / num_stages in the
+# reference's tuned configurations (triton_implementation/kernels.py:152-159).  The tuner ranks the loops named here
+# per product shape; the four-wave loop joins them through CUTE_GEMM_WAVES_CANDIDATES="8,4" (it is compiled into the
+# library, and stays out of the default candidates until it has been timed against the other on an MI355X).
+def _gemm_waves_candidates() -> list[int]:
+    named = [int(w) for w in os.environ.get("CUTE_GEMM_WAVES_CANDIDATES", "8").split(",") if w.strip()]
+    assert named and all(w in (4, 8) for w in named), "CUTE_GEMM_WAVES_CANDIDATES names 4 and / or 8"
+    return named
+
+
+GEMM_WAVES_CANDIDATES = _gemm_waves_candidates()
+_GEMM_TRIGGERS = {"X.dtype", "X.size(1)", "W.size(0)"}
+
+
 # The reference tunes the tile of its grouped products per shape (triton_implementation/kernels.py:152-159, BLOCK_M of
-# groupXtY); the choice that moves these kernels is how the last, partly filled round of tiles is run: whole tiles
-# (the CUs without one idle for a tile time) or cut along the contraction over the idle CUs and summed by a second
-# launch (a few per cent either way, depending on how full the last round is and how long the contraction).
+# groupXtY); the choices that move these kernels are the loop (above) and how the last, partly filled round of tiles
+# is run: whole tiles (the CUs without one idle for a tile time) or cut along the contraction over the idle CUs and
+# summed by a second launch (a few per cent either way, depending on how full the last round is and how long the
+# contraction).
+def _has_tail_to_split(X, W, out, split_tile_tail, **_) -> bool:
+    # a candidate that splits is a candidate only where the library would split
+    return not split_tile_tail or _C.scatter2scatter_workspace_size(out.size(0), X.size(1), out.size(1), W.size(0), X.dtype) > 0
+
+
 @cutotune(
-    configs=get_cartesian_product_cutotune_configs(split_tile_tail=[True, False]),
-    default_config=CutoTuneConfig({"split_tile_tail": True}),
+    configs=get_cartesian_product_cutotune_configs(
+        condition=_has_tail_to_split, split_tile_tail=[True, False], waves=GEMM_WAVES_CANDIDATES
+    ),
+    default_config=CutoTuneConfig({"split_tile_tail": True, "waves": 0}),
     triggers={"X.dtype", "X.size(1)", "out.size(1)", "W.size(0)"},
     functional_triggers={"rows_log2": lambda **kwargs: int(kwargs["out"].size(0)).bit_length()},
 )
@@ -60,6 +86,7 @@ def scatter2scatter_launch(
     y_grouped: bool,
     bias: torch.Tensor | None,
     split_tile_tail: bool,
+    waves: int,
 ) -> None:
     workspace = None
     if split_tile_tail:
@@ -68,7 +95,43 @@ def scatter2scatter_launch(
         if nbytes > 0:
             workspace = torch.empty(nbytes, dtype=torch.uint8, device=X.device)
     _C.scatter2scatter(X, W, sorted_scattered_idxs, expert_offsets, out, FAN_OUT, x_grouped, y_grouped, workspace,
-                       bias)
+                       bias, waves)
+
+
+def _rows_log2(name: str):
+    return lambda **kwargs: int(kwargs[name].size(0)).bit_length()
+
+
+@cutotune(
+    configs=get_cartesian_product_cutotune_configs(waves=GEMM_WAVES_CANDIDATES),
+    default_config=CutoTuneConfig({"waves": 0}),
+    triggers=_GEMM_TRIGGERS | {"h.size(1)"},
+    functional_triggers={"rows_log2": _rows_log2("h")},
+)
+def scatter2scatter_glu_launch(X, W, sorted_scattered_idxs, expert_offsets, h, act, FAN_OUT: int, x_grouped: bool,
+                               waves: int) -> None:
+    _C.scatter2scatter_glu(X, W, sorted_scattered_idxs, expert_offsets, h, act, FAN_OUT, x_grouped, waves)
+
+
+@cutotune(
+    configs=get_cartesian_product_cutotune_configs(waves=GEMM_WAVES_CANDIDATES),
+    default_config=CutoTuneConfig({"waves": 0}),
+    triggers={"DY.dtype", "DY.size(1)", "W.size(0)", "h.size(1)"},
+    functional_triggers={"rows_log2": _rows_log2("h")},
+)
+def scatter2scatter_glu_bwd_launch(DY, W, expert_offsets, h, d_h, waves: int) -> None:
+    _C.scatter2scatter_glu_bwd(DY, W, expert_offsets, h, d_h, waves)
+
+
+# the reference tunes this product over BLOCK_M and num_stages (triton_implementation/kernels.py:152-159)
+@cutotune(
+    configs=get_cartesian_product_cutotune_configs(waves=GEMM_WAVES_CANDIDATES),
+    default_config=CutoTuneConfig({"waves": 0}),
+    triggers={"X.dtype", "X.size(1)", "DY.size(1)", "DW.size(0)"},
+    functional_triggers={"rows_log2": _rows_log2("X")},
+)
+def group_bwd_W_launch(DY, X, expert_offsets, DW, E: int, waves: int) -> None:
+    _C.group_bwd_W(DY, X, expert_offsets, DW, E, waves)
 
 
 @cute_op(f"{LIBRARY_NAME}::scatter2scatter", mutates_args={"out"})
@@ -95,17 +158,20 @@ def scatter2scatter(
         _C.offsets_from_sorted(sorted_expert_idxs.contiguous(), expert_offsets)
     if X.stride(1) != 1:
         X = X.contiguous()
-    # only long contractions over few column tiles have a tail worth splitting; everything else has one form
+    # only long contractions over few column tiles have a tail worth splitting; with one loop to choose from, every
+    # other product has a single form and does not go through the tuner
     eligible = _C.scatter2scatter_workspace_size(out.size(0), X.size(1), out.size(1), W.size(0), X.dtype) > 0
-    if not eligible:
+    if SPLIT_TILE_TAIL is not None:
+        choice = SPLIT_TILE_TAIL and eligible
+    elif not eligible and len(GEMM_WAVES_CANDIDATES) == 1:
         choice = False
-    elif SPLIT_TILE_TAIL is None:
-        choice = CutoTuneParameter()
     else:
-        choice = SPLIT_TILE_TAIL
+        choice = CutoTuneParameter()
+    # the caller fixes both tunable arguments or neither: a fixed form of the tail takes the library's choice of loop
+    waves = CutoTuneParameter() if isinstance(choice, CutoTuneParameter) else 0
     scatter2scatter_launch(X=X, W=W, sorted_scattered_idxs=sorted_scattered_idxs, expert_offsets=expert_offsets,
                            out=out, FAN_OUT=FAN_OUT, x_grouped=x_grouped, y_grouped=y_grouped, bias=bias,
-                           split_tile_tail=choice)
+                           split_tile_tail=choice, waves=waves)
 
 
 @cute_op(f"{LIBRARY_NAME}::scatter2scatter_glu", mutates_args={"h", "act"})
@@ -126,7 +192,8 @@ def scatter2scatter_glu(
     assert X.size(1) == W.size(1)
     if X.stride(1) != 1:
         X = X.contiguous()
-    _C.scatter2scatter_glu(X, W, sorted_scattered_idxs, expert_offsets, h, act, FAN_OUT, x_grouped)
+    scatter2scatter_glu_launch(X=X, W=W, sorted_scattered_idxs=sorted_scattered_idxs, expert_offsets=expert_offsets,
+                               h=h, act=act, FAN_OUT=FAN_OUT, x_grouped=x_grouped, waves=CutoTuneParameter())
 
 
 @cute_op(f"{LIBRARY_NAME}::scatter2scatter_glu_bwd", mutates_args={"d_h"})
@@ -138,7 +205,7 @@ def scatter2scatter_glu_bwd(
     assert h.shape == d_h.shape and h.size(1) == 2 * W.size(2)
     if DY.stride(1) != 1:
         DY = DY.contiguous()
-    _C.scatter2scatter_glu_bwd(DY, W, expert_offsets, h, d_h)
+    scatter2scatter_glu_bwd_launch(DY=DY, W=W, expert_offsets=expert_offsets, h=h, d_h=d_h, waves=CutoTuneParameter())
 
 
 @cute_op(f"{LIBRARY_NAME}::group_bwd_W", mutates_args={"DW"})
@@ -149,7 +216,7 @@ def group_bwd_W(DY: torch.Tensor, X: torch.Tensor, expert_offsets: torch.Tensor,
         DY = DY.contiguous()
     if X.stride(1) != 1:
         X = X.contiguous()
-    _C.group_bwd_W(DY, X, expert_offsets, DW, E)
+    group_bwd_W_launch(DY=DY, X=X, expert_offsets=expert_offsets, DW=DW, E=E, waves=CutoTuneParameter())
 
 
 @cute_op(f"{LIBRARY_NAME}::group", mutates_args={"out"})

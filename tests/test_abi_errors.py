@@ -120,32 +120,42 @@ def test_grouped_gemm_argument_checks(lib):
     assert need > 0
     assert lib.ck_scatter2scatter_workspace_size(1024, 1024, 256, 4, BF16) == 0  # contraction too short to cut
     assert lib.ck_scatter2scatter_workspace_size(1024, 8192, 256, 4, F32) == 0
-    #       X  ldx   W  se          sk sn    idx off out ldo slots K     N    E  fan xg yg bias dtype ws  bytes stream
-    assert ws(P, 8192, P, 8192 * 256, 1, 8192, P, P, P, 256, 1024, 8192, 256, 4, 1, 0, 1, None, BF16, P, need - 1, None) == WORKSPACE
-    assert ws(P, 8192, P, 8192 * 256, 1, 8192, P, P, P, 256, 1024, 8192, 256, 4, 1, 0, 1, None, BF16, P + 4, need, None) == WORKSPACE
-    assert ws(P, 8192, P, 8192 * 256, 1, 8192, P, None, P, 256, 1024, 8192, 256, 4, 1, 0, 1, None, BF16, P, need, None) == NULL
-    assert ws(P, 8192, P, 8192 * 256, 1, 8192, P, P, P, 256, 0, 8192, 256, 4, 1, 0, 1, None, BF16, P, need, None) == OK  # no rows
+    #       X  ldx   W  se          sk sn    idx off out ldo slots K     N    E  fan xg yg bias dtype waves ws  bytes stream
+    assert ws(P, 8192, P, 8192 * 256, 1, 8192, P, P, P, 256, 1024, 8192, 256, 4, 1, 0, 1, None, BF16, 0, P, need - 1, None) == WORKSPACE
+    assert ws(P, 8192, P, 8192 * 256, 1, 8192, P, P, P, 256, 1024, 8192, 256, 4, 1, 0, 1, None, BF16, 0, P + 4, need, None) == WORKSPACE
+    assert ws(P, 8192, P, 8192 * 256, 1, 8192, P, None, P, 256, 1024, 8192, 256, 4, 1, 0, 1, None, BF16, 0, P, need, None) == NULL
+    assert ws(P, 8192, P, 8192 * 256, 1, 8192, P, P, P, 256, 0, 8192, 256, 4, 1, 0, 1, None, BF16, 0, P, need, None) == OK  # no rows
     glu = lib.ck_scatter2scatter_glu
-    #        X  ldx W  se    sk sn idx off h  ldh  act lda slots K  I  E  fan xg dtype stream
-    assert glu(P, 64, P, 8192, 1, 64, P, P, P, 128, P, 64, 16, 64, 64, 0, 1, 0, BF16, None) == SHAPE  # E = 0
-    assert glu(P, 64, P, 8192, 1, 64, P, P, P, 128, None, 64, 16, 64, 64, 2, 1, 0, BF16, None) == NULL  # no act
-    assert glu(P, 64, P, 8192, 1, 64, None, P, P, 128, P, 64, 16, 64, 64, 2, 1, 0, BF16, None) == NULL  # gather without index
-    assert glu(P, 64, P, 8192, 1, 64, P, P, P, 128, P, 64, 16, 64, 64, 2, 1, 0, 8, None) == DTYPE
-    assert glu(P, 64, P, 8192, 1, 64, P, P, P, 128, P + 1, 64, 16, 64, 64, 2, 1, 0, BF16, None) == ALIGN
-    assert glu(P, 64, P, 8192, 1, 64, P, P, P, 128, P, 64, 0, 64, 64, 2, 1, 0, BF16, None) == OK  # no rows
+    #        X  ldx W  se    sk sn idx off h  ldh  act lda slots K  I  E  fan xg dtype waves stream
+    assert glu(P, 64, P, 8192, 1, 64, P, P, P, 128, P, 64, 16, 64, 64, 0, 1, 0, BF16, 0, None) == SHAPE  # E = 0
+    assert glu(P, 64, P, 8192, 1, 64, P, P, P, 128, None, 64, 16, 64, 64, 2, 1, 0, BF16, 0, None) == NULL  # no act
+    assert glu(P, 64, P, 8192, 1, 64, None, P, P, 128, P, 64, 16, 64, 64, 2, 1, 0, BF16, 0, None) == NULL  # gather without index
+    assert glu(P, 64, P, 8192, 1, 64, P, P, P, 128, P, 64, 16, 64, 64, 2, 1, 0, 8, 0, None) == DTYPE
+    assert glu(P, 64, P, 8192, 1, 64, P, P, P, 128, P + 1, 64, 16, 64, 64, 2, 1, 0, BF16, 0, None) == ALIGN
+    assert glu(P, 64, P, 8192, 1, 64, P, P, P, 128, P, 64, 0, 64, 64, 2, 1, 0, BF16, 0, None) == OK  # no rows
     glu_bwd = lib.ck_scatter2scatter_glu_bwd
-    #            DY ldy W  se    sk  sn off h  ldh  d_h ldd slots K  I  E  dtype stream
-    assert glu_bwd(P, 64, P, 4096, 64, 1, P, P, 128, P, 128, 16, 64, 64, 0, BF16, None) == SHAPE
-    assert glu_bwd(P, 64, P, 4096, 64, 1, P, None, 128, P, 128, 16, 64, 64, 2, BF16, None) == NULL  # no h
-    assert glu_bwd(P, 64, P, 4096, 64, 1, None, P, 128, P, 128, 16, 64, 64, 2, BF16, None) == NULL  # no offsets
-    assert glu_bwd(P, 64, P, 4096, 64, 1, P, P, 128, P, 128, 16, 64, 64, 2, 5, None) == DTYPE
-    assert glu_bwd(P, 64, P, 4096, 64, 1, P, P, 128, P, 128, 16, 64, 0, 2, BF16, None) == OK  # I = 0
+    #            DY ldy W  se    sk  sn off h  ldh  d_h ldd slots K  I  E  dtype waves stream
+    assert glu_bwd(P, 64, P, 4096, 64, 1, P, P, 128, P, 128, 16, 64, 64, 0, BF16, 0, None) == SHAPE
+    assert glu_bwd(P, 64, P, 4096, 64, 1, P, None, 128, P, 128, 16, 64, 64, 2, BF16, 0, None) == NULL  # no h
+    assert glu_bwd(P, 64, P, 4096, 64, 1, None, P, 128, P, 128, 16, 64, 64, 2, BF16, 0, None) == NULL  # no offsets
+    assert glu_bwd(P, 64, P, 4096, 64, 1, P, P, 128, P, 128, 16, 64, 64, 2, 5, 0, None) == DTYPE
+    assert glu_bwd(P, 64, P, 4096, 64, 1, P, P, 128, P, 128, 16, 64, 0, 2, BF16, 0, None) == OK  # I = 0
     xty = lib.ck_group_bwd_W
-    #        DY ldy X  ldx off DW se    sk  sn M   K   N   E  dtype stream
-    assert xty(P, 64, P, 64, P, P, 4096, 64, 1, 16, 64, 64, 0, BF16, None) == SHAPE
-    assert xty(P, 64, P, 64, P, None, 4096, 64, 1, 16, 64, 64, 2, BF16, None) == NULL
-    assert xty(P, 64, P, 64, None, P, 4096, 64, 1, 16, 64, 64, 2, BF16, None) == NULL
-    assert xty(P, 64, P, 64, P, P, 4096, 64, 1, 16, 64, 64, 2, 4, None) == DTYPE
+    #        DY ldy X  ldx off DW se    sk  sn M   K   N   E  dtype waves stream
+    assert xty(P, 64, P, 64, P, P, 4096, 64, 1, 16, 64, 64, 0, BF16, 0, None) == SHAPE
+    assert xty(P, 64, P, 64, P, None, 4096, 64, 1, 16, 64, 64, 2, BF16, 0, None) == NULL
+    assert xty(P, 64, P, 64, None, P, 4096, 64, 1, 16, 64, 64, 2, BF16, 0, None) == NULL
+    assert xty(P, 64, P, 64, P, P, 4096, 64, 1, 16, 64, 64, 2, 4, 0, None) == DTYPE
+    # the loop of the matrix-core kernel: 0 (the library's choice), 4 or 8 wavefronts per tile, nothing else
+    assert xty(P, 64, P, 64, P, P, 4096, 64, 1, 16, 64, 64, 2, BF16, 2, None) == SHAPE
+    assert glu_bwd(P, 64, P, 4096, 64, 1, P, P, 128, P, 128, 16, 64, 64, 2, BF16, 16, None) == SHAPE
+    assert glu(P, 64, P, 8192, 1, 64, P, P, P, 128, P, 64, 16, 64, 64, 2, 1, 0, BF16, -4, None) == SHAPE
+    assert ws(P, 8192, P, 8192 * 256, 1, 8192, P, P, P, 256, 1024, 8192, 256, 4, 1, 0, 1, None, BF16, 6, P, need, None) == SHAPE
+    for waves in (4, 8):  # accepted: with nothing to do the call returns before any launch
+        assert xty(P, 64, P, 64, P, P, 4096, 64, 1, 16, 0, 64, 2, BF16, waves, None) == OK
+        assert glu_bwd(P, 64, P, 4096, 64, 1, P, P, 128, P, 128, 16, 64, 0, 2, BF16, waves, None) == OK
+        assert glu(P, 64, P, 8192, 1, 64, P, P, P, 128, P, 64, 0, 64, 64, 2, 1, 0, BF16, waves, None) == OK
+        assert ws(P, 8192, P, 8192 * 256, 1, 8192, P, P, P, 256, 0, 8192, 256, 4, 1, 0, 1, None, BF16, waves, P, need, None) == OK
     assert lib.ck_group(None, 64, P, None, P, 64, 16, 64, 1, BF16, None) == NULL
     assert lib.ck_group(P, 64, P, None, P, 64, 16, 64, 0, BF16, None) == SHAPE
     assert lib.ck_moe_combine_forward(P, P, P, 16, 0, 64, BF16, None) == SHAPE  # k = 0

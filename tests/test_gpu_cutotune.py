@@ -117,9 +117,11 @@ def test_scatter2scatter_launches_the_cached_choice(monkeypatch, K):
     seen = {}
     real = _C.scatter2scatter
 
-    def spy(X, W, idx, offsets, out, fan_out, x_grouped, y_grouped, workspace=None, bias=None):
+    def spy(X, W, idx, offsets, out, fan_out, x_grouped, y_grouped, workspace=None, bias=None, waves=0):
         seen["split"] = workspace is not None
-        return real(X, W, idx, offsets, out, fan_out, x_grouped, y_grouped, workspace, bias)
+        # the cache was written with the eight-wave loop as the only candidate: such an entry takes the default
+        assert waves == 0
+        return real(X, W, idx, offsets, out, fan_out, x_grouped, y_grouped, workspace, bias, waves)
 
     monkeypatch.setattr(_C, "scatter2scatter", spy)
     assert ops.SPLIT_TILE_TAIL is None, "the tuner decides unless somebody fixed the choice"
