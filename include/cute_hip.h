@@ -75,8 +75,8 @@ int ck_swiglu_unchunked_backward(const void* x, const void* output_grad, void* x
  * H must be <= 65536 (the reference's MAX_TRITON_BLOCK_SIZE limit, rmsnorm/forward.py:31-32).
  * block_size_b is the reference's tunable BLOCK_SIZE_B (rows per program, kernels_forward.py:63-107,
  * kernels_backward.py:177-228), here the launch variant for rows that one wavefront holds (up to 512 packets of 16
- * bytes: 4096 16-bit elements): forward 1, 2, 4 = rows a wave requests at once before it ends, 8 or more = waves that
- * walk rows with the next row in flight; backward 1 = two workgroups per compute unit without a row in flight,
+ * bytes: 4096 16-bit elements): forward 1, 2 = rows a wave requests at once before it ends (3 .. 7 are the launch of
+ * 2), 8 or more = waves that walk rows with the next row in flight; backward 1 = two workgroups per compute unit without a row in flight,
  * 2 or more = one workgroup per compute unit with.  0 = the library's default.  Every variant gives the same values.
  * ------------------------------------------------------------------------------------------- */
 int ck_rmsnorm_forward(const void* x, const void* weight, void* output, float* rstd, int64_t B, int64_t H,

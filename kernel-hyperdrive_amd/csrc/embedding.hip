@@ -17,7 +17,8 @@
 //                  token position.  A run that fits one chunk is rounded and stored straight into dW; longer
 //                  runs leave one fp32 partial row per chunk in the workspace.
 //               3. combine kernel: sums the partial rows of each long run and stores the dW row.
-//             No floating-point atomics, no zero-fill of rows that are written anyway, deterministic.
+//             No floating-point atomics, deterministic.  Of the rows that receive a sum, only those inside the two
+//             ranges cleared before the marks exist are written twice.
 #include "ck_block_sort.h"
 #include "ck_grid_sort.h"
 

@@ -4,8 +4,8 @@ Public function and autograd signature follow cute_kernels/kernels/rmsnorm/__ini
 ``eps=None`` -> ``torch.finfo(dtype).eps``, optional weight, ``memory_efficient`` recomputation of 1/rms).
 BLOCK_SIZE_B (the reference's rows per program, tuned per dtype, row length and presence of a weight,
 kernels_forward.py:63-107 and kernels_backward.py:177-228) selects the launch variant of the kernels for rows that
-one wavefront holds: forward 1, 2, 4 rows requested at once by a wave that then ends, 8 waves that walk rows with
-the next one in flight; backward 1 two workgroups per compute unit, 2 one workgroup with the next row in flight.
+one wavefront holds: forward 1 or 2 rows requested at once by a wave that then ends (3 .. 7 are the launch of 2), 8
+waves that walk rows with the next one in flight; backward 1 two workgroups per compute unit, 2 one workgroup with the next row in flight.
 Every variant gives the same values; the tuner picks per (dtype, row length, weight).  BLOCK_SIZE_H is accepted for
 call compatibility: a row is always held whole.
 """
@@ -59,7 +59,7 @@ def rmsnorm_backward_hip(
 
 
 # launch variants (see the module docstring)
-FORWARD_ROWS = [1, 2, 4, 8]
+FORWARD_ROWS = [1, 2, 8]  # distinct launches only: 3 .. 7 would time the launch of 2 again
 BACKWARD_VARIANTS = [1, 2]
 # the reference's cache keys: dtype, row length, presence of a weight (kernels_forward.py:63-76)
 _TRIGGERS = {"x.dtype", "x.size(-1)"}
