@@ -50,6 +50,9 @@ def gemm_hbm_bytes_per_launch():
     return float(found[-1]) if found else None
 
 
+LOOP_PRODUCTS = ("fwd_c_fc", "fwd_c_proj", "dx_c_proj", "dx_c_fc", "dw_c_proj", "dw_c_fc")  # --loop-product
+
+
 def parse_args():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
@@ -63,6 +66,13 @@ def parse_args():
     p.add_argument("--yardstick", action="store_true",
                    help="also time the vendor library's dense bf16 kernels on the six products (extras.dense_yardstick)")
     p.add_argument("--only-yardstick", action="store_true", help="only that leg (for a kernel trace)")
+    p.add_argument("--only-skewed", action="store_true",
+                   help="only the fine-grained skewed MoE step (extras.moe_fine_grained_skewed), for a kernel trace of it")
+    p.add_argument("--loop-product", choices=sorted(LOOP_PRODUCTS), default=None,
+                   help="run ONE grouped product of the Mixtral step back to back for --loop-seconds and print its rate "
+                        "(a steady load to read socket power and clocks beside, e.g. with amd-smi)")
+    p.add_argument("--loop-seconds", type=float, default=8.0)
+    p.add_argument("--zeros", action="store_true", help="with --loop-product: all-zero operands (no switching activity)")
     p.add_argument("--tokens", type=int, default=8192, help="T of the MoE workload (default: the BASELINE shape)")
     p.add_argument("--copy-calibration", action="store_true",
                    help="also run three 1 GiB device copies before the steps (a kernel of known HBM traffic, to scale "
@@ -307,6 +317,57 @@ def bench_extras(device, embedding_ids="both"):
     return out
 
 
+# ---- one product in a loop ---------------------------------------------------------------------------------
+def bench_loop_product(device, name, seconds, zeros):
+    """One grouped product of the Mixtral step (T=8192 top-2 over 8 experts, random routing, bf16), launched back to
+    back for `seconds`: a steady load for reading socket power and clocks from outside, and its rate."""
+    from cute_kernels import _C
+    from cute_kernels.kernels.scattermoe import moe_sort
+
+    T, H, I, E, k = 8192, 4096, 14336, 8, 2
+    M = T * k
+    dtype = torch.bfloat16
+    g = torch.Generator(device=device).manual_seed(0)
+    selected = torch.stack([torch.randperm(E, generator=g, device=device)[:k] for _ in range(T)])
+    _, s_idx, off = moe_sort(selected, E)
+
+    def rnd(*shape, std=1.0):
+        t = torch.randn(*shape, generator=g, device=device, dtype=torch.float32).mul_(std).to(dtype)
+        return t.zero_() if zeros else t
+
+    if name == "fwd_c_fc":
+        x, w, out = rnd(T, H), rnd(E, 2 * I, H, std=0.02), torch.empty(M, 2 * I, device=device, dtype=dtype)
+        fn, flop = (lambda: _C.scatter2scatter(x, w.permute(0, 2, 1), s_idx, off, out, k, False, True)), 2.0 * M * H * 2 * I
+    elif name == "fwd_c_proj":
+        x, w, out = rnd(M, I), rnd(E, H, I, std=0.02), torch.empty(M, H, device=device, dtype=dtype)
+        fn, flop = (lambda: _C.scatter2scatter(x, w.permute(0, 2, 1), s_idx, off, out, 1, True, False)), 2.0 * M * H * I
+    elif name == "dx_c_proj":
+        x, w, out = rnd(M, H), rnd(E, H, I, std=0.02), torch.empty(M, I, device=device, dtype=dtype)
+        fn, flop = (lambda: _C.scatter2scatter(x, w, s_idx, off, out, 1, True, True)), 2.0 * M * H * I
+    elif name == "dx_c_fc":
+        x, w, out = rnd(M, 2 * I), rnd(E, 2 * I, H, std=0.02), torch.empty(M, H, device=device, dtype=dtype)
+        fn, flop = (lambda: _C.scatter2scatter(x, w, s_idx, off, out, 1, True, False)), 2.0 * M * H * 2 * I
+    elif name == "dw_c_proj":
+        dy, x, dw = rnd(M, H), rnd(M, I), torch.empty(E, H, I, device=device, dtype=dtype)
+        fn, flop = (lambda: _C.group_bwd_W(dy, x, off, dw.permute(0, 2, 1), E)), 2.0 * M * H * I
+    else:
+        dy, x, dw = rnd(M, 2 * I), rnd(M, H), torch.empty(E, 2 * I, H, device=device, dtype=dtype)
+        fn, flop = (lambda: _C.group_bwd_W(dy, x, off, dw.permute(0, 2, 1), E)), 2.0 * M * H * 2 * I
+    for _ in range(3):
+        fn()
+    torch.cuda.synchronize()
+    t0, launches = time.perf_counter(), 0
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
+        launches += 20
+    elapsed = time.perf_counter() - t0
+    tflops = flop * launches / elapsed / 1e12
+    return {"product": name, "operands": "zeros" if zeros else "random", "launches": launches, "seconds": round(elapsed, 2),
+            "TFLOP/s": round(tflops, 1), "frac_of_mfma_peak": round(tflops / BF16_MFMA_PEAK_TFLOPS, 4)}
+
+
 # ---- dense yardstick --------------------------------------------------------------------------------------
 def bench_dense_yardstick(device, iters=5, warmup=2):
     """What the vendor library's dense bf16 kernels reach on this box, under the same power cap, on the six products
@@ -433,6 +494,12 @@ def main():
         copy_calibration(device)
     if args.only_extras:
         print(json.dumps({"extras": bench_extras(device, args.embedding_ids)}))
+        return
+    if args.only_skewed:
+        print(json.dumps({"extras": {"moe_fine_grained_skewed": bench_moe_skewed(device)}}))
+        return
+    if args.loop_product:
+        print(json.dumps({"loop_product": bench_loop_product(device, args.loop_product, args.loop_seconds, args.zeros)}))
         return
     if args.only_yardstick:
         print(json.dumps({"extras": {"dense_yardstick": bench_dense_yardstick(device)}}))

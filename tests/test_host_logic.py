@@ -344,6 +344,67 @@ def test_shipped_tuning_cache_loads_and_covers_the_tuned_launchers():
     assert all(len(entries) >= 2 for entries in sw.values()), "every candidate's timing is kept"
 
 
+def test_grouped_product_launchers_pass_the_loop_and_the_tail_choice_on(monkeypatch):
+    """The tuned launchers of the grouped products hand the binding the loop (`waves`) and, for scatter2scatter, the
+    workspace of the split tail: the cached choice where the cache has the key (a cache written before the loop was
+    tunable names no loop: the library's choice, 0), one fixed form where only one exists, and what a caller fixes.
+    The binding is replaced by a recorder, so nothing is launched."""
+    import torch
+
+    from cute_kernels import _C
+    from cute_kernels.cutotune import CutoTuneConfig
+    from cute_kernels.kernels.scattermoe import ops
+
+    calls = []
+    eligible = {"yes": True}
+    monkeypatch.setattr(_C, "scatter2scatter_workspace_size", lambda slots, K, N, E, dtype: 64 if eligible["yes"] and K >= 4096 else 0)
+    monkeypatch.setattr(_C, "scatter2scatter", lambda *a: calls.append(("s2s", a[8] is not None, a[10])))
+    monkeypatch.setattr(_C, "scatter2scatter_glu", lambda *a: calls.append(("glu", a[8])))
+    monkeypatch.setattr(_C, "scatter2scatter_glu_bwd", lambda *a: calls.append(("glu_bwd", a[5])))
+    monkeypatch.setattr(_C, "group_bwd_W", lambda *a: calls.append(("dw", a[5])))
+    monkeypatch.setattr(torch, "empty", lambda *a, **k: torch.zeros(*a, **{**k, "device": "cpu"}))
+    assert ops.GEMM_WAVES_CANDIDATES == [8], "the default candidates are the loop that has been measured"
+
+    E, M, K, N = 4, 64, 4096, 256
+    X = torch.zeros(M, K, dtype=torch.bfloat16)
+    W = torch.zeros(E, K, N, dtype=torch.bfloat16)
+    out = torch.zeros(M, N, dtype=torch.bfloat16)
+    idx = torch.arange(M)
+    off = torch.tensor([16, 32, 48, 64])
+    tuner = ops.scatter2scatter_launch.tuner
+    key = tuner._lookup_key(dict(X=X, W=W, out=out))
+    # (a) a cached entry from before the loop was tunable: its tail choice, the library's loop
+    monkeypatch.setitem(tuner.best_configs, key, (CutoTuneConfig({"split_tile_tail": False}), 1.0))
+    ops.scatter2scatter(X, W, idx, idx, out, 1, True, True, off)
+    assert calls.pop() == ("s2s", False, 0)
+    monkeypatch.setitem(tuner.best_configs, key, (CutoTuneConfig({"split_tile_tail": True, "waves": 4}), 1.0))
+    ops.scatter2scatter(X, W, idx, idx, out, 1, True, True, off)
+    assert calls.pop() == ("s2s", True, 4)
+    # (b) the caller fixes the form of the tail: no tuner, the library's loop
+    monkeypatch.setattr(ops, "SPLIT_TILE_TAIL", True)
+    ops.scatter2scatter(X, W, idx, idx, out, 1, True, True, off)
+    assert calls.pop() == ("s2s", True, 0)
+    monkeypatch.setattr(ops, "SPLIT_TILE_TAIL", None)
+    # (c) a product without a tail to split and one candidate loop: a single form, never through the tuner
+    Xs, Ws = X[:, :128].contiguous(), W[:, :128].contiguous()
+    before = dict(tuner.best_configs)
+    ops.scatter2scatter(Xs, Ws, idx, idx, out, 1, True, True, off)
+    assert calls.pop() == ("s2s", False, 0) and dict(tuner.best_configs) == before
+    # (d) the other three products: one candidate, passed as it is, no timing
+    h = torch.zeros(M, 2 * N, dtype=torch.bfloat16)
+    act = torch.zeros(M, N, dtype=torch.bfloat16)
+    ops.scatter2scatter_glu(Xs, torch.zeros(E, 128, 2 * N, dtype=torch.bfloat16), idx, off, h, act, 1, True)
+    assert calls.pop() == ("glu", 8)
+    ops.scatter2scatter_glu_bwd(Xs, torch.zeros(E, 128, N, dtype=torch.bfloat16), off, h, torch.zeros_like(h))
+    assert calls.pop() == ("glu_bwd", 8)
+    ops.group_bwd_W(out, Xs, off, torch.zeros(E, 128, N, dtype=torch.bfloat16), E)
+    assert calls.pop() == ("dw", 8)
+    assert not calls
+    # the binding itself refuses a loop that does not exist, before it touches the library
+    with pytest.raises(ValueError, match="waves"):
+        _C._waves(2, "scatter2scatter")
+
+
 def test_matrix_core_kernels_do_not_spill():
     """The grouped GEMM's main kernel runs two waves per SIMD at up to 256 registers each; a change that pushes an
     instantiation past that makes the compiler spill to scratch memory, which costs far more than the change is
