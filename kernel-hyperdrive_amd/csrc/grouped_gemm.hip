@@ -1348,6 +1348,10 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
             *reinterpret_cast<u32x2_t*>(Ch + row * C_LD + col) = four;
         }
     }
+    // The tile leaves LDS as 16-byte packets along rows.  Two copies of that code: the eight-wave kernels keep theirs
+    // statement for statement, so that they compile to the instructions that were measured (written as passes, the
+    // same code was scheduled and register-allocated differently); the four-wave kernels, with twice the packets per
+    // lane, take them in two passes over one set of registers.
     if constexpr (NWAVES == 8) {
         S* Cbase = reinterpret_cast<S*>(p.C) + (GROUP_K ? (int64_t)expert * p.c_stride_e : 0);
         typedef VPack<T, 8> P8;
@@ -1434,7 +1438,6 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
             }
         }
     } else {
-        // four waves: twice the packets per lane, taken in two passes over the same registers
         S* Cbase = reinterpret_cast<S*>(p.C) + (GROUP_K ? (int64_t)expert * p.c_stride_e : 0);
         typedef VPack<T, 8> P8;
         // GLU == 1: a lane takes an "up" packet together with its "gate" packet, so packets are counted over half a row
