@@ -1,13 +1,14 @@
-"""GPU: the HBM-bound operators at the full sizes BASELINE.json names for them (bf16).  The CPU oracle would
-take minutes there, so each result is held to what its definition fixes at any size - stock torch ops run in
-fp32 on the same device and rounded once, and size-independent properties (homogeneity, scale invariance,
-bit-exact gather, conservation of the gradient mass, untouched rows exactly zero, run-to-run identity)."""
+"""GPU: the HBM-bound operators at the full sizes BASELINE.json names for them (bf16).  Each result is held to the CPU
+oracle (whole tensors where that takes seconds - RMSNorm, the selected rows of the embedding gradient - and a seeded
+sample of rows for SwiGLU), to stock torch ops run in fp32 / fp64 on the same device and rounded once, and to what its
+definition fixes at any size (homogeneity, scale invariance, bit-exact gather, conservation of the gradient mass,
+untouched rows exactly zero, run-to-run identity)."""
 
 import pytest
 import torch
 import torch.nn.functional as F
 
-from helpers import announce
+from helpers import announce, assert_close
 from oracle import cute_oracle as O
 
 
@@ -23,6 +24,34 @@ def gpu_randn(shape, gpu, seed, scale=1.0, shift=0.0):
 
 def close(actual, expected, what):
     torch.testing.assert_close(actual, expected, rtol=TOL["rtol"], atol=TOL["atol"], msg=lambda m: f"{what}: {m}")
+
+
+# ---- the same results against the CPU oracle ------------------------------------------------------------------
+def oracle_swiglu_rows(gate, up, dy, y, gate_grad, up_grad, rows=256):
+    """A seeded sample of rows (the operator is element-wise: a row depends on nothing else)."""
+    pick = torch.randperm(gate.size(0), generator=torch.Generator().manual_seed(11))[:rows].sort().values.to(gate.device)
+    g, u, d = gate[pick].cpu(), up[pick].cpu(), dy[pick].cpu()
+    assert_close(y[pick], O.swiglu_forward(g, u), DTYPE, "y against the oracle")
+    exp_gate_grad, exp_up_grad = O.swiglu_backward(g, u, d)
+    assert_close(gate_grad[pick], exp_gate_grad, DTYPE, "gate_grad against the oracle")
+    assert_close(up_grad[pick], exp_up_grad, DTYPE, "up_grad against the oracle")
+
+
+def oracle_rmsnorm(x, w, dy, eps, y, dx, dw):
+    """Whole tensors: the oracle's closed forms in float64, rounded once (dw sums 16384 rows per element)."""
+    exp_y, _ = O.rmsnorm_forward(x, w, eps, compute_dtype=torch.float64)
+    assert_close(y, exp_y, DTYPE, "y against the oracle")
+    exp_dx, exp_dw = O.rmsnorm_backward(x, w, dy, eps, compute_dtype=torch.float64)
+    assert_close(dx, exp_dx, DTYPE, "dx against the oracle")
+    assert_close(dw, exp_dw, DTYPE, "dw against the oracle")
+
+
+def oracle_embedding_rows(ids, dy, V, out, table, dw):
+    """The gather bit for bit, and every selected row of the table gradient (the others are checked to be zero)."""
+    assert torch.equal(out, O.embedding_forward(ids, table.cpu()))
+    expected = O.embedding_backward(ids, dy, V)
+    selected = torch.unique(ids)
+    assert_close(dw[selected.to(dw.device)], expected[selected], DTYPE, "dw rows against the oracle")
 
 
 def test_swiglu_full_size(gpu):
@@ -42,6 +71,7 @@ def test_swiglu_full_size(gpu):
     close(gate.grad, g32.grad.to(DTYPE), "gate_grad")
     close(up.grad, u32.grad.to(DTYPE), "up_grad")
     del ref, g32, u32
+    oracle_swiglu_rows(gate.detach(), up.detach(), dy, y.detach(), gate.grad, up.grad)
     # homogeneous of degree one in `up`, and powers of two are exact in bf16
     with torch.no_grad():
         assert torch.equal(swiglu_cute(gate, up * 2), y.detach() * 2)
@@ -70,6 +100,8 @@ def test_rmsnorm_full_size(gpu):
     close(x.grad, x64.grad.to(DTYPE), "dx")
     # every element of dw is a sum over 16384 rows: exact math rounded once is the expectation
     close(w.grad, w64.grad.to(DTYPE), "dw")
+    del ref, x64, w64
+    oracle_rmsnorm(x.detach().cpu(), w.detach().cpu(), dy.cpu(), eps, y.detach().cpu(), x.grad.cpu(), w.grad.cpu())
     # scale invariance (up to eps): y(4x) = y(x) within one rounding step of the output
     with torch.no_grad():
         y4 = rmsnorm_cute(x.detach() * 4, w.detach(), eps)
@@ -104,6 +136,7 @@ def test_embedding_full_size(gpu, ids_kind):
     expected.index_add_(0, ids_gpu.flatten(), dy.view(-1, H).float())
     close(dw, expected.to(DTYPE), "dw")
     del expected
+    oracle_embedding_rows(ids, dy.cpu(), V, out.detach().cpu(), table.detach(), dw)
     # conservation: the columns of dw add up to the columns of dy (fp64 sums of bf16 values; the rounding of each
     # dw element is the only difference)
     lhs, rhs = dw.double().sum(0), dy.view(-1, H).double().sum(0)
