@@ -74,19 +74,25 @@ def build(verbose: bool = False, jobs: int | None = None) -> str:
     return LIB_PATH
 
 
-def kernel_resources(source: str) -> dict[str, dict[str, int]]:
+def kernel_resources(source: str, loops: bool = False) -> dict[str, dict[str, int]]:
     """Registers and scratch of every kernel of one source, as the compiler reports them
-    (``-Rpass-analysis=kernel-resource-usage``): {mangled name: {"vgprs": n, "scratch": bytes per lane}}.  Scratch
-    above zero means the kernel spills registers to memory."""
+    (``-Rpass-analysis=kernel-resource-usage``): {mangled name: {"vgprs": n, "agprs": n, "scratch": bytes per lane}}.
+    Scratch above zero means the kernel spills registers to memory.  With ``loops``, the device assembly of the same
+    compilation is read as well and every kernel gets ``"loops"``: one dict per innermost loop that holds matrix
+    instructions, counting them ("mfma") and what must not sit beside them - scratch accesses ("scratch") and copies
+    between the two halves of the register file ("acc_moves") - plus LDS reads, direct-to-LDS copies and barriers."""
     import re
     import tempfile
 
     with tempfile.TemporaryDirectory() as tmp:
-        cmd = [find_hipcc(), *HIPCC_FLAGS, "-Rpass-analysis=kernel-resource-usage", "-c",
-               os.path.join(CSRC_DIR, source), "-o", os.path.join(tmp, "out.o")]
+        out = os.path.join(tmp, "out.s" if loops else "out.o")
+        mode = ["--cuda-device-only", "-S"] if loops else ["-c"]
+        cmd = [find_hipcc(), *HIPCC_FLAGS, "-Rpass-analysis=kernel-resource-usage", *mode,
+               os.path.join(CSRC_DIR, source), "-o", out]
         result = subprocess.run(cmd, capture_output=True, text=True)
-    if result.returncode != 0:
-        raise RuntimeError(f"hipcc failed on {source}:\n{result.stderr}")
+        if result.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {source}:\n{result.stderr}")
+        assembly = open(out).read().split("\n") if loops else []
     found: dict[str, dict[str, int]] = {}
     name = None
     for line in result.stderr.splitlines():
@@ -95,8 +101,32 @@ def kernel_resources(source: str) -> dict[str, dict[str, int]]:
             found[name] = {}
         elif name and (match := re.search(r"remark:\s+VGPRs: (\d+)", line)):
             found[name]["vgprs"] = int(match.group(1))
+        elif name and (match := re.search(r"remark:\s+AGPRs: (\d+)", line)):
+            found[name]["agprs"] = int(match.group(1))
         elif name and (match := re.search(r"ScratchSize \[bytes/lane\]: (\d+)", line)):
             found[name]["scratch"] = int(match.group(1))
+    if loops:
+        starts = [(i, line.split(":")[0]) for i, line in enumerate(assembly) if re.match(r"^_Z\w+:", line)]
+        for k, (first, kernel) in enumerate(starts):
+            if kernel not in found:
+                continue
+            body = assembly[first:starts[k + 1][0] if k + 1 < len(starts) else len(assembly)]
+            labels = {m.group(1): i for i, line in enumerate(body) if (m := re.match(r"^(\.LBB\d+_\d+):", line))}
+            spans = []
+            for i, line in enumerate(body):
+                m = re.search(r"s_cbranch_\w+ (\.LBB\d+_\d+)", line)
+                if m and labels.get(m.group(1), i) < i:
+                    spans.append((labels[m.group(1)], i))
+            innermost = [s for s in spans if not any(o != s and s[0] <= o[0] and o[1] <= s[1] for o in spans)]
+            found[kernel]["loops"] = []
+            for lo, hi in innermost:
+                text = body[lo:hi]
+                count = lambda word: sum(word in line for line in text)
+                if count("v_mfma") > 0:
+                    found[kernel]["loops"].append({
+                        "mfma": count("v_mfma"), "scratch": count("scratch_"), "acc_moves": count("v_accvgpr"),
+                        "lds_reads": count("ds_read"), "copies": count("global_load_lds"), "barriers": count("s_barrier"),
+                    })
     return found
 
 

@@ -411,7 +411,7 @@ def test_matrix_core_kernels_do_not_spill():
     likely to gain and shows nowhere but in the timing.  The compiler's own report is checked instead."""
     from cute_kernels._build import kernel_resources
 
-    kernels = {n: r for n, r in kernel_resources("grouped_gemm.hip").items() if "grouped_gemm_m16_kernel" in n}
+    kernels = {n: r for n, r in kernel_resources("grouped_gemm.hip", loops=True).items() if "grouped_gemm_m16_kernel" in n}
     eight = {n: r for n, r in kernels.items() if "TileILi256ELi256ELi64ELi2ELi4EE" in n}
     four = {n: r for n, r in kernels.items() if "TileILi256ELi256ELi64ELi2ELi2EE" in n}
     assert len(eight) >= 18 and len(four) == len(eight), sorted(kernels)  # bf16 and fp16: 3 modes x 2 layouts, 2 fused, dW
@@ -422,6 +422,19 @@ def test_matrix_core_kernels_do_not_spill():
     # tile, outside the loop (20 bytes per lane), which is what the bound leaves room for.
     for name, res in four.items():
         assert res["vgprs"] <= 256 and res["scratch"] <= 32, (name, res)
+        # Its accumulators must stay in the accumulation registers: left to the register allocator they wandered between
+        # the two halves of the register file (two moves per matrix instruction) and through scratch.  Every loop with
+        # matrix instructions is free of both; the pipelined loops (two steps: 64 to 256 matrix instructions, depending on
+        # which halves of the tile hold data) keep their 32 copies and 8 barriers per turn.
+        pipelined = [loop for loop in res["loops"] if loop["copies"] == 32]
+        if "ELi0ELi2EEEv" not in name:  # (the launch that adds up partial tiles multiplies nothing)
+            counts = sorted(loop["mfma"] for loop in pipelined)
+            # (the forward SwiGLU tile is always full along the columns: two forms instead of four)
+            assert counts in ([64, 128, 128, 256], [128, 256]), (name, res["loops"])
+        for loop in res["loops"]:
+            assert loop["scratch"] == 0 and loop["acc_moves"] == 0, (name, loop)
+        for loop in pipelined:
+            assert loop["barriers"] == 8, (name, loop)
 
 
 def test_row_kernels_do_not_spill():
