@@ -16,6 +16,7 @@
 #include <type_traits>
 
 #include "ck_device.h"
+#include "ck_gemm_prims.h"
 
 namespace ck {
 
@@ -45,11 +46,8 @@ struct Mma16<BF16> {
     static __device__ __forceinline__ f32x4_t mma(frag_t a, frag_t b, f32x4_t c) {
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
     }
-    // the same with the accumulator pinned to the accumulation half of the register file (a loop with 256
-    // accumulator registers per lane: left to itself the register allocator moves them between the halves)
-    static __device__ __forceinline__ void mma_acc(frag_t a, frag_t b, f32x4_t& c) {
-        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
-    }
+    // the same with the accumulator pinned to the accumulation half of the register file
+    static __device__ __forceinline__ void mma_acc(frag_t a, frag_t b, f32x4_t& c) { mfma16_acc(a, b, c); }
 };
 template <>
 struct Mma16<F16> {
@@ -57,9 +55,7 @@ struct Mma16<F16> {
     static __device__ __forceinline__ f32x4_t mma(frag_t a, frag_t b, f32x4_t c) {
         return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
     }
-    static __device__ __forceinline__ void mma_acc(frag_t a, frag_t b, f32x4_t& c) {
-        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
-    }
+    static __device__ __forceinline__ void mma_acc(frag_t a, frag_t b, f32x4_t& c) { mfma16_acc(a, b, c); }
 };
 
 struct GemmParams {
@@ -380,18 +376,6 @@ struct DtlOperand {
     }
 };
 
-// Hides how a value was computed from the optimiser, which then cannot move the arithmetic that follows out
-// of the loop and keep every variant of it alive in a register of its own.
-__device__ __forceinline__ int opaque(int v) {
-    asm volatile("" : "+v"(v));
-    return v;
-}
-
-__device__ __forceinline__ uint64_t opaque_s64(uint64_t v) {  // same for a wave-uniform 64-bit value
-    asm volatile("" : "+s"(v));
-    return v;
-}
-
 // two fp32 values rounded to the storage type (round to nearest even) and packed into one dword, first value low
 template <typename T>
 __device__ __forceinline__ uint32_t pack2(float a, float b) {
@@ -419,7 +403,7 @@ __device__ __forceinline__ void unpack2(uint32_t w, float& a, float& b) {
 template <typename T, typename TL, bool B_KC, bool GROUP_K, int GLU = 0, int MODE = 0>
 // Two waves per SIMD is all the LDS footprint allows; telling the compiler keeps it from spilling to reach a
 // higher occupancy that cannot happen.
-__global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_eu(TL::WM * TL::WN / 4, TL::WM * TL::WN / 4)))
+__global__ void __launch_bounds__(TL::THREADS) CK_WAVES_PER_SIMD(TL::WM * TL::WN / 4)
     grouped_gemm_m16_kernel(GemmParams p) {
     static_assert(MODE == 0 || (GLU == 0 && !GROUP_K), "tail splitting is for the plain per-expert products");
     typedef typename T::storage_t S;
@@ -502,7 +486,6 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
 
     // ---- global sources of the LDS slots this lane fills ---------------------------------------------
     typedef __attribute__((address_space(1))) const char* gchar_t;
-    typedef __attribute__((address_space(3))) void* lptr_t;
     const gchar_t a_base = (gchar_t)p.A + (A_KC ? (int64_t)k_begin : (int64_t)k_begin * p.lda + i_base) * 2;
     const gchar_t b_base = (gchar_t)p.B + ((GROUP_K ? 0 : (int64_t)expert * p.b_stride_e) +
                                           (B_KCC ? (int64_t)k_begin : (int64_t)k_begin * p.ldb + n_base)) * 2;
@@ -547,18 +530,11 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
             }
     }
 
-    // One copy instruction: 64 lanes x 16 bytes from (wave-uniform base + 32-bit lane offset) to 1 KB of LDS at dst.
-    // Written as assembly so that the compiler's wait-count bookkeeping does not see the LDS writes: the waits for
-    // them are placed by hand below.
-    // (m0 carries the LDS address of the copy; nothing else in this kernel uses it)
-#pragma clang diagnostic push
-#pragma clang diagnostic ignored "-Winline-asm"
+    // One copy instruction: 64 lanes x 16 bytes from (wave-uniform base + 32-bit lane offset) to 1 KB of LDS at dst
+    // (lds_copy16: the compiler's wait-count bookkeeping does not see it; the waits are placed by hand below)
     auto dma = [&](gchar_t base, uint32_t voff, const char* dst) __attribute__((always_inline)) {
-        const uint32_t la = (uint32_t)(uintptr_t)((lptr_t)dst);
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(la), "v"(voff), "s"((uint64_t)base)
-                     : "memory", "m0");
+        lds_copy16(lds_address(dst), voff, (uint64_t)base);
     };
-#pragma clang diagnostic pop
     // one half operand (0: A lower, 1: A upper, 2: B lower, 3: B upper) of tile t, which lies inside the contraction range
     auto issue_part = [&](char* st, int part, int t) __attribute__((always_inline)) {
         if (part < 2) {
@@ -786,7 +762,7 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
 #define CK_M_END(PART)                                        \
     do {                                                      \
         issue_part(X, PART, tf);                              \
-        asm volatile("s_waitcnt vmcnt(12)" ::: "memory");     \
+        wait_copies<12>();     \
         __builtin_amdgcn_s_waitcnt(0xC07F); /* lgkmcnt(0) */  \
         CK_PHASE_END();                                       \
     } while (0)
@@ -889,7 +865,7 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
 #define CK_Q_END()                                                \
     do {                                                          \
         __builtin_amdgcn_sched_barrier(0);                        \
-        asm volatile("s_waitcnt vmcnt(24)" ::: "memory");         \
+        wait_copies<24>();         \
         __builtin_amdgcn_s_waitcnt(0xC07F); /* lgkmcnt(0) */      \
         __builtin_amdgcn_s_barrier();                             \
         __builtin_amdgcn_sched_barrier(0);                        \
@@ -966,7 +942,7 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
             else if (upper_cols_live) run(std::false_type{}, std::true_type{});
             else if (upper_rows_live) run(std::true_type{}, std::false_type{});
             else run(std::false_type{}, std::false_type{});
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            wait_copies<0>();
             __syncthreads();
             if (kt < n_full) {  // an odd number of full tiles: the last one is complete in lds0
                 multiply_tile(lds0);
@@ -987,7 +963,7 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
         issue_part(lds1, 0, 1);
         issue_part(lds1, 3, 1);
         issue_part(lds1, 1, 1);
-        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        wait_copies<8>();
         __syncthreads();
         read_b(lds0, 0, fb0);
         __builtin_amdgcn_s_waitcnt(0xC07F);
@@ -1005,7 +981,7 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
         else if (upper_rows_live) run(std::true_type{}, std::false_type{});
         else run(std::false_type{}, std::false_type{});
         if (wm == 0) CK_PHASE_END();
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        wait_copies<0>();
         __syncthreads();
         if (kt < n_full) {  // an odd number of full tiles: the last one is complete in lds0
             multiply_tile(lds0);
@@ -1015,7 +991,7 @@ __global__ void __launch_bounds__(TL::THREADS) __attribute__((amdgpu_waves_per_e
     }
     for (; kt < k_tiles; ++kt) {
         issue(kt, lds0);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        wait_copies<0>();
         __syncthreads();
         multiply_tile(lds0);
         __syncthreads();
