@@ -15,6 +15,7 @@
 #include <map>
 #include <random>
 #include <string>
+#include <type_traits>
 
 #include "../../kernel-hyperdrive_amd/csrc/ck_device.h"
 
@@ -168,11 +169,13 @@ void expose(std::initializer_list<std::pair<Buffer*, const char*>> buffers) {
 }
 
 // values whose products and sums are exact in fp32: multiples of 1/2 (activations) and of 1/4 (weights), small
+template <typename S = bf16>
 void fill(Buffer& b, std::mt19937& rng, int scale_quarters) {
-    bf16* v = b.as<bf16>();
-    for (size_t i = 0; i < b.size() / 2; ++i) v[i] = (bf16)(((int)(rng() % 9) - 4) * 0.25f * scale_quarters);
+    S* v = b.as<S>();
+    for (size_t i = 0; i < b.size() / 2; ++i) v[i] = (S)(((int)(rng() % 9) - 4) * 0.25f * scale_quarters);
 }
 float f(bf16 v) { return (float)v; }
+float f(_Float16 v) { return (float)v; }
 
 struct Routing {
     std::vector<int64_t> sorted_scattered, offsets;
@@ -206,41 +209,47 @@ int expert_of(const Routing& r, int slot) {
 int g_cases = 0;
 
 // out[out_row(i)] = X[in_row(i)] @ W[e(i)], W as the view [E, K, N] of [E, N, K] (k contiguous) or [E, K, N] (n contiguous)
+template <typename S = bf16>
 void scatter2scatter_case(std::mt19937& rng, int T, int k, int E, int K, int N, bool w_k_contiguous, bool x_grouped, bool y_grouped,
-                          bool split, int waves, bool late, int empty_expert) {
+                          bool split, int waves, bool late, int empty_expert, bool with_bias = false) {
+    const int dtype = sizeof(S) == 2 && std::is_same<S, bf16>::value ? CK_BF16 : CK_F16;
     char text[200];
-    std::snprintf(text, sizeof text, "scatter2scatter T=%d k=%d E=%d K=%d N=%d %s %s%s%s waves=%d copies %s", T, k, E, K, N,
-                  w_k_contiguous ? "NT" : "NN", x_grouped ? "grouped-in " : "gather-in ", y_grouped ? "grouped-out" : "scatter-out",
-                  split ? " split-tail" : "", waves, late ? "late" : "at once");
+    std::snprintf(text, sizeof text, "scatter2scatter %s T=%d k=%d E=%d K=%d N=%d %s %s%s%s%s waves=%d copies %s",
+                  dtype == CK_BF16 ? "bf16" : "fp16", T, k, E, K, N, w_k_contiguous ? "NT" : "NN", x_grouped ? "grouped-in " : "gather-in ",
+                  y_grouped ? "grouped-out" : "scatter-out", split ? " split-tail" : "", with_bias ? " bias" : "", waves,
+                  late ? "late" : "at once");
     emu::g_case = text;
     emu::g_late_copies = late;
     const Routing r = route(rng, T, k, E, empty_expert);
     const int fan_out = x_grouped ? 1 : k;
     const int x_rows = x_grouped ? r.slots : T;
     Buffer X = make((size_t)x_rows * K * 2, "X"), W = make((size_t)E * K * N * 2, "W"), out = make((size_t)r.slots * N * 2, "out");
-    fill(X, rng, 2);
-    fill(W, rng, 1);
-    for (size_t i = 0; i < out.size() / 2; ++i) out.as<bf16>()[i] = (bf16)-777.f;
+    fill<S>(X, rng, 2);
+    fill<S>(W, rng, 1);
+    Buffer bias = make((size_t)E * N * 2, "bias");
+    fill<S>(bias, rng, 3);
+    for (size_t i = 0; i < out.size() / 2; ++i) out.as<S>()[i] = (S)-777.f;
     Buffer idx = make(r.slots * 8, "idx"), off = make(E * 8, "offsets");
     std::memcpy(idx.bytes.data(), r.sorted_scattered.data(), r.slots * 8);
     std::memcpy(off.bytes.data(), r.offsets.data(), E * 8);
-    const int64_t ws_bytes = split ? ck_scatter2scatter_workspace_size(r.slots, K, N, E, CK_BF16) : 0;
+    const int64_t ws_bytes = split ? ck_scatter2scatter_workspace_size(r.slots, K, N, E, dtype) : 0;
     if (split && ws_bytes == 0) emu::die("the case is meant to have a tail to split");
     Buffer ws = make((size_t)std::max<int64_t>(ws_bytes, 16), "workspace");
     expose({{&X, "X"}, {&W, "W"}});
     const int64_t se = (int64_t)K * N, sk = w_k_contiguous ? 1 : N, sn = w_k_contiguous ? K : 1;
     const int status = ck_scatter2scatter_ws(X.as<void>(), K, W.as<void>(), se, sk, sn, idx.as<int64_t>(), off.as<int64_t>(),
-                                             out.as<void>(), N, r.slots, K, N, E, fan_out, x_grouped, y_grouped, nullptr, CK_BF16,
-                                             waves, split ? ws.as<void>() : nullptr, ws_bytes, nullptr);
+                                             out.as<void>(), N, r.slots, K, N, E, fan_out, x_grouped, y_grouped,
+                                             with_bias ? bias.as<void>() : nullptr, dtype, waves, split ? ws.as<void>() : nullptr,
+                                             ws_bytes, nullptr);
     if (status != CK_OK) emu::die("status " + std::to_string(status));
-    const bf16 *x = X.as<bf16>(), *w = W.as<bf16>(), *o = out.as<bf16>();
+    const S *x = X.as<S>(), *w = W.as<S>(), *o = out.as<S>(), *bv = bias.as<S>();
     for (int i = 0; i < r.slots; ++i) {
         const int e = expert_of(r, i);
         const int64_t in_row = x_grouped ? i : r.sorted_scattered[i] / fan_out, out_row = y_grouped ? i : r.sorted_scattered[i];
         for (int n = 0; n < N; ++n) {
-            float sum = 0.f;
+            float sum = with_bias ? f(bv[(int64_t)e * N + n]) : 0.f;  // the bias joins the fp32 sum before its one rounding
             for (int kk = 0; kk < K; ++kk) sum += f(x[in_row * K + kk]) * f(w[e * se + kk * sk + n * sn]);
-            const bf16 expected = (bf16)sum;
+            const S expected = (S)sum;
             if (std::memcmp(&expected, &o[out_row * N + n], 2) != 0) {
                 std::snprintf(text, sizeof text, "slot %d (expert %d) column %d: %g, expected %g", i, e, n, f(o[out_row * N + n]), f(expected));
                 emu::die(text);
@@ -383,6 +392,11 @@ int main(int argc, char** argv) {
         group_bwd_w_case(rng, 90, 2, 3, 136, 264, false, waves, true, 1);
         glu_case(rng, 40, 2, 2, 192, 128, waves, true);
         if (emu::g_lax_waits) continue;
+        // fp16 storage; a per-expert bias, whole tiles and split tail (a product with a bias takes the eight-wave loop
+        // whichever is asked for)
+        scatter2scatter_case<_Float16>(rng, 70, 2, 3, 192 + 8, 264, true, false, false, false, waves, true, -1);
+        scatter2scatter_case(rng, 70, 2, 3, 256, 136, true, false, true, false, waves, true, 1, true);
+        scatter2scatter_case(rng, 30, 1, 2, 4096, 128, false, true, true, true, waves, true, -1, true);
         // Copies that land at once (a copy that overwrites a half too early would show here)
         scatter2scatter_case(rng, 150, 2, 3, 320, 256, true, false, true, false, waves, false, -1);
         scatter2scatter_case(rng, 40, 1, 2, 192, 136, false, true, false, false, waves, false, -1);

@@ -43,7 +43,7 @@ def emulation(tmp_path_factory):
 def test_grouped_gemm_loops_under_emulation(emulation, waves):
     result = subprocess.run([emulation, waves], capture_output=True, text=True, timeout=900)
     assert result.returncode == 0, result.stdout + result.stderr
-    assert result.stdout.startswith("ok: 12 cases"), result.stdout
+    assert result.stdout.startswith("ok: 15 cases"), result.stdout
 
 
 @pytest.mark.parametrize("waves", ["8", "4"])
