@@ -21,6 +21,7 @@
 
 // ---- the instructions behind ck_gemm_prims.h, emulated ---------------------------------------------------------------
 #define CK_GEMM_PRIMS_H
+#define CK_GEMM_PRIMS_HOST
 #define CK_WAVES_PER_SIMD(n)
 namespace emu {
 struct Region {
@@ -146,7 +147,10 @@ inline emu_v4i16 emu_ds_read_tr16(Ptr p) {
 }
 #define __builtin_amdgcn_ds_read_tr16_b64_v4i16(p) emu_ds_read_tr16(p)
 
-#include "../../kernel-hyperdrive_amd/csrc/grouped_gemm.hip"
+#ifndef CK_GEMM_SOURCE  // (another copy of the kernel source can be named on the compiler's command line)
+#define CK_GEMM_SOURCE "../../kernel-hyperdrive_amd/csrc/grouped_gemm.hip"
+#endif
+#include CK_GEMM_SOURCE
 
 // ---- problems -----------------------------------------------------------------------------------------------------------
 namespace {
