@@ -367,10 +367,15 @@ void glu_case(std::mt19937& rng, int T, int k, int E, int K, int I, int waves, b
 }  // namespace
 
 int main(int argc, char** argv) {
-    // arguments: "8" or "4" (one loop only), "--lax-waits" (every wait on the copies eight short: the results must differ)
+    // arguments: "8" or "4" (one loop only), "--lax-waits" (every wait on the copies eight short: the results must differ),
+    // "--random N [--seed S]" (N random cases per loop instead of the fixed list)
     std::string only;
+    int random_cases = 0;
+    unsigned random_seed = 1;
     for (int i = 1; i < argc; ++i) {
         if (std::string(argv[i]) == "--lax-waits") emu::g_lax_waits = 8;
+        else if (std::string(argv[i]) == "--random" && i + 1 < argc) random_cases = std::atoi(argv[++i]);
+        else if (std::string(argv[i]) == "--seed" && i + 1 < argc) random_seed = (unsigned)std::atoi(argv[++i]);
         else only = argv[i];
     }
     emu::g_after_block = [] {
@@ -381,6 +386,25 @@ int main(int argc, char** argv) {
             }
     };
     std::mt19937 rng(2024);
+    if (random_cases > 0) {
+        // "--random N": N cases of random shape, layout, routing and copy timing per loop (for a longer soak than the fixed list)
+        rng.seed(random_seed);
+        for (int c = 0; c < random_cases; ++c) {
+            const int E = 1 + (int)(rng() % 5), k = 1 + (int)(rng() % std::min(E, 3)), T = 1 + (int)(rng() % 400);
+            const int K = 8 * (1 + (int)(rng() % 80)), N = 8 * (1 + (int)(rng() % 70));
+            const bool late = rng() % 2, kc = rng() % 2, xg = rng() % 2, yg = rng() % 2;
+            const int empty = E > k && rng() % 3 == 0 ? (int)(rng() % E) : -1;
+            for (int waves : {8, 4}) {
+                if (!only.empty() && only != std::to_string(waves)) continue;
+                if (rng() % 2)
+                    scatter2scatter_case(rng, T, k, E, K, N, kc, xg, yg, false, waves, late, empty);
+                else
+                    group_bwd_w_case(rng, T, k, E, K, N, kc, waves, late, empty);
+            }
+        }
+        std::printf("ok: %d random cases\n", g_cases);
+        return 0;
+    }
     for (int waves : {8, 4}) {
         if (!only.empty() && only != std::to_string(waves)) continue;
         // Copies that land as late as the kernel's waits allow: contractions of 2, 3 (odd: the last tile outside the
