@@ -125,6 +125,7 @@ __device__ __forceinline__ void block_radix_pass(SortShared& sh, int n, int shif
             int pos = 0;
             if (valid) pos = sh.digit_base[digit] + sh.hist[wave][digit] + __popcll(lower);
             // all lanes have read the running offset before the group's first lane advances it
+            CK_WAVE_LOCKSTEP();
             if (valid && lower == 0) sh.hist[wave][digit] += __popcll(m);
             if (valid) store(pos, keys[u], vals[u]);
         }

@@ -83,6 +83,13 @@ __device__ __forceinline__ void nt_store(const P& v, P* p) {
 // ---- wave64 primitives ---------------------------------------------------------------------
 __device__ __forceinline__ int lane_id() { return __lane_id(); }
 
+// Marks a point where lanes of one wavefront hand data to each other through memory and rely on the wavefront's
+// lock-step execution for the order (the LDS serves a wave's accesses in program order).  No instruction and no
+// constraint on the GPU; a host build that runs the lanes as separate threads of control makes them meet here.
+#ifndef CK_WAVE_LOCKSTEP
+#define CK_WAVE_LOCKSTEP()
+#endif
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, CK_WAVE);

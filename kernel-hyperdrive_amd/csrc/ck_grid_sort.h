@@ -54,6 +54,7 @@ __device__ __forceinline__ void grid_sort_histogram(GridSortShared& sh, int n, i
         // groups of one batch hold different digits, batches follow each other in program order
         if (valid && (m & lanemask_lt()) == 0) bins[digit] += (uint32_t)__popcll(m);
     }
+    CK_WAVE_LOCKSTEP();
     for (int d = lane; d < nbins; d += CK_WAVE) hist[(int64_t)d * num_waves + gw] = bins[d];
 }
 
@@ -157,6 +158,7 @@ __device__ __forceinline__ void grid_sort_scatter(GridSortShared& sh, int n, int
         uint32_t pos = 0;
         if (valid) pos = next[digit] + (uint32_t)__popcll(lower);
         // every lane of the group has read the offset before its first lane advances it
+        CK_WAVE_LOCKSTEP();
         if (valid && lower == 0) next[digit] += (uint32_t)__popcll(m);
         if (valid) store((int)pos, keys[u], vals[u]);
     }

@@ -17,135 +17,7 @@
 #include <string>
 #include <type_traits>
 
-#include "../../kernel-hyperdrive_amd/csrc/ck_device.h"
-
-// ---- the instructions behind ck_gemm_prims.h, emulated ---------------------------------------------------------------
-#define CK_GEMM_PRIMS_H
-#define CK_GEMM_PRIMS_HOST
-#define CK_WAVES_PER_SIMD(n)
-namespace emu {
-struct Region {
-    const char* begin;
-    const char* end;
-    std::string name;
-};
-inline std::vector<Region> g_regions;  // global memory the kernels may read through copies
-inline bool g_late_copies = false;     // copies land only when a wait forces them to (else at once)
-inline int g_lax_waits = 0;            // --lax-waits: every wait leaves this many more copies under way than it says
-struct PendingCopy {
-    char* dst;
-    const char* src;
-};
-inline std::vector<PendingCopy> g_pending[kMaxLanes];
-inline std::string g_case;
-
-[[noreturn]] inline void die(const std::string& what) {
-    std::printf("FAILED (%s): %s\n", g_case.c_str(), what.c_str());
-    std::exit(1);
-}
-inline void land(const PendingCopy& c) { std::memcpy(c.dst, c.src, 16); }
-}  // namespace emu
-
-namespace ck {
-typedef uintptr_t lds_addr_t;
-inline lds_addr_t lds_address(const char* p) { return (lds_addr_t)p; }
-inline void lds_copy16(lds_addr_t la, uint32_t voff, uint64_t base) {
-    const char* src = reinterpret_cast<const char*>(base) + voff;
-    bool inside = false;
-    for (const emu::Region& r : emu::g_regions) inside = inside || (src >= r.begin && src + 16 <= r.end);
-    if (!inside) {
-        char text[160];
-        std::snprintf(text, sizeof text, "a copy reads 16 bytes at %p, outside every operand (workgroup %u, thread %d)",
-                      (const void*)src, emu::g_block_index.x, emu::g_current);
-        emu::die(text);
-    }
-    const emu::PendingCopy copy{reinterpret_cast<char*>(la) + 16 * (emu::g_current % emu::kWave), src};
-    if (emu::g_late_copies)
-        emu::g_pending[emu::g_current].push_back(copy);
-    else
-        emu::land(copy);
-}
-template <int N>
-inline void wait_copies() {
-    auto& mine = emu::g_pending[emu::g_current];
-    while ((int)mine.size() > N + (N > 0 ? emu::g_lax_waits : 0)) {
-        emu::land(mine.front());
-        mine.erase(mine.begin());
-    }
-}
-inline int opaque(int v) { return v; }
-inline uint64_t opaque_s64(uint64_t v) { return v; }
-
-// v_mfma_f32_16x16x32: lane l holds A[i = l % 16][k = 8 (l / 16) .. + 7], B[k = 8 (l / 16) .. + 7][j = l % 16] and
-// D[i = 4 (l / 16) + r][j = l % 16], r = 0 .. 3
-template <typename Frag>
-inline f32x4_t emu_mfma16(Frag a, Frag b, f32x4_t c) {
-    struct In {
-        Frag a, b;
-    } in{a, b};
-    const int me = __lane_id();
-    return emu::wave_instruction(in, [me, c](auto lane) {
-        f32x4_t d = c;
-        const int j = me % 16;
-        for (int r = 0; r < 4; ++r) {
-            const int i = 4 * (me / 16) + r;
-            float sum = 0.f;
-            for (int g = 0; g < 4; ++g) {
-                const In a_lane = lane(16 * g + i), b_lane = lane(16 * g + j);
-                for (int e = 0; e < 8; ++e) sum += (float)a_lane.a[e] * (float)b_lane.b[e];
-            }
-            d[r] += sum;
-        }
-        return d;
-    });
-}
-inline void mfma16_acc(bf16x8_t a, bf16x8_t b, f32x4_t& c) { c = emu_mfma16(a, b, c); }
-inline void mfma16_acc(f16x8_t a, f16x8_t b, f32x4_t& c) { c = emu_mfma16(a, b, c); }
-}  // namespace ck
-#define __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, x, y, z) ck::emu_mfma16(a, b, c)
-#define __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, x, y, z) ck::emu_mfma16(a, b, c)
-
-// v_mfma_f32_32x32x16 (the 64-bit-address kernel): lane l holds A[i = l % 32][k = 8 (l / 32) .. + 7], B likewise, and
-// D[i = 8 (r / 4) + 4 (l / 32) + r % 4][j = l % 32], r = 0 .. 15
-template <typename Frag>
-inline ck::f32x16_t emu_mfma32(Frag a, Frag b, ck::f32x16_t c) {
-    struct In {
-        Frag a, b;
-    } in{a, b};
-    const int me = __lane_id();
-    return emu::wave_instruction(in, [me, c](auto lane) {
-        ck::f32x16_t d = c;
-        const int j = me % 32;
-        for (int r = 0; r < 16; ++r) {
-            const int i = 8 * (r / 4) + 4 * (me / 32) + r % 4;
-            float sum = 0.f;
-            for (int g = 0; g < 2; ++g) {
-                const In a_lane = lane(32 * g + i), b_lane = lane(32 * g + j);
-                for (int e = 0; e < 8; ++e) sum += (float)a_lane.a[e] * (float)b_lane.b[e];
-            }
-            d[r] += sum;
-        }
-        return d;
-    });
-}
-#define __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, x, y, z) emu_mfma32(a, b, c)
-#define __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, x, y, z) emu_mfma32(a, b, c)
-
-// ds_read_b64_tr_b16: inside each group of 16 lanes, lanes 4 r .. 4 r + 3 fetch the 16 elements of row r (8 bytes
-// each), and lane i receives element i of rows 0 .. 3
-typedef short emu_v4i16 __attribute__((ext_vector_type(4)));
-template <typename Ptr>
-inline emu_v4i16 emu_ds_read_tr16(Ptr p) {
-    const short* mine = (const short*)p;
-    const int me = __lane_id();
-    return emu::wave_instruction(mine, [me](auto lane) {
-        const int group = me / 16 * 16, i = me % 16;
-        emu_v4i16 out;
-        for (int r = 0; r < 4; ++r) out[r] = lane(group + 4 * r + i / 4)[i % 4];
-        return out;
-    });
-}
-#define __builtin_amdgcn_ds_read_tr16_b64_v4i16(p) emu_ds_read_tr16(p)
+#include "shim/ck_gemm_prims_emulated.h"
 
 #ifndef CK_GEMM_SOURCE  // (another copy of the kernel source can be named on the compiler's command line)
 #define CK_GEMM_SOURCE "../../kernel-hyperdrive_amd/csrc/grouped_gemm.hip"

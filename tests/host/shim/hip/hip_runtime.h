@@ -1,5 +1,5 @@
-// Stand-in for <hip/hip_runtime.h> in host builds of the kernel sources (tests/host/gemm_emulation.cpp): a workgroup is
-// emulated as one coroutine per lane; lanes run freely and meet only where the hardware makes them meet - at workgroup
+// Stand-in for <hip/hip_runtime.h> in host builds of the kernel sources (tests/host/gemm_emulation.cpp and the emulated
+// library of tests/host/emulated_library.py): a workgroup is emulated as one coroutine per lane; lanes run freely and meet only where the hardware makes them meet - at workgroup
 // barriers and at wave-wide instructions (shuffles, ballots, matrix instructions, transposing LDS reads), where every
 // lane of the wave leaves its operand, waits for the others and computes its own result from all 64.
 // Nothing here is part of the product; only the test harness includes it (through -I tests/host/shim).
@@ -23,6 +23,7 @@
 #define __shared__ static
 #define __launch_bounds__(...)
 #define __restrict__
+#define __align__(n) __attribute__((aligned(n)))
 
 struct dim3 {
     unsigned x, y, z;
@@ -32,6 +33,31 @@ typedef void* hipStream_t;
 typedef int hipError_t;
 constexpr hipError_t hipSuccess = 0;
 inline hipError_t hipGetLastError() { return hipSuccess; }
+// the one emulated device: few compute units, so that grids sized by the device stay small
+constexpr int hipDeviceAttributeMultiprocessorCount = 0;
+inline hipError_t hipGetDevice(int* device) {
+    *device = 0;
+    return hipSuccess;
+}
+inline hipError_t hipDeviceGetAttribute(int* value, int, int) {
+    *value = 4;
+    return hipSuccess;
+}
+template <typename Kernel>
+hipError_t hipOccupancyMaxActiveBlocksPerMultiprocessor(int* blocks, Kernel, int, size_t) {
+    *blocks = 1;
+    return hipSuccess;
+}
+#define HIP_SYMBOL(x) (x)
+template <typename Symbol>
+hipError_t hipGetSymbolAddress(void** address, Symbol& symbol) {
+    *address = (void*)&symbol;
+    return hipSuccess;
+}
+struct float4 {
+    float x, y, z, w;
+};
+inline float4 make_float4(float x, float y, float z, float w) { return float4{x, y, z, w}; }
 
 namespace emu {
 constexpr int kWave = 64;
@@ -196,16 +222,49 @@ struct EmuGridDim {
         operator unsigned() const { return emu::g_grid_dim.y; }
     } y;
 };
+struct EmuBlockDim {
+    struct X {
+        operator unsigned() const { return emu::g_block_dim.x; }
+    } x;
+};
 inline EmuThreadIdx threadIdx;
 inline EmuBlockIdx blockIdx;
 inline EmuGridDim gridDim;
+inline EmuBlockDim blockDim;
 
 using std::max;
 using std::min;
 
 inline int __lane_id() { return emu::g_current % emu::kWave; }
 inline void __syncthreads() { emu::sync(emu::g_block); }
+// barrier that also counts the lanes whose predicate holds (three meetings: cleared by all, added by all, read by all)
+inline int g_emu_votes;
+inline int __syncthreads_count(int predicate) {
+    g_emu_votes = 0;
+    emu::sync(emu::g_block);
+    g_emu_votes += predicate != 0;
+    emu::sync(emu::g_block);
+    const int votes = g_emu_votes;
+    emu::sync(emu::g_block);
+    return votes;
+}
 inline int __ffsll(unsigned long long v) { return __builtin_ffsll((long long)v); }
+inline int __popcll(unsigned long long v) { return __builtin_popcountll(v); }
+inline int __popc(unsigned v) { return __builtin_popcount(v); }
+inline float rsqrtf(float x) { return 1.0f / std::sqrt(x); }
+// one host thread runs every lane: a read-modify-write cannot be torn
+template <typename T, typename V>
+T atomicAdd(T* p, V v) {
+    const T old = *p;
+    *p = old + (T)v;
+    return old;
+}
+template <typename T, typename V>
+T atomicMax(T* p, V v) {
+    const T old = *p;
+    *p = std::max(old, (T)v);
+    return old;
+}
 inline uint64_t __ballot(bool p) {
     return emu::wave_instruction((int)p, [](auto lane) {
         uint64_t m = 0;
@@ -240,7 +299,84 @@ inline int emu_readfirstlane(int v) {
 }
 #define __builtin_amdgcn_readfirstlane(v) emu_readfirstlane(v)
 #define __builtin_amdgcn_s_barrier() emu::sync(emu::g_block)
+// The lanes of a wavefront run in lock-step on the hardware; here they run freely between the instructions that make
+// them meet.  Where a kernel lets lanes of one wave talk through memory and relies on the lock-step, it says so with a
+// wave barrier (no instruction on the GPU, an ordering for the compiler) - here the lanes of the wave do meet there.
+inline void emu_wave_barrier() { emu::sync(emu::g_waves[emu::g_current / emu::kWave].group); }
+#define __builtin_amdgcn_wave_barrier() emu_wave_barrier()
+#define CK_WAVE_LOCKSTEP() emu_wave_barrier()
+inline void __threadfence_block() {}
+inline void __threadfence() {}
 #define __builtin_amdgcn_sched_barrier(mask) emu_nothing()
 #define __builtin_amdgcn_s_waitcnt(code) emu_nothing()
 #define __builtin_amdgcn_s_setprio(level) emu_nothing()
 #define __builtin_amdgcn_rcpf(x) (1.0f / (x))
+
+// ---- gfx950 wave-wide instructions, modelled by their lane layouts -------------------------------------------------------
+// v_mfma_f32_16x16x32: lane l holds A[i = l % 16][k = 8 (l / 16) .. + 7], B[k = 8 (l / 16) .. + 7][j = l % 16] and
+// D[i = 4 (l / 16) + r][j = l % 16], r = 0 .. 3
+template <typename Frag, typename Acc>
+inline Acc emu_mfma16(Frag a, Frag b, Acc c) {
+    struct In {
+        Frag a, b;
+    } in{a, b};
+    const int me = __lane_id();
+    return emu::wave_instruction(in, [me, c](auto lane) {
+        Acc d = c;
+        const int j = me % 16;
+        for (int r = 0; r < 4; ++r) {
+            const int i = 4 * (me / 16) + r;
+            float sum = 0.f;
+            for (int g = 0; g < 4; ++g) {
+                const In a_lane = lane(16 * g + i), b_lane = lane(16 * g + j);
+                for (int e = 0; e < 8; ++e) sum += (float)a_lane.a[e] * (float)b_lane.b[e];
+            }
+            d[r] += sum;
+        }
+        return d;
+    });
+}
+#define __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, x, y, z) emu_mfma16(a, b, c)
+#define __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, x, y, z) emu_mfma16(a, b, c)
+
+// v_mfma_f32_32x32x16: lane l holds A[i = l % 32][k = 8 (l / 32) .. + 7], B likewise, and
+// D[i = 8 (r / 4) + 4 (l / 32) + r % 4][j = l % 32], r = 0 .. 15
+template <typename Frag, typename Acc>
+inline Acc emu_mfma32(Frag a, Frag b, Acc c) {
+    struct In {
+        Frag a, b;
+    } in{a, b};
+    const int me = __lane_id();
+    return emu::wave_instruction(in, [me, c](auto lane) {
+        Acc d = c;
+        const int j = me % 32;
+        for (int r = 0; r < 16; ++r) {
+            const int i = 8 * (r / 4) + 4 * (me / 32) + r % 4;
+            float sum = 0.f;
+            for (int g = 0; g < 2; ++g) {
+                const In a_lane = lane(32 * g + i), b_lane = lane(32 * g + j);
+                for (int e = 0; e < 8; ++e) sum += (float)a_lane.a[e] * (float)b_lane.b[e];
+            }
+            d[r] += sum;
+        }
+        return d;
+    });
+}
+#define __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, x, y, z) emu_mfma32(a, b, c)
+#define __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, x, y, z) emu_mfma32(a, b, c)
+
+// ds_read_b64_tr_b16: inside each group of 16 lanes, lanes 4 r .. 4 r + 3 fetch the 16 elements of row r (8 bytes
+// each), and lane i receives element i of rows 0 .. 3
+typedef short emu_v4i16 __attribute__((ext_vector_type(4)));
+template <typename Ptr>
+inline emu_v4i16 emu_ds_read_tr16(Ptr p) {
+    const short* mine = (const short*)p;
+    const int me = __lane_id();
+    return emu::wave_instruction(mine, [me](auto lane) {
+        const int group = me / 16 * 16, i = me % 16;
+        emu_v4i16 out;
+        for (int r = 0; r < 4; ++r) out[r] = lane(group + 4 * r + i / 4)[i % 4];
+        return out;
+    });
+}
+#define __builtin_amdgcn_ds_read_tr16_b64_v4i16(p) emu_ds_read_tr16(p)

@@ -1,0 +1,141 @@
+"""The GPU parity tests, run without a GPU: every kernel source of the library is compiled for the host against an
+emulation of a gfx950 workgroup (tests/host/emulated_library.py, tests/host/shim - one coroutine per lane; barriers,
+shuffles, ballots, the matrix instructions, the transposing LDS read and the direct global -> LDS copy modelled by what
+they do to the 64 lanes), linked into a library with the same C entry points, and put behind the package's ctypes
+binding.  The bodies of the GPU tests then run unchanged on CPU tensors - the same Python launchers, autograd functions
+and layer, the same device code, the same oracle and tolerances - at shapes the emulation finishes in seconds.
+
+What this pins: the device code's arithmetic and indexing, lane for lane, and every place where lanes meet.  What it
+cannot: timing, the memory model between workgroups (they run one after the other here) and the real instructions'
+corner cases - the GPU tests stay the parity tests proper, and the emulation's own models are checked against them by
+the kernels whose GPU results are already pinned."""
+
+import pytest
+import torch
+
+import test_golden as G
+import test_gpu_elementwise as E
+import test_gpu_moe as M
+import test_gpu_moe_int as I
+import wip_four_wave as W
+from host import emulated_library
+
+
+BF16, F16, F32 = torch.bfloat16, torch.float16, torch.float32
+
+
+@pytest.fixture(scope="module")
+def library(tmp_path_factory):
+    if emulated_library.host_clang() is None:
+        pytest.skip("no clang of the ROCm toolchain to build the host emulation with")
+    return emulated_library.build(str(tmp_path_factory.mktemp("emulated_library")))
+
+
+@pytest.fixture
+def emulated(library):
+    """The binding points at the emulated library for the length of one test only."""
+    with emulated_library.bound_to(library):
+        yield torch.device("cpu")
+
+
+CASES = []
+
+
+def case(function, **arguments):
+    label = function.__name__[5:] + "-" + "-".join(str(v).replace("torch.", "") for v in arguments.values())
+    CASES.append(pytest.param(function, arguments, id=label[:90]))
+
+
+# ---- the HBM-bound operators ---------------------------------------------------------------------------------------------
+case(E.test_add_tensor_and_scalar, dtype=F32, size=(4099,))
+case(E.test_add_tensor_and_scalar, dtype=F32, size=(37, 513))  # (16-bit: stock torch on the CPU rounds the scalar first)
+case(E.test_add_layouts_and_errors)
+case(E.test_swiglu, dtype=BF16, size=(37, 513))
+case(E.test_swiglu, dtype=F32, size=(4099,))
+case(E.test_swiglu_unaligned_views_and_block_sizes, dtype=F16)
+case(E.test_swiglu_unchunked, dtype=BF16, size=(400, 1026))
+case(E.test_swiglu_unchunked, dtype=F32, size=(3, 18))
+for dtype, has_weight, memory_efficient, size in [
+    (BF16, True, False, (37, 4096)), (BF16, False, True, (5, 72)), (F16, True, True, (3, 70)),
+    (BF16, True, False, (2, 40000)), (F32, True, True, (37, 4096)), (F32, False, False, (2, 40000)),
+]:
+    case(E.test_rmsnorm, dtype=dtype, has_weight=has_weight, memory_efficient=memory_efficient, size=size)
+case(E.test_fused_residual_add_rmsnorm, dtype=BF16, has_weight=True, memory_efficient=False, size=(37, 4096))
+case(E.test_fused_residual_add_rmsnorm, dtype=F32, has_weight=False, memory_efficient=True, size=(3, 70))
+case(E.test_embedding, dtype=BF16, ids_shape=(51, 17), table=(7153, 937))
+case(E.test_embedding, dtype=F32, ids_shape=(3, 5), table=(11, 16384))
+for kind in ("zipf", "one_row", "run_lengths", "int32_ids", "empty"):
+    case(E.test_embedding_duplicates, dtype=BF16, case=kind)
+case(E.test_embedding_duplicates, dtype=F32, case="one_row")
+
+# ---- histogram, expert sort, offsets ---------------------------------------------------------------------------------------
+case(I.test_contiguous_count, dtype=torch.int64, n=4099, size=4096)
+case(I.test_contiguous_count, dtype=torch.int32, n=100000, size=72)
+case(I.test_contiguous_count, dtype=torch.int64, n=0, size=8)
+for dtype, rows, experts in [(torch.int64, 0, 8), (torch.int64, 1, 1), (torch.int32, 1000, 6), (torch.int64, 16385, 5),
+                             (torch.int64, 5000, 72), (torch.int32, 3000, 300), (torch.int64, 40000, 512)]:
+    case(I.test_moe_sort, dtype=dtype, M=rows, E=experts)
+case(I.test_moe_sort_on_topk_output)
+case(I.test_offsets_from_sorted)
+
+# ---- the grouped products and the kernels around them ---------------------------------------------------------------------
+for dtype, w_layout, mode, shape in [
+    (BF16, "k_contiguous", "gather_in", M.S2S_SHAPES[1]), (BF16, "n_contiguous", "scatter_out", M.S2S_SHAPES[2]),
+    (F16, "k_contiguous", "grouped_both", M.S2S_SHAPES[2]), (F16, "n_contiguous", "gather_in", M.S2S_SHAPES[1]),
+    (F32, "k_contiguous", "scatter_out", M.S2S_SHAPES[2]), (BF16, "k_contiguous", "gather_in", M.S2S_SHAPES[5]),
+]:
+    case(M.test_scatter2scatter, dtype=dtype, w_layout=w_layout, mode=mode, shape=shape)
+case(M.test_scatter2scatter_glu, dtype=BF16, shape=M.GLU_SHAPES[0])
+case(M.test_scatter2scatter_glu, dtype=F16, shape=M.GLU_SHAPES[3])
+case(M.test_scatter2scatter_glu, dtype=F32, shape=M.GLU_SHAPES[0])
+case(M.test_group_bwd_W, dtype=BF16, dw_layout="k_contiguous", shape=(100, 2, 4, 72, 136, (1,)))
+case(M.test_group_bwd_W, dtype=F16, dw_layout="n_contiguous", shape=(300, 3, 7, 200, 40, (0, 6)))
+case(M.test_group_bwd_W, dtype=F32, dw_layout="k_contiguous", shape=(300, 3, 7, 200, 40, (0, 6)))
+case(M.test_group, dtype=BF16, K=100, with_coeff=True)
+case(M.test_group, dtype=F32, K=4096, with_coeff=False)
+case(M.test_moe_combine, dtype=BF16, shape=(77, 2, 4096))
+case(M.test_moe_combine, dtype=F32, shape=(50, 3, 30))
+for dtype, (tokens, experts, k, ties) in [(BF16, M.ROUTER_CASES[1]), (F16, M.ROUTER_CASES[2]), (F32, M.ROUTER_CASES[3]),
+                                           (BF16, M.ROUTER_CASES[4]), (F32, M.ROUTER_CASES[5])]:
+    case(M.test_router_topk_softmax, dtype=dtype, T=tokens, E=experts, k=k, ties=ties)
+for dtype, (tokens, hidden, experts, k) in [(BF16, M.ROUTER_LINEAR_CASES[0]), (F16, M.ROUTER_LINEAR_CASES[1]),
+                                             (BF16, M.ROUTER_LINEAR_CASES[2])]:
+    case(M.test_router_linear_topk_softmax, dtype=dtype, T=tokens, H=hidden, E=experts, k=k)
+case(M.test_router_weight_grad, dtype=BF16, T=1000, H=200, E=5)
+case(M.test_router_weight_grad, dtype=F16, T=8, H=8, E=1)
+case(M.test_expert_bias_ops, dtype=BF16, T=300, k=3, E=7, N=200, empty=(0, 6))
+case(M.test_expert_bias_ops, dtype=F32, T=257, k=2, E=5, N=36, empty=(2,))
+for dtype in (F32, BF16, F16):
+    case(G.test_hip_router_golden, dtype=dtype)
+    case(G.test_hip_residual_rmsnorm_golden, dtype=dtype)
+case(G.test_hip_router_linear_golden, dtype=BF16)
+case(G.test_hip_router_linear_golden, dtype=F16)
+
+# ---- the layer: forward and backward through the Python stack ---------------------------------------------------------------
+TOP1, ODD_ROWS = M.MOE_CASES[3], M.MOE_CASES[1]
+case(M.test_moe_layer_against_oracle, dtype=BF16, case=TOP1)
+case(M.test_moe_layer_against_oracle, dtype=F16, case=TOP1)
+case(M.test_moe_layer_against_oracle, dtype=F32, case=ODD_ROWS)
+case(M.test_moe_layer_with_expert_biases, dtype=BF16, case=TOP1)
+case(M.test_moe_layer_fused_swiglu_equals_separate_ops, dtype=BF16, case=TOP1)
+case(M.test_moe_3d_input_and_weight_grad_layout)
+
+# ---- the four-wave loop of the grouped products against the eight-wave loop, bit for bit ---------------------------------------
+case(W.test_scatter2scatter_four_waves, dtype=BF16, w_layout="k_contiguous", mode="gather_in", shape=W.SHAPES[0])
+case(W.test_scatter2scatter_four_waves, dtype=F16, w_layout="n_contiguous", mode="scatter_out", shape=W.SHAPES[1])
+case(W.test_fused_swiglu_products_four_waves, dtype=BF16, shape=(300, 2, 3, 192, 128))
+case(W.test_group_bwd_W_four_waves, dtype=BF16, dw_layout="k_contiguous", shape=(300, 2, 3, 256, 256, ()))
+
+
+@pytest.mark.parametrize("function,arguments", CASES)
+def test_gpu_test_body_on_the_emulated_device(emulated, function, arguments):
+    function(emulated, **arguments)
+
+
+def test_the_package_itself_still_refuses_cpu_tensors():
+    """Outside the emulation's binding the product path is the GPU library or an error: no CPU route."""
+    from cute_kernels import _C
+
+    with pytest.raises(RuntimeError, match="need GPU tensors"):
+        _C._require_gpu(torch.zeros(4))
+    assert _C._Launch.__name__ == "_Launch"

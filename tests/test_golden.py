@@ -132,7 +132,7 @@ def test_hip_router_golden(gpu, dtype):
 
     announce("golden router", dtype)
     f = load("router")
-    logits = f["logits"].to(dtype).to(gpu).requires_grad_(True)
+    logits = f["logits"].to(dtype).to(gpu, copy=True).requires_grad_(True)
     weights, selected = router_topk_softmax(logits, int(f["top_k"]))
     weights.backward(f["d_weights"].to(dtype).to(gpu))
     assert torch.equal(selected.cpu(), f["selected"]), "largest first, equal logits in the order of their positions"
@@ -172,7 +172,7 @@ def test_hip_residual_rmsnorm_golden(gpu, dtype):
 
     announce("golden residual rmsnorm", dtype)
     f = load("residual_rmsnorm")
-    x, r, w = (f[key].to(dtype).to(gpu).requires_grad_(True) for key in ("x", "r", "w"))
+    x, r, w = (f[key].to(dtype).to(gpu, copy=True).requires_grad_(True) for key in ("x", "r", "w"))
     y, s = fused_residual_add_rmsnorm_cute(x, r, w, float(f["eps"]))
     torch.autograd.backward([y, s], [f["dy"].to(dtype).to(gpu), f["ds"].to(dtype).to(gpu)])
     assert torch.equal(s.detach().cpu().double(), f["s"]), "the sum is exact in every storage type"
@@ -199,7 +199,7 @@ def test_hip_moe_bias_golden(gpu, dtype):
         for param, key in ((moe.gate.weight, "w_gate"), (moe.c_fc.weight, "w_fc"), (moe.c_proj.weight, "w_proj"),
                            (moe.c_fc.bias, "b_fc"), (moe.c_proj.bias, "b_proj")):
             param.copy_(f[key])
-    x = f["x"].to(dtype).to(gpu).requires_grad_(True)
+    x = f["x"].to(dtype).to(gpu, copy=True).requires_grad_(True)
     y, _ = moe(x)
     (y * f["dy"].to(dtype).to(gpu)).sum().backward()
     with torch.no_grad():
@@ -222,14 +222,14 @@ def test_hip_swiglu_golden(gpu, dtype):
     announce("golden swiglu", dtype)
     f = load("swiglu")
     hip = KernelBackend.hip
-    gate = f["gate"].to(dtype).to(gpu).requires_grad_(True)
-    up = f["up"].to(dtype).to(gpu).requires_grad_(True)
+    gate = f["gate"].to(dtype).to(gpu, copy=True).requires_grad_(True)
+    up = f["up"].to(dtype).to(gpu, copy=True).requires_grad_(True)
     y = swiglu_cute(gate, up, hip, hip, 256, 256)
     y.backward(f["dy"].to(dtype).to(gpu))
     assert_close(y.detach(), f["y"].to(dtype), dtype, "y")
     assert_close(gate.grad, f["d_gate"].to(dtype), dtype, "d_gate")
     assert_close(up.grad, f["d_up"].to(dtype), dtype, "d_up")
-    x = torch.cat([f["up"], f["gate"]], dim=-1).to(dtype).to(gpu).requires_grad_(True)
+    x = torch.cat([f["up"], f["gate"]], dim=-1).to(dtype).to(gpu, copy=True).requires_grad_(True)
     y2 = swiglu_unchunked_cute(x, hip, hip, 256, 64, 256, 64)
     y2.backward(f["dy"].to(dtype).to(gpu))
     assert_close(y2.detach(), f["y"].to(dtype), dtype, "unchunked y")
@@ -244,8 +244,8 @@ def test_hip_rmsnorm_golden(gpu, dtype):
     announce("golden rmsnorm", dtype)
     f = load("rmsnorm")
     hip = KernelBackend.hip
-    x = f["x"].to(dtype).to(gpu).requires_grad_(True)
-    w = f["w"].to(dtype).to(gpu).requires_grad_(True)
+    x = f["x"].to(dtype).to(gpu, copy=True).requires_grad_(True)
+    w = f["w"].to(dtype).to(gpu, copy=True).requires_grad_(True)
     y = rmsnorm_cute(x, w, float(f["eps"]), False, hip, hip, 1, 1, 64, 64)
     y.backward(f["dy"].to(dtype).to(gpu))
     assert_close(y.detach(), f["y"].to(dtype), dtype, "y")
@@ -262,7 +262,7 @@ def test_hip_embedding_and_sort_golden(gpu, dtype):
     announce("golden embedding / sort", dtype)
     f = load("embedding")
     hip = KernelBackend.hip
-    table = f["table"].to(dtype).to(gpu).requires_grad_(True)
+    table = f["table"].to(dtype).to(gpu, copy=True).requires_grad_(True)
     out = embedding_cute(f["ids"].to(gpu), table, hip, hip, 4, 4, 64, 64)
     assert torch.equal(out.detach().cpu(), f["out"].to(dtype)), "gather must be a bit-exact copy"
     out.backward(f["dy"].to(dtype).to(gpu))
@@ -294,7 +294,7 @@ def test_hip_moe_golden(gpu, dtype):
         moe.gate.weight.copy_(f["w_gate"])
         moe.c_fc.weight.copy_(f["w_fc"])
         moe.c_proj.weight.copy_(f["w_proj"])
-    x = f["x"].to(dtype).to(gpu).requires_grad_(True)
+    x = f["x"].to(dtype).to(gpu, copy=True).requires_grad_(True)
     y, logits = moe(x)
     (y * f["dy"].to(dtype).to(gpu)).sum().backward()
     with torch.no_grad():

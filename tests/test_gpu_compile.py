@@ -27,21 +27,21 @@ def test_compiled_elementwise_ops(gpu, dtype):
 
     announce("compiled elementwise", dtype)
     g, u, dy = randn((64, 512), dtype, 1), randn((64, 512), dtype, 2), randn((64, 512), dtype, 3)
-    gg, ug = g.to(gpu).requires_grad_(True), u.to(gpu).requires_grad_(True)
+    gg, ug = g.to(gpu, copy=True).requires_grad_(True), u.to(gpu, copy=True).requires_grad_(True)
     y = torch.compile(swiglu_cute, fullgraph=True)(gg, ug)
     y.backward(dy.to(gpu))
     assert_close(y, O.swiglu_forward(g, u), dtype, "swiglu y")
     assert_close(gg.grad, O.swiglu_backward(g, u, dy)[0], dtype, "swiglu dg")
 
     x = randn((64, 1024), dtype, 4)
-    xg = x.to(gpu).requires_grad_(True)
+    xg = x.to(gpu, copy=True).requires_grad_(True)
     y = torch.compile(swiglu_unchunked_cute, fullgraph=True)(xg)
     y.backward(dy.to(gpu))
     assert_close(y, O.swiglu_unchunked_forward(x), dtype, "unchunked y")
     assert_close(xg.grad, O.swiglu_unchunked_backward(x, dy), dtype, "unchunked dx")
 
     w = randn((512,), dtype, 5, 0.1, 1.0)
-    xg, wg = g.to(gpu).requires_grad_(True), w.to(gpu).requires_grad_(True)
+    xg, wg = g.to(gpu, copy=True).requires_grad_(True), w.to(gpu, copy=True).requires_grad_(True)
     y = torch.compile(rmsnorm_cute, fullgraph=True)(xg, wg, 1e-5)
     y.backward(dy.to(gpu))
     assert_close(y, O.rmsnorm_forward(g, w, 1e-5)[0], dtype, "rmsnorm y")
@@ -52,7 +52,7 @@ def test_compiled_elementwise_ops(gpu, dtype):
     ids = torch.randint(0, 300, (4, 33), generator=torch.Generator().manual_seed(6))
     table = randn((300, 512), dtype, 7, 0.02)
     d_out = randn((4, 33, 512), dtype, 8)
-    tg = table.to(gpu).requires_grad_(True)
+    tg = table.to(gpu, copy=True).requires_grad_(True)
     out = torch.compile(embedding_cute, fullgraph=True)(ids.to(gpu), tg)
     out.backward(d_out.to(gpu))
     assert torch.equal(out.cpu(), O.embedding_forward(ids, table))
@@ -65,12 +65,12 @@ def test_compiled_additions(gpu, dtype):
 
     announce("compiled additions", dtype)
     x, y, dz = randn((33, 517), dtype, 21), randn((33, 517), dtype, 22), randn((33, 517), dtype, 23)
-    xg, yg = x.to(gpu).requires_grad_(True), y.to(gpu).requires_grad_(True)
+    xg, yg = x.to(gpu, copy=True).requires_grad_(True), y.to(gpu, copy=True).requires_grad_(True)
     z = torch.compile(add_tensor_cute, fullgraph=True)(xg, yg)
     z.backward(dz.to(gpu))
     assert torch.equal(z.detach().cpu(), O.add_tensor(x, y))
     assert torch.equal(xg.grad.cpu(), dz) and torch.equal(yg.grad.cpu(), dz)
-    xs = x.to(gpu).requires_grad_(True)
+    xs = x.to(gpu, copy=True).requires_grad_(True)
     s = torch.compile(add_scalar_cute, fullgraph=True)(xs, 0.42)
     s.backward(dz.to(gpu))
     assert torch.equal(s.detach().cpu(), O.add_scalar(x, 0.42))
@@ -85,7 +85,7 @@ def test_compiled_residual_rmsnorm_and_router(gpu, dtype):
     announce("compiled residual rmsnorm / router", dtype)
     x, r, dy, ds = (randn((33, 520), dtype, 24 + i) for i in range(4))
     w = randn((520,), dtype, 28, 0.1, 1.0)
-    xg, rg, wg = x.to(gpu).requires_grad_(True), r.to(gpu).requires_grad_(True), w.to(gpu).requires_grad_(True)
+    xg, rg, wg = x.to(gpu, copy=True).requires_grad_(True), r.to(gpu, copy=True).requires_grad_(True), w.to(gpu, copy=True).requires_grad_(True)
     y, s = torch.compile(fused_residual_add_rmsnorm_cute, fullgraph=True)(xg, rg, wg, 1e-5)
     torch.autograd.backward([y, s], [dy.to(gpu), ds.to(gpu)])
     y_o, s_o = O.residual_rmsnorm_forward(x, r, w, 1e-5)
@@ -97,7 +97,7 @@ def test_compiled_residual_rmsnorm_and_router(gpu, dtype):
     assert_close(wg.grad, dw_o, dtype, "weight_grad")
 
     logits = randn((200, 16), dtype, 29)
-    lg = logits.to(gpu).requires_grad_(True)
+    lg = logits.to(gpu, copy=True).requires_grad_(True)
     weights, selected = torch.compile(router_topk_softmax, fullgraph=True)(lg, 4)
     dw_ = randn((200, 4), dtype, 30)
     weights.backward(dw_.to(gpu))
@@ -127,7 +127,7 @@ def test_compiled_moe(gpu, dtype, E):
     x, w_gate, w_fc, w_proj, dy = O.moe_inputs(T, H, I, E, dtype, seed=81)
     moe = build_moe(MoE_Triton, gpu, dtype, E, k, H, I, w_gate, w_fc, w_proj)
     compiled = torch.compile(moe, fullgraph=True)
-    xg = x.to(gpu).requires_grad_(True)
+    xg = x.to(gpu, copy=True).requires_grad_(True)
     y, _ = compiled(xg)
     (y * dy.to(gpu)).sum().backward()
     with torch.no_grad():

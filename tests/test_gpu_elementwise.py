@@ -24,8 +24,8 @@ def test_add_tensor_and_scalar(gpu, dtype, size):
 
     announce("add", dtype, size)
     x, y, dz = randn(size, dtype, 11, 3.0), randn(size, dtype, 12, 0.01), randn(size, dtype, 13)
-    xg = x.to(gpu).requires_grad_(True)
-    yg = y.to(gpu).requires_grad_(True)
+    xg = x.to(gpu, copy=True).requires_grad_(True)
+    yg = y.to(gpu, copy=True).requires_grad_(True)
     z = add_tensor_cute(xg, yg)
     z.backward(dz.to(gpu))
     assert z.dtype == dtype and z.shape == x.shape
@@ -37,7 +37,7 @@ def test_add_tensor_and_scalar(gpu, dtype, size):
         z2 = add_tensor_cute(xg, yg, kernel_backend=KernelBackend.cuda, vector_instruction_width=width, BLOCK_SIZE=1024)
         assert torch.equal(z2, z)
 
-    xs = x.to(gpu).requires_grad_(True)
+    xs = x.to(gpu, copy=True).requires_grad_(True)
     s = add_scalar_cute(xs, 0.42)
     s.mean().backward()
     assert torch.equal(s.detach().cpu(), O.add_scalar(x, 0.42))
@@ -76,8 +76,8 @@ def test_swiglu(gpu, dtype, size):
 
     announce("swiglu", dtype, size)
     gate, up, dy = randn(size, dtype, 1, 2.0), randn(size, dtype, 2), randn(size, dtype, 3)
-    g = gate.to(gpu).requires_grad_(True)
-    u = up.to(gpu).requires_grad_(True)
+    g = gate.to(gpu, copy=True).requires_grad_(True)
+    u = up.to(gpu, copy=True).requires_grad_(True)
     y = swiglu_cute(g, u)
     y.backward(dy.to(gpu))
     assert y.dtype == dtype and y.shape == gate.shape
@@ -127,7 +127,7 @@ def test_swiglu_unchunked(gpu, dtype, size):
     announce("swiglu_unchunked", dtype, size)
     x = randn(size, dtype, 6, 1.5)
     dy = randn(size[:-1] + (size[-1] // 2,), dtype, 7)
-    xg = x.to(gpu).requires_grad_(True)
+    xg = x.to(gpu, copy=True).requires_grad_(True)
     y = swiglu_unchunked_cute(xg)
     y.backward(dy.to(gpu))
     assert y.shape == dy.shape
@@ -152,8 +152,8 @@ def test_rmsnorm(gpu, dtype, has_weight, memory_efficient, size):
     w = randn((H,), dtype, 9, 0.1, 1.0) if has_weight else None
     dy = randn(size, dtype, 10)
     eps = 1e-5
-    xg = x.to(gpu).requires_grad_(True)
-    wg = w.to(gpu).requires_grad_(True) if has_weight else None
+    xg = x.to(gpu, copy=True).requires_grad_(True)
+    wg = w.to(gpu, copy=True).requires_grad_(True) if has_weight else None
     y = rmsnorm_cute(xg, wg, eps, memory_efficient=memory_efficient)
     y.backward(dy.to(gpu))
     y_ref, _ = O.rmsnorm_forward(x, w, eps)
@@ -174,8 +174,8 @@ def test_rmsnorm_config2_shape_slice_and_eps_default(gpu):
     dtype = torch.bfloat16
     x, w, dy = randn((2048, 4096), dtype, 11), randn((4096,), dtype, 12, 0.1, 1.0), randn((2048, 4096), dtype, 13)
     for eps in (1e-5, None):
-        xg = x.to(gpu).requires_grad_(True)
-        wg = w.to(gpu).requires_grad_(True)
+        xg = x.to(gpu, copy=True).requires_grad_(True)
+        wg = w.to(gpu, copy=True).requires_grad_(True)
         y = rmsnorm_cute(xg, wg, eps)
         y.backward(dy.to(gpu))
         assert_close(y, O.rmsnorm_forward(x, w, eps)[0], dtype, "y")
@@ -208,8 +208,8 @@ def test_fused_residual_add_rmsnorm(gpu, dtype, has_weight, memory_efficient, si
     eps = 1e-5
 
     def leaves():
-        return (x.to(gpu).requires_grad_(True), r.to(gpu).requires_grad_(True),
-                w.to(gpu).requires_grad_(True) if has_weight else None)
+        return (x.to(gpu, copy=True).requires_grad_(True), r.to(gpu, copy=True).requires_grad_(True),
+                w.to(gpu, copy=True).requires_grad_(True) if has_weight else None)
 
     xf, rf, wf = leaves()
     y, s = fused_residual_add_rmsnorm_cute(xf, rf, wf, eps, memory_efficient=memory_efficient)
@@ -255,7 +255,7 @@ def test_embedding(gpu, dtype, ids_shape, table):
     ids = torch.randint(0, V, ids_shape, generator=g)
     w = randn(table, dtype, 15, 0.02)
     dy = randn(ids_shape + (H,), dtype, 16)
-    wg = w.to(gpu).requires_grad_(True)
+    wg = w.to(gpu, copy=True).requires_grad_(True)
     out = embedding_cute(ids.to(gpu), wg)
     out.backward(dy.to(gpu))
     assert out.shape == ids_shape + (H,)
@@ -286,7 +286,7 @@ def test_embedding_duplicates(gpu, dtype, case):
         ids = torch.zeros((0,), dtype=torch.long)
     w = randn((V, H), dtype, 19, 0.02)
     dy = randn(tuple(ids.shape) + (H,), dtype, 20)
-    wg = w.to(gpu).requires_grad_(True)
+    wg = w.to(gpu, copy=True).requires_grad_(True)
     out = embedding_cute(ids.to(gpu), wg)
     out.backward(dy.to(gpu))
     assert torch.equal(out.cpu(), O.embedding_forward(ids, w))

@@ -454,7 +454,7 @@ def test_router_linear_topk_softmax(gpu, dtype, T, H, E, k):
     wide[:, :H] = x.to(gpu)
     for source in (x.to(gpu), wide[:, :H]):
         xg = source.detach().requires_grad_(True)
-        wg = w.to(gpu).requires_grad_(True)
+        wg = w.to(gpu, copy=True).requires_grad_(True)
         assert _C.router_forward_supported(xg, wg, k)
         logits, weights, selected = moe_router(xg, wg, k, fused=True)
         assert_close(logits, O.router_linear(x, w), dtype, "router logits")
@@ -519,7 +519,7 @@ def test_expert_bias_ops(gpu, dtype, T, k, E, N, empty):
     y = randn((M, N), dtype, seed=72)
     bias = randn((E, N), dtype, seed=73)
     # expert-grouped rows, then rows in (token, slot) order; a row stride wider than N in the second case
-    got = y.to(gpu)
+    got = y.to(gpu, copy=True)
     expert_bias_forward(got, bias.to(gpu), offsets.to(gpu))
     assert torch.equal(got.cpu(), O.expert_bias_forward(y, bias, offsets)), "grouped: one fp32 add, one rounding"
     wide = torch.zeros(M, N + 8, dtype=dtype, device=gpu)
@@ -555,7 +555,7 @@ def build_moe(cls, gpu, dtype, E, k, H, I, w_gate, w_fc, w_proj):
 
 
 def run_moe(moe, x, dy, gpu):
-    xg = x.to(gpu).requires_grad_(True)
+    xg = x.to(gpu, copy=True).requires_grad_(True)
     y, logits = moe(xg)
     (y * dy.to(gpu)).sum().backward()
     with torch.no_grad():
@@ -755,8 +755,8 @@ def test_moe_3d_input_and_weight_grad_layout(gpu):
     x, w_gate, w_fc, w_proj, dy = O.moe_inputs(6 * 50, 128, 64, 4, dtype, seed=71)
     moe = build_moe(MoE_Triton, gpu, dtype, 4, 2, 128, 64, w_gate, w_fc, w_proj)
     ref = build_moe(MoE_Torch, gpu, dtype, 4, 2, 128, 64, w_gate, w_fc, w_proj)
-    xg = x.view(6, 50, 128).to(gpu).requires_grad_(True)
-    xr = x.view(6, 50, 128).to(gpu).requires_grad_(True)
+    xg = x.view(6, 50, 128).to(gpu, copy=True).requires_grad_(True)
+    xr = x.view(6, 50, 128).to(gpu, copy=True).requires_grad_(True)
     y, logits = moe(xg)
     yr, logits_r = ref(xr)
     assert y.shape == (6, 50, 128) and logits.shape == (300, 4)
