@@ -65,6 +65,20 @@ __device__ __forceinline__ void mfma16_acc(f16x8_t a, f16x8_t b, f32x4_t& c) {
     asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
 
+// To the compiler the matrix instructions above are text: it does not count the wait states the hardware needs, and
+// does not interlock, between a matrix instruction's write of its result and a vector-ALU or memory instruction that
+// reads it (up to 18 for a 16-pass instruction) - and it is free to move such a read up to right behind them.  Called
+// behind the last matrix instruction, for every row of accumulators, before the results are read: the accumulators
+// pass through the statement, so no read of them can be scheduled ahead of it, and the first statement waits.
+template <bool WAIT>
+__device__ __forceinline__ void settle_matrix_results(f32x4_t (&c)[8]) {
+    if (WAIT)
+        asm volatile("s_nop 15\n\ts_nop 15"
+                     : "+a"(c[0]), "+a"(c[1]), "+a"(c[2]), "+a"(c[3]), "+a"(c[4]), "+a"(c[5]), "+a"(c[6]), "+a"(c[7]));
+    else
+        asm volatile("" : "+a"(c[0]), "+a"(c[1]), "+a"(c[2]), "+a"(c[3]), "+a"(c[4]), "+a"(c[5]), "+a"(c[6]), "+a"(c[7]));
+}
+
 }  // namespace ck
 
 #endif  // CK_GEMM_PRIMS_H

@@ -998,6 +998,12 @@ __global__ void __launch_bounds__(TL::THREADS) CK_WAVES_PER_SIMD(TL::WM * TL::WN
     }
 #undef CK_M_END
 #undef CK_PHASE_END
+    if constexpr (NWAVES == 4 && MODE != 2) {  // (the eight-wave loop's matrix instructions are builtins: the compiler counts)
+        static_assert(NWAVES != 4 || TN == 8, "one statement per row of eight accumulators");
+        settle_matrix_results<true>(acc[0]);
+#pragma unroll
+        for (int i = 1; i < TM; ++i) settle_matrix_results<false>(acc[i]);
+    }
 
     // ---- pieces of a split tile ------------------------------------------------------------------------
     // A partial tile is stored the way the accumulators lie in the registers: float4 number

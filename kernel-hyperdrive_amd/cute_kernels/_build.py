@@ -80,7 +80,9 @@ def kernel_resources(source: str, loops: bool = False) -> dict[str, dict[str, in
     Scratch above zero means the kernel spills registers to memory.  With ``loops``, the device assembly of the same
     compilation is read as well and every kernel gets ``"loops"``: one dict per innermost loop that holds matrix
     instructions, counting them ("mfma") and what must not sit beside them - scratch accesses ("scratch") and copies
-    between the two halves of the register file ("acc_moves") - plus LDS reads, direct-to-LDS copies and barriers."""
+    between the two halves of the register file ("acc_moves") - plus LDS reads, direct-to-LDS copies and barriers; and
+    ``"unsettled"``: the instructions that touch an accumulation register fewer than 19 wait states behind a matrix
+    instruction issued through ``asm`` on some path (see ``_unsettled_accumulator_accesses``)."""
     import re
     import tempfile
 
@@ -118,6 +120,7 @@ def kernel_resources(source: str, loops: bool = False) -> dict[str, dict[str, in
                 if m and labels.get(m.group(1), i) < i:
                     spans.append((labels[m.group(1)], i))
             innermost = [s for s in spans if not any(o != s and s[0] <= o[0] and o[1] <= s[1] for o in spans)]
+            found[kernel]["unsettled"] = _unsettled_accumulator_accesses(body)
             found[kernel]["loops"] = []
             for lo, hi in innermost:
                 text = body[lo:hi]
@@ -127,6 +130,88 @@ def kernel_resources(source: str, loops: bool = False) -> dict[str, dict[str, in
                         "mfma": count("v_mfma"), "scratch": count("scratch_"), "acc_moves": count("v_accvgpr"),
                         "lds_reads": count("ds_read"), "copies": count("global_load_lds"), "barriers": count("s_barrier"),
                     })
+    return found
+
+
+def _unsettled_accumulator_accesses(body: list[str], settled: int = 19) -> list[str]:
+    """A matrix instruction writes its result several passes after it issues, and the hardware does not hold back a
+    vector-ALU or memory instruction that reads (or overwrites) the register earlier: the compiler counts wait states
+    and pads with ``s_nop`` - for the matrix instructions it knows.  One written in ``asm`` is text to it.  This walks
+    the control-flow graph of one kernel's assembly and reports every instruction other than a matrix instruction that
+    names an accumulation register and can be reached from an ``asm`` matrix instruction in fewer than ``settled`` wait
+    states (one per instruction, ``s_nop n`` counting n + 1; 18 is the longest requirement, of a 16-pass instruction)."""
+    import re
+
+    blocks: list[dict] = [{"label": None, "code": []}]
+    in_asm = False
+    for line in body[1:]:
+        text = line.split(";")[0].rstrip() if not line.lstrip().startswith(";;#") else line.strip()
+        if text.startswith(";;#ASMSTART"):
+            in_asm = True
+            continue
+        if text.startswith(";;#ASMEND"):
+            in_asm = False
+            continue
+        if match := re.match(r"^(\.LBB\d+_\d+):", line):
+            blocks.append({"label": match.group(1), "code": []})
+            continue
+        if not line.startswith("\t") or not text.strip() or text.strip().startswith("."):
+            continue
+        blocks[-1]["code"].append((text.strip(), in_asm))
+        if re.match(r"^(s_branch|s_cbranch_\w+|s_endpgm|s_setpc_b64)\b", text.strip()):
+            blocks.append({"label": None, "code": []})
+    index = {b["label"]: i for i, b in enumerate(blocks) if b["label"]}
+    successors: list[list[int]] = []
+    for i, b in enumerate(blocks):
+        last = b["code"][-1][0] if b["code"] else ""
+        nxt = [i + 1] if i + 1 < len(blocks) else []
+        if match := re.match(r"^s_branch (\S+)", last):
+            successors.append([index[match.group(1)]] if match.group(1) in index else [])
+        elif match := re.match(r"^s_cbranch_\w+ (\S+)", last):
+            successors.append(nxt + ([index[match.group(1)]] if match.group(1) in index else []))
+        elif re.match(r"^(s_endpgm|s_setpc_b64)", last):
+            successors.append([])
+        else:
+            successors.append(nxt)
+
+    def registers(text: str) -> set[int]:
+        named: set[int] = set()
+        for lo, hi in re.findall(r"\ba\[(\d+):(\d+)\]", text):
+            named.update(range(int(lo), int(hi) + 1))
+        named.update(int(n) for n in re.findall(r"\ba(\d+)\b", text))
+        return named
+
+    # state: accumulation register -> wait states since an asm matrix instruction wrote it (absent: settled)
+    def walk(i: int, state: dict[int, int], report: list[str] | None) -> dict[int, int]:
+        state = dict(state)
+        for text, from_asm in blocks[i]["code"]:
+            if text.startswith("v_mfma"):
+                if from_asm:
+                    for reg in registers(text.split(",")[0]):
+                        state[reg] = 0
+                    continue
+            elif state and report is not None:
+                early = {reg: state[reg] for reg in registers(text) if reg in state}
+                if early:
+                    report.append(f"{text}  ({min(early.values())} wait states behind the matrix instruction that wrote it)")
+            step = int(text.split()[1]) + 1 if text.startswith("s_nop") else 1
+            state = {reg: d + step for reg, d in state.items() if d + step < settled}
+        return state
+
+    entry: list[dict[int, int]] = [{} for _ in blocks]
+    changed = True
+    while changed:
+        changed = False
+        for i in range(len(blocks)):
+            out = walk(i, entry[i], None)
+            for j in successors[i]:
+                for reg, d in out.items():
+                    if d < entry[j].get(reg, settled):
+                        entry[j][reg] = d
+                        changed = True
+    found: list[str] = []
+    for i in range(len(blocks)):
+        walk(i, entry[i], found)
     return found
 
 

@@ -63,6 +63,8 @@ inline void wait_copies() {
 }
 inline int opaque(int v) { return v; }
 inline uint64_t opaque_s64(uint64_t v) { return v; }
+template <bool WAIT>
+inline void settle_matrix_results(f32x4_t (&)[8]) {}
 inline void mfma16_acc(bf16x8_t a, bf16x8_t b, f32x4_t& c) { c = emu_mfma16(a, b, c); }
 inline void mfma16_acc(f16x8_t a, f16x8_t b, f32x4_t& c) { c = emu_mfma16(a, b, c); }
 }  // namespace ck

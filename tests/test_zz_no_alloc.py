@@ -55,6 +55,14 @@ def test_moe_sort_noalloc_matches_moe_sort(gpu, dtype):
         expected = _reference_sort(lib, ids, E, stream)
         got = [torch.full((M,), -1, dtype=torch.int64, device=gpu) for _ in range(2)]
         offsets = torch.full((E,), -1, dtype=torch.int64, device=gpu)
+        # Once unmeasured with this case's shape, so that whatever the runtime sets up lazily for a launch configuration
+        # it has not seen (argument buffers, code) exists before the measured call; a library that allocated per call
+        # would do so again there.
+        assert lib.ck_moe_sort_noalloc(ids.data_ptr(), int(dtype == torch.int32), got[0].data_ptr(), got[1].data_ptr(),
+                                       offsets.data_ptr(), M, E, stream) == 0
+        torch.cuda.synchronize()
+        for t in (*got, offsets):
+            t.fill_(-1)
         torch.cuda.synchronize()
         # torch's allocator counters see nothing the library would allocate by itself; the driver's count of free
         # device memory does
