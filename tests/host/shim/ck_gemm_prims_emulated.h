@@ -3,6 +3,7 @@
 // header through that header's include guard.
 #pragma once
 #define CK_GEMM_PRIMS_H
+#define CK_GEMM_PRIMS_HOST  // (a source can tell that it is being built against these models)
 #define CK_WAVES_PER_SIMD(n)
 
 #include <hip/hip_runtime.h>
