@@ -103,6 +103,9 @@ int ck_rmsnorm_backward(const void* x, const void* weight, const void* output_gr
  *   forward : output[i, :] = weight[ids[i], :]  (bit-exact copy; an id outside [0, V) yields a zero row)
  *   backward: weight_grad[V, H] is written completely (rows no id selects become zero); duplicates are
  *             accumulated in fp32 in ascending token position and rounded once.
+ *             (CK_EMBEDDING_BWD_PRELUDE=short in the environment, read at every call, sorts the ids in one
+ *             workgroup behind two small launches instead of seven grid-wide ones, for up to 131072 ids; the
+ *             results are the same bits.)
  * ------------------------------------------------------------------------------------------- */
 int ck_embedding_forward(const void* ids, int ids_are_i32, const void* weight, void* output,
                          int64_t num_ids, int64_t V, int64_t H, int dtype, void* stream);

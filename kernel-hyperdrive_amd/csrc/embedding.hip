@@ -19,6 +19,8 @@
 //               3. combine kernel: sums the partial rows of each long run and stores the dW row.
 //             No floating-point atomics, deterministic.  Of the rows that receive a sum, only those inside the two
 //             ranges cleared before the marks exist are written twice.
+#include <cstdlib>
+
 #include "ck_block_sort.h"
 #include "ck_grid_sort.h"
 
@@ -232,14 +234,10 @@ __global__ void __launch_bounds__(256)
 // first one, else by a 64-way search), then walks its slots 64 at a time carrying the latest head forward with a wave
 // max-scan.
 constexpr int kRunsWaveSlots = 4 * CK_WAVE;
-__global__ void __launch_bounds__(256)
-    embedding_runs_kernel(const uint32_t* __restrict__ skeys, uint32_t* __restrict__ run_head, int n, FillJob fill) {
-    if (run_fill_job(fill)) return;
+// the slots [begin, end) of one wave
+__device__ __forceinline__ void run_heads_of_range(const uint32_t* __restrict__ skeys, uint32_t* __restrict__ run_head,
+                                                   int begin, int end) {
     const int lane = lane_id();
-    const int gw = (blockIdx.x * blockDim.x + threadIdx.x) / CK_WAVE;
-    const int begin = gw * kRunsWaveSlots;
-    if (begin >= n) return;
-    const int end = min(begin + kRunsWaveSlots, n);
     // head of the run that contains slot `begin`: the last slot j <= begin with skeys[j - 1] != skeys[j]
     int carry = -1;
     const uint32_t first_key = skeys[begin];
@@ -279,6 +277,80 @@ __global__ void __launch_bounds__(256)
         if (i < end) run_head[i] = (uint32_t)incl;
         carry = __shfl(incl, CK_WAVE - 1, CK_WAVE);
     }
+}
+
+__global__ void __launch_bounds__(256)
+    embedding_runs_kernel(const uint32_t* __restrict__ skeys, uint32_t* __restrict__ run_head, int n, FillJob fill) {
+    if (run_fill_job(fill)) return;
+    const int gw = (blockIdx.x * blockDim.x + threadIdx.x) / CK_WAVE;
+    const int begin = gw * kRunsWaveSlots;
+    if (begin >= n) return;
+    run_heads_of_range(skeys, run_head, begin, min(begin + kRunsWaveSlots, n));
+}
+
+// ---- backward 1, the short form: three launches instead of seven ----------------------------------------------------
+// For the id counts this operator sees (tens of thousands) one workgroup sorts the pairs in tens of microseconds
+// (ck_block_sort.h: three passes of 6 bits for a 17-bit vocabulary, all in one launch, then the run heads), which is
+// less than the zero fill needs anyway: the launch's other workgroups carry all of the fill that is left, in one
+// piece and at the rate of a plain fill, where the seven launches of the grid-wide sort each pay a ramp up and down.
+// Before it, two small launches clear and set the row marks (and carry an unconditional share of the fill each).
+__global__ void __launch_bounds__(256)
+    embedding_clear_marks_kernel(uint32_t* __restrict__ clear, int64_t clear_words, FillJob fill) {
+    if (run_fill_job(fill)) return;
+    const int64_t own = min((int64_t)gridDim.x, (int64_t)fill.first_block);
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < clear_words; i += own * blockDim.x) clear[i] = 0u;
+}
+
+template <bool I32>
+__global__ void __launch_bounds__(256)
+    embedding_mark_kernel(IdLoader<I32> load, int n, int64_t V, uint8_t* __restrict__ touched, FillJob fill) {
+    if (run_fill_job(fill)) return;
+    const int64_t own = min((int64_t)gridDim.x, (int64_t)fill.first_block);
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += own * blockDim.x) {
+        uint32_t key, val;
+        load((int)i, key, val);
+        if ((int64_t)key < V) touched[key] = 1;
+    }
+}
+
+// Workgroup 0 sorts (id, position) by id - the sorted pairs end in keys[(passes - 1) & 1] / vals[(passes - 1) & 1], as
+// the grid-wide sort leaves them - and records the run heads; the others fill.
+template <bool I32>
+__global__ void __launch_bounds__(kSortThreads)
+    embedding_block_sort_kernel(IdLoader<I32> first_load, uint32_t* keys0, uint32_t* vals0, uint32_t* keys1, uint32_t* vals1,
+                                uint32_t* __restrict__ run_head, int n, int key_bits, FillJob fill) {
+    __shared__ SortShared sh;
+    if (run_fill_job(fill)) return;
+    const int passes = ck_sort_passes(key_bits);
+    const int bits_per_pass = (key_bits + passes - 1) / passes;
+    uint32_t* kbuf[2] = {keys0, keys1};
+    uint32_t* vbuf[2] = {vals0, vals1};
+    for (int p = 0; p < passes; ++p) {
+        const int shift = p * bits_per_pass;
+        const int bits = min(bits_per_pass, key_bits - shift);
+        const bool first = p == 0;
+        const uint32_t* kin = kbuf[(p + 1) & 1];
+        const uint32_t* vin = vbuf[(p + 1) & 1];
+        uint32_t* kout = kbuf[p & 1];
+        uint32_t* vout = vbuf[p & 1];
+        auto load = [&](int i, uint32_t& k, uint32_t& v) {
+            if (first) {
+                first_load(i, k, v);
+            } else {
+                k = kin[i];
+                v = vin[i];
+            }
+        };
+        auto store = [&](int pos, uint32_t k, uint32_t v) {
+            kout[pos] = k;
+            vout[pos] = v;
+        };
+        block_radix_pass(sh, n, shift, bits, load, store);
+    }
+    const uint32_t* skeys = kbuf[(passes - 1) & 1];
+    const int wave = threadIdx.x / CK_WAVE;
+    for (int begin = wave * kRunsWaveSlots; begin < n; begin += kSortWaves * kRunsWaveSlots)
+        run_heads_of_range(skeys, run_head, begin, min(begin + kRunsWaveSlots, n));
 }
 
 // ---- backward 2: one launch for the two row-wise jobs ---------------------------------------------
@@ -556,6 +628,14 @@ extern "C" int64_t ck_embedding_backward_workspace_size(int64_t num_ids, int64_t
 // 60 / 80 / 100 / 120 / 150 MB each; Zipf(1.1) ids 352 / 343 / 339 / 338 / 339 us)
 constexpr int64_t kCarrierFillBytes = (int64_t)100 << 20;
 
+// ids the one-workgroup sort of the short prelude takes (beyond that the grid-wide sort is the faster one by far)
+constexpr int kBlockSortMaxIds = 1 << 17;
+// CK_EMBEDDING_BWD_PRELUDE=short selects the three-launch prelude where it applies (default: the grid-wide sort)
+static int embedding_backward_prelude() {
+    const char* v = getenv("CK_EMBEDDING_BWD_PRELUDE");
+    return v && v[0] == 's' ? 1 : 0;
+}
+
 template <typename T, int VEC>
 static void launch_bwd(hipStream_t s, const ck::EmbWorkspace& ws, int passes, const void* dy, void* dw, int n,
                        int64_t V, int64_t H, int64_t fill_begin) {
@@ -606,6 +686,40 @@ extern "C" int ck_embedding_backward(const void* ids, int ids_are_i32, const voi
     // from the row-sum launch, where the fill hides the latency of the sums, to here
     int64_t spread_rows = spread_fill ? carriers * (kCarrierFillBytes / row_bytes) : 0;
     if (spread_rows > V) spread_rows = V;
+    const bool short_prelude = spread_fill && n <= kBlockSortMaxIds && embedding_backward_prelude() == 1;
+    if (short_prelude) {
+        // clear marks | set marks | sort + run heads, with the fill on all three: an unconditional share on each of the
+        // first two (the marks do not exist yet), everything else - by the marks - on the third
+        const int64_t share = kCarrierFillBytes / row_bytes < V / 2 ? kCarrierFillBytes / row_bytes : V / 2;
+        ck::FillJob f = {nullptr, (char*)weight_grad, row_bytes, 0, share, 4};
+        hipLaunchKernelGGL(ck::embedding_clear_marks_kernel, dim3((unsigned)(4 + ck::fill_job_blocks(share, 256))), dim3(256),
+                           0, s, (uint32_t*)ws.touched, clear_words, f);
+        const int mark_own = (int)ck_ceil_div(n, 4 * 256);
+        const unsigned mark_grid = (unsigned)(mark_own + ck::fill_job_blocks(share, 256));
+        const unsigned sort_grid_1 = (unsigned)(1 + ck::fill_job_blocks(V - 2 * share, ck::kSortThreads));
+        const ck::FillJob mark_fill = {nullptr, (char*)weight_grad, row_bytes, share, 2 * share, mark_own};
+        const ck::FillJob sort_fill = {ws.touched, (char*)weight_grad, row_bytes, 2 * share, V, 1};
+        if (ids_are_i32) {
+            const ck::IdLoader<true> load = {ids, V};
+            hipLaunchKernelGGL(ck::embedding_mark_kernel<true>, dim3(mark_grid), dim3(256), 0, s, load, n, V, ws.touched,
+                               mark_fill);
+            hipLaunchKernelGGL(ck::embedding_block_sort_kernel<true>, dim3(sort_grid_1), dim3(ck::kSortThreads), 0, s, load,
+                               ws.keys[0], ws.vals[0], ws.keys[1], ws.vals[1], ws.run_head, n, key_bits, sort_fill);
+        } else {
+            const ck::IdLoader<false> load = {ids, V};
+            hipLaunchKernelGGL(ck::embedding_mark_kernel<false>, dim3(mark_grid), dim3(256), 0, s, load, n, V, ws.touched,
+                               mark_fill);
+            hipLaunchKernelGGL(ck::embedding_block_sort_kernel<false>, dim3(sort_grid_1), dim3(ck::kSortThreads), 0, s, load,
+                               ws.keys[0], ws.vals[0], ws.keys[1], ws.vals[1], ws.run_head, n, key_bits, sort_fill);
+        }
+        const int sort_passes = ck::ck_sort_passes(key_bits);
+        CK_DISPATCH_DTYPE(dtype, {
+            const bool vec = ck_aligned16(weight_grad) && (!output_grad || ck_aligned16(output_grad)) && (H % T::kVec == 0);
+            if (vec) launch_bwd<T, T::kVec>(s, ws, sort_passes, output_grad, weight_grad, (int)num_ids, V, H, V);
+            else launch_bwd<T, 1>(s, ws, sort_passes, output_grad, weight_grad, (int)num_ids, V, H, V);
+        });
+        return ck_launch_status();
+    }
     int carrier = 0;
     auto fill_share = [&](int own_blocks, int threads, unsigned& grid, bool marks_known = true) {
         ck::FillJob f = {marks_known ? ws.touched : nullptr, (char*)weight_grad, row_bytes, 0, 0, 0x7fffffff};

@@ -10,6 +10,8 @@ cannot: timing, the memory model between workgroups (they run one after the othe
 corner cases - the GPU tests stay the parity tests proper, and the emulation's own models are checked against them by
 the kernels whose GPU results are already pinned."""
 
+import inspect
+
 import pytest
 import torch
 
@@ -17,6 +19,7 @@ import test_golden as G
 import test_gpu_elementwise as E
 import test_gpu_moe as M
 import test_gpu_moe_int as I
+import wip_embedding_short_prelude as S
 import wip_four_wave as W
 from host import emulated_library
 
@@ -126,9 +129,16 @@ case(W.test_scatter2scatter_four_waves, dtype=F16, w_layout="n_contiguous", mode
 case(W.test_fused_swiglu_products_four_waves, dtype=BF16, shape=(300, 2, 3, 192, 128))
 case(W.test_group_bwd_W_four_waves, dtype=BF16, dw_layout="k_contiguous", shape=(300, 2, 3, 256, 256, ()))
 
+# ---- the short prelude of the embedding backward against the default one, bit for bit ---------------------------------------
+for dtype, kind, table in [(BF16, "zipf", (5000, 1024)), (F32, "one_row", (300, 64)), (BF16, "outside", (131072 + 9, 8)),
+                           (BF16, "int32", (5000, 1024)), (F32, "single", (300, 64))]:
+    case(S.test_short_prelude_equals_the_default, dtype=dtype, kind=kind, table=table)
+
 
 @pytest.mark.parametrize("function,arguments", CASES)
-def test_gpu_test_body_on_the_emulated_device(emulated, function, arguments):
+def test_gpu_test_body_on_the_emulated_device(emulated, monkeypatch, function, arguments):
+    if "monkeypatch" in inspect.signature(function).parameters:
+        arguments = dict(arguments, monkeypatch=monkeypatch)
     function(emulated, **arguments)
 
 
