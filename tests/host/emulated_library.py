@@ -33,7 +33,7 @@ def build(directory: str, sources=None) -> str:
     compiler = host_clang()
     if compiler is None:
         raise RuntimeError("no clang of the ROCm toolchain to build the host emulation with")
-    sources = sorted(sources or glob.glob(os.path.join(CSRC, "*.hip")))
+    sources = sorted(sources or glob.glob(os.path.join(CSRC, "*.hip"))) + [os.path.join(HOST_DIR, "emulated_support.cpp")]
     objects = [os.path.join(directory, os.path.basename(s) + ".o") for s in sources]
 
     def compile_one(pair):

@@ -14,6 +14,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <functional>
+#include <memory>
 #include <vector>
 
 #define __global__
@@ -62,6 +63,7 @@ inline float4 make_float4(float x, float y, float z, float w) { return float4{x,
 namespace emu {
 constexpr int kWave = 64;
 constexpr int kMaxLanes = 1024;
+constexpr size_t kStackBytes = 512 * 1024;
 
 struct Group {
     int arrived = 0, generation = 0, members = 0;
@@ -75,7 +77,7 @@ struct Wave {
 };
 struct Lane {
     ucontext_t context;
-    std::vector<char> stack;
+    std::unique_ptr<char[]> stack;  // (not a vector: its pages are touched only as deep as the lane's calls go)
     bool done = true;
     const Group* waits_for = nullptr;  // the group whose next generation this lane sleeps until
     int waits_since = 0;
@@ -127,6 +129,14 @@ inline void trampoline() {
 // hook of the harness, called once per workgroup after its last lane has left the kernel
 inline std::function<void()> g_after_block;
 
+inline bool lanes_reversed() {  // read once, when the first workgroup runs
+    static const bool reversed = [] {
+        const char* order = std::getenv("EMU_LANE_ORDER");
+        return order != nullptr && order[0] == 'r';
+    }();
+    return reversed;
+}
+
 inline void run_block(int threads) {
     g_threads = threads;
     g_block = Group{};
@@ -137,19 +147,23 @@ inline void run_block(int threads) {
     }
     for (int l = 0; l < threads; ++l) {
         Lane& lane = g_lanes[l];
-        if (lane.stack.empty()) lane.stack.resize(512 * 1024);
+        if (!lane.stack) lane.stack.reset(new char[kStackBytes]);
         getcontext(&lane.context);
-        lane.context.uc_stack.ss_sp = lane.stack.data();
-        lane.context.uc_stack.ss_size = lane.stack.size();
+        lane.context.uc_stack.ss_sp = lane.stack.get();
+        lane.context.uc_stack.ss_size = kStackBytes;
         lane.context.uc_link = &g_main;
         makecontext(&lane.context, trampoline, 0);
         lane.done = false;
         lane.waits_for = nullptr;
     }
+    // The order in which the runnable lanes get their turn is free on the hardware; a result that depends on it is a
+    // race.  EMU_LANE_ORDER=reverse runs the last lane first (default: the first lane first).
+    const bool reversed = lanes_reversed();
     for (bool any = true; any;) {
         any = false;
         bool progress = false;
-        for (int l = 0; l < threads; ++l) {
+        for (int turn = 0; turn < threads; ++turn) {
+            const int l = reversed ? threads - 1 - turn : turn;
             Lane& lane = g_lanes[l];
             if (lane.done) continue;
             any = true;
