@@ -32,7 +32,8 @@ def gpu(request, tmp_path_factory):
 
         if emulated_library.host_clang() is None:
             pytest.skip("no clang of the ROCm toolchain to build the host emulation with")
-        binding = emulated_library.bound_to(emulated_library.build(str(tmp_path_factory.mktemp("emulated_library"))))
+        binding = emulated_library.bound_to(emulated_library.build(str(tmp_path_factory.mktemp("emulated_library"))),
+                                            guarded=True)
         binding.__enter__()
         request.addfinalizer(lambda: binding.__exit__(None, None, None))
         return torch.device("cpu")

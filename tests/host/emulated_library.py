@@ -47,19 +47,91 @@ def build(directory: str, sources=None) -> str:
     return library
 
 
+_libc = ctypes.CDLL(None, use_errno=True)
+_libc.mmap.restype = ctypes.c_void_p
+_libc.mmap.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_long]
+_libc.mprotect.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+_libc.munmap.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
+_PAGE = 4096
+
+
+class _GuardedCall:
+    """One call into the library with every tensor moved, for its length, to memory that ends (within 15 bytes: the
+    pointer keeps its alignment modulo 16, which the entry points branch on) at a page nobody may touch - or, with
+    `before`, that begins right behind one: a kernel that
+    reads or writes past the end of an operand - what faults a GPU, or silently corrupts a neighbour - ends the process
+    with a segmentation fault here, and faulthandler names the test.  The contents travel back when the call returns."""
+
+    def __init__(self, before: bool = False):
+        self.before = before  # the inaccessible page lies before the operand instead of behind it
+        self.regions = []  # (first byte, end) of the tensor's storage range, address of its guarded copy, mapping, size
+
+    def pointer(self, t):
+        if t is None:
+            return None
+        if t.numel() == 0:
+            return t.data_ptr()
+        nbytes = (sum((size - 1) * stride for size, stride in zip(t.shape, t.stride())) + 1) * t.element_size()
+        lo, hi = t.data_ptr(), t.data_ptr() + nbytes
+        for first, end, copy, _, _ in self.regions:
+            if first <= lo and hi <= end:
+                return copy + (lo - first)
+            if lo < end and first < hi:
+                raise RuntimeError("two operands of one call overlap in part: the guarded copies cannot stand for both")
+        pages = (nbytes + 16 + _PAGE - 1) // _PAGE
+        size = (pages + 1) * _PAGE
+        mapping = _libc.mmap(None, size, 3, 0x22, -1, 0)  # PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS
+        if mapping in (None, ctypes.c_void_p(-1).value):
+            raise MemoryError("mmap")
+        fence = mapping if self.before else mapping + pages * _PAGE
+        if _libc.mprotect(fence, _PAGE, 0) != 0:
+            raise OSError(ctypes.get_errno(), "mprotect")
+        if self.before:
+            copy = mapping + _PAGE + lo % 16
+        else:
+            copy = fence - nbytes
+            copy -= (copy - lo) % 16
+        ctypes.memmove(copy, lo, nbytes)
+        self.regions.append((lo, hi, copy, mapping, size))
+        return copy
+
+    def finish(self):
+        for first, end, copy, mapping, size in self.regions:
+            ctypes.memmove(first, copy, end - first)
+            _libc.munmap(mapping, size)
+        self.regions = []
+
+
+_current_call = None
+
+
 class _HostLaunch:
     """Stands in for the binding's launch context: no device to make current, no stream."""
 
     stream = None
+    guarded = False  # False, True / "behind", or "before": where the inaccessible page lies
 
     def __init__(self, *tensors):
         pass
 
     def __enter__(self):
+        global _current_call
+        if self.guarded:
+            _current_call = _GuardedCall(before=self.guarded == "before")
         return self
 
     def __exit__(self, *exc):
+        global _current_call
+        if _current_call is not None:
+            _current_call.finish()
+            _current_call = None
         return False
+
+
+def _pointer(t):
+    if _current_call is not None:
+        return _current_call.pointer(t)
+    return None if t is None else t.data_ptr()
 
 
 def _with_aligned_workspace(function, pointer_at: int, bytes_at: int):
@@ -78,8 +150,10 @@ def _with_aligned_workspace(function, pointer_at: int, bytes_at: int):
 
 
 @contextlib.contextmanager
-def bound_to(library: str):
-    """While active, the package's ctypes binding (cute_kernels._C) calls the emulated library and takes CPU tensors."""
+def bound_to(library: str, guarded=False):
+    """While active, the package's ctypes binding (cute_kernels._C) calls the emulated library and takes CPU tensors.
+    `guarded` (True or "before"): every operand of every call sits in front of an inaccessible page, or right behind
+    one (see _GuardedCall)."""
     from cute_kernels import _C
 
     lib = ctypes.CDLL(library)
@@ -90,12 +164,13 @@ def bound_to(library: str):
     from cute_kernels.cutotune import tuner
 
     lib.ck_embedding_backward = _with_aligned_workspace(lib.ck_embedding_backward, 4, 5)
-    saved = (_C._lib, _C._Launch, _C.rmsnorm_backward_workspace_size, tuner._DISABLE_CUTOTUNE)
-    _C._lib, _C._Launch = lib, _HostLaunch
+    saved = (_C._lib, _C._Launch, _C.rmsnorm_backward_workspace_size, tuner._DISABLE_CUTOTUNE, _C._ptr, _HostLaunch.guarded)
+    _C._lib, _C._Launch, _C._ptr, _HostLaunch.guarded = lib, _HostLaunch, _pointer, guarded
     _C.rmsnorm_backward_workspace_size = lambda B, H, device: lib.ck_rmsnorm_backward_workspace_size(B, H)
     # nothing to time here: every tuned launcher takes its default configuration (the tests name other ones explicitly)
     tuner._DISABLE_CUTOTUNE = True
     try:
         yield lib
     finally:
-        _C._lib, _C._Launch, _C.rmsnorm_backward_workspace_size, tuner._DISABLE_CUTOTUNE = saved
+        (_C._lib, _C._Launch, _C.rmsnorm_backward_workspace_size, tuner._DISABLE_CUTOTUNE, _C._ptr,
+         _HostLaunch.guarded) = saved

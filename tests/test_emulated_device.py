@@ -5,6 +5,9 @@ they do to the 64 lanes), linked into a library with the same C entry points, an
 binding.  The bodies of the GPU tests then run unchanged on CPU tensors - the same Python launchers, autograd functions
 and layer, the same device code, the same oracle and tolerances - at shapes the emulation finishes in seconds.
 
+Every operand of every call sits in front of an inaccessible page, so a kernel that walked past the end of one would
+end the run with a segmentation fault.
+
 What this pins: the device code's arithmetic and indexing, lane for lane, and every place where lanes meet.  What it
 cannot: timing, the memory model between workgroups (they run one after the other here) and the real instructions'
 corner cases - the GPU tests stay the parity tests proper, and the emulation's own models are checked against them by
@@ -14,6 +17,9 @@ import ctypes
 import inspect
 import os
 import shutil
+import signal
+import subprocess
+import sys
 
 import pytest
 import torch
@@ -40,7 +46,7 @@ def library(tmp_path_factory):
 @pytest.fixture
 def emulated(library):
     """The binding points at the emulated library for the length of one test only."""
-    with emulated_library.bound_to(library):
+    with emulated_library.bound_to(library, guarded=True):
         yield torch.device("cpu")
 
 
@@ -73,7 +79,7 @@ def library_with_lanes_reversed(library, tmp_path_factory):
 def emulated_lanes_reversed(library_with_lanes_reversed):
     """The hardware leaves the order of the lanes open between the points where they meet, so a result that changes
     with it is a race."""
-    with emulated_library.bound_to(library_with_lanes_reversed):
+    with emulated_library.bound_to(library_with_lanes_reversed, guarded="before"):  # (the page before the operands here)
         yield torch.device("cpu")
 
 
@@ -189,6 +195,31 @@ def test_results_do_not_depend_on_the_order_of_the_lanes(emulated_lanes_reversed
     if "monkeypatch" in inspect.signature(function).parameters:
         arguments = dict(arguments, monkeypatch=monkeypatch)
     function(emulated_lanes_reversed, **arguments)
+
+
+def test_the_guard_page_ends_a_call_that_reads_past_an_operand(library):
+    """The tests above run with every operand in front of an inaccessible page (emulated_library._GuardedCall).  That
+    this does end a kernel that walks past the end of an operand is shown here, in a process of its own: an addition
+    told that its operands are 4096 elements longer than they are dies of a segmentation fault, the honest call does
+    not."""
+    program = f"""
+import ctypes, sys, torch
+sys.path[:0] = {[os.path.dirname(os.path.abspath(__file__)), os.path.join(os.path.dirname(os.path.abspath(__file__)), "host")]!r}
+import conftest, emulated_library
+from cute_kernels import _C
+with emulated_library.bound_to({library!r}, guarded=True) as lib:
+    call = emulated_library._GuardedCall()
+    x, y, out = torch.ones(1000), torch.ones(1000), torch.zeros(1000)
+    pointers = [call.pointer(t) for t in (x, y, out)]
+    extra = int(sys.argv[1])
+    status = lib.ck_add_tensor_forward(*pointers, 1000 + extra, _C.CK_F32, 256, None)
+    call.finish()
+    print("status", status, "sum", float(out.sum()), flush=True)
+"""
+    honest = subprocess.run([sys.executable, "-c", program, "0"], capture_output=True, text=True, timeout=600)
+    assert honest.returncode == 0 and "status 0 sum 2000.0" in honest.stdout, honest.stdout + honest.stderr
+    lying = subprocess.run([sys.executable, "-c", program, "4096"], capture_output=True, text=True, timeout=600)
+    assert lying.returncode == -signal.SIGSEGV, (lying.returncode, lying.stdout, lying.stderr[-500:])
 
 
 def test_the_package_itself_still_refuses_cpu_tensors():
