@@ -12,6 +12,8 @@ import os
 import shutil
 import subprocess
 
+import torch
+
 
 HOST_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(os.path.dirname(os.path.dirname(HOST_DIR)), "kernel-hyperdrive_amd", "csrc")
@@ -91,7 +93,12 @@ class _GuardedCall:
         else:
             copy = fence - nbytes
             copy -= (copy - lo) % 16
-        ctypes.memmove(copy, lo, nbytes)
+        if t.dtype == torch.uint8:
+            # a workspace: its contents are undefined by contract, so a kernel that reads a byte of it before writing
+            # it reads ones here (NaNs as floats, -1 as integers) and the results show it
+            ctypes.memset(copy, 0xFF, nbytes)
+        else:
+            ctypes.memmove(copy, lo, nbytes)
         self.regions.append((lo, hi, copy, mapping, size))
         return copy
 
@@ -143,6 +150,7 @@ def _with_aligned_workspace(function, pointer_at: int, bytes_at: int):
         args = list(args)
         if args[pointer_at] and args[pointer_at] % 256:
             scratch = ctypes.create_string_buffer(args[bytes_at] + 256)
+            ctypes.memset(scratch, 0xFF, args[bytes_at] + 256)  # (undefined contents: not zeros, which could pass for cleared)
             args[pointer_at] = (ctypes.addressof(scratch) + 255) // 256 * 256
         return function(*args)
 
