@@ -36,16 +36,25 @@ def build(directory: str, sources=None) -> str:
     if compiler is None:
         raise RuntimeError("no clang of the ROCm toolchain to build the host emulation with")
     sources = sorted(sources or glob.glob(os.path.join(CSRC, "*.hip"))) + [os.path.join(HOST_DIR, "emulated_support.cpp")]
+    flags, link = FLAGS, []
+    if os.environ.get("EMULATED_LIBRARY_SANITIZE"):
+        # The host's AddressSanitizer over the device code: LDS buffers are globals and per-lane arrays stack objects
+        # here, so an index that leaves one is reported.  The runtime is a shared library that comes in with this one;
+        # the process needs ASAN_OPTIONS=verify_asan_link_order=0:detect_leaks=0 and the directory of
+        # libclang_rt.asan-x86_64.so (under the toolchain's lib/clang) on LD_LIBRARY_PATH.  Three minutes to build.
+        sanitize = ["-fsanitize=address", "-shared-libsan", "-fno-omit-frame-pointer"]
+        flags = [f for f in FLAGS if f != "-O0"] + ["-O1", "-g", *sanitize]
+        link = sanitize
     objects = [os.path.join(directory, os.path.basename(s) + ".o") for s in sources]
 
     def compile_one(pair):
         source, obj = pair
-        subprocess.run([compiler, *FLAGS, "-c", source, "-o", obj], check=True, capture_output=True, text=True)
+        subprocess.run([compiler, *flags, "-c", source, "-o", obj], check=True, capture_output=True, text=True)
 
     with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(sources))) as pool:
         list(pool.map(compile_one, zip(sources, objects)))
     library = os.path.join(directory, "libcute_hip_emulated.so")
-    subprocess.run([compiler, "-shared", "-o", library, *objects], check=True, capture_output=True, text=True)
+    subprocess.run([compiler, "-shared", *link, "-o", library, *objects], check=True, capture_output=True, text=True)
     return library
 
 
