@@ -197,6 +197,14 @@ def test_results_do_not_depend_on_the_order_of_the_lanes(emulated_lanes_reversed
     function(emulated_lanes_reversed, **arguments)
 
 
+def test_smoke_body_on_the_emulated_device(emulated):
+    """What __graft_entry__.smoke() runs on cuda:0 - a small layer forward and backward, one RMSNorm, one embedding
+    gather, each against the oracle - on the emulation."""
+    import __graft_entry__
+
+    __graft_entry__._smoke_on(emulated)
+
+
 def test_the_guard_page_ends_a_call_that_reads_past_an_operand(library):
     """The tests above run with every operand in front of an inaccessible page (emulated_library._GuardedCall).  That
     this does end a kernel that walks past the end of an operand is shown here, in a process of its own: an addition
