@@ -176,6 +176,7 @@ case(W.test_scatter2scatter_four_waves, also_reversed=True, dtype=BF16, w_layout
 case(W.test_scatter2scatter_four_waves, dtype=F16, w_layout="n_contiguous", mode="scatter_out", shape=W.SHAPES[1])
 case(W.test_fused_swiglu_products_four_waves, also_reversed=True, dtype=BF16, shape=(300, 2, 3, 192, 128))
 case(W.test_group_bwd_W_four_waves, also_reversed=True, dtype=BF16, dw_layout="k_contiguous", shape=(300, 2, 3, 256, 256, ()))
+case(W.test_moe_layer_four_waves_equals_eight, shape=(200, 128, 256, 4, 2))
 
 # ---- the short prelude of the embedding backward against the default one, bit for bit ---------------------------------------
 for dtype, kind, table in [(BF16, "zipf", (5000, 1024)), (F32, "one_row", (300, 64)), (BF16, "outside", (131072 + 9, 8)),

@@ -131,14 +131,16 @@ def test_group_bwd_W_four_waves(gpu, dtype, dw_layout, shape):
     assert_close(res[4], O.group_bwd_W(DY, X, off, E, acc_dtype(dtype)), dtype, "DW")
 
 
-def test_moe_layer_four_waves_equals_eight(gpu, monkeypatch):
+@pytest.mark.parametrize("shape", [(2048, 512, 1408, 8, 2), (200, 128, 256, 4, 2)])
+def test_moe_layer_four_waves_equals_eight(gpu, monkeypatch, shape):
     """The whole layer (fused SwiGLU epilogues, split tails where the tuner's cache says so) with every grouped product
     sent through the four-wave loop: outputs and gradients equal the eight-wave run's bit for bit."""
     from cute_kernels import _C, MoE_Triton
     from test_gpu_moe import build_moe, run_moe
 
     dtype = torch.bfloat16
-    T, H, I, E, k = 2048, 512, 1408, 8, 2
+    T, H, I, E, k = shape
+    announce("MoE layer, four waves against eight", shape)
     x, w_gate, w_fc, w_proj, dy = O.moe_inputs(T, H, I, E, dtype, seed=161)
     results = {}
     for waves in (8, 4):
