@@ -4,7 +4,7 @@
 
 Grouped products (all three modes, both weight layouts, both loops of the kernel, with and without a bias, empty
 experts, sizes that are and are not multiples of 8), weight gradients, RMSNorm forward and backward, the embedding in
-both preludes of its backward, the expert sort - each case with shapes, types and routing drawn from SEED, every
+both preludes of its backward, the expert sort, the whole layer forward and backward - each case with shapes, types and routing drawn from SEED, every
 operand in front of or behind an inaccessible page, held to the oracle at the tolerances of the GPU tests.  Not part
 of the test suite: it is the long run beside it (six processes for ninety minutes: 5000 cases)."""
 import sys, time, traceback, random, os
@@ -105,7 +105,19 @@ def case_sort():
     assert torch.equal(s, es) and torch.equal(idx, eidx) and torch.equal(off, eoff), desc
     return desc
 
-cases = [case_s2s] * 4 + [case_dw] * 2 + [case_rmsnorm] * 2 + [case_embedding] * 2 + [case_sort]
+def case_moe():
+    # the whole layer, forward and backward, as the GPU test of it checks it (fused SwiGLU epilogues where the
+    # intermediate size is a multiple of 128, the separate launches elsewhere; the router and mixing kernels)
+    import test_gpu_moe as M
+    dtype = rng.choice(DT); E = rng.randint(1, 8); k = rng.randint(1, min(4, E)); T = rng.randint(1, 160)
+    H = 8 * rng.randint(2, 32); I = rng.choice([128, 256, 8 * rng.randint(2, 40)])
+    case = (f"random T{T} H{H} I{I} E{E} k{k}", T, H, I, E, k, None)
+    fn = rng.choice([M.test_moe_layer_against_oracle, M.test_moe_layer_against_oracle, M.test_moe_layer_with_expert_biases,
+                     M.test_moe_layer_fused_swiglu_equals_separate_ops])
+    fn(cpu, dtype, case)
+    return f"{fn.__name__[5:]} {dtype} {case[0]}"
+
+cases = [case_s2s] * 4 + [case_dw] * 2 + [case_rmsnorm] * 2 + [case_embedding] * 2 + [case_sort] + [case_moe] * 2
 if len(sys.argv) > 3:
     lib = sys.argv[3]
 else:
